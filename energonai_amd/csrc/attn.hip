@@ -1,0 +1,521 @@
+// The two attention contractions on the padded [B,H,S,*] layout, restricted to
+// the region softmax actually uses (valid query rows, visible keys):
+//
+//   scores = alpha * Q K^T      (attn_qk_kernel)
+//   ctx    = P V                (attn_pv_kernel)
+//
+// Both run on the 32x32 MFMA of gfx950 (32x32x16 for fp16/bf16, 32x32x2 for
+// fp32) with fp32 accumulation.  A workgroup is four waves in a 2x2 arrangement
+// over a 128-query tile; the operand that is streamed (K tiles for QK^T, P and
+// V tiles for PV) is staged through LDS with coalesced 128-bit loads and the
+// next tile is prefetched into registers while the current one is multiplied.
+//
+// The MFMA result layout has lanes running along the N operand and registers
+// along M, so the operands are assigned to make the registers run along the
+// contiguous output dimension: QK^T computes (K)(Q)^T so that each lane owns
+// four consecutive keys of one query row, PV computes (V^T)(P)^T so that each
+// lane owns four consecutive channels of one query row.
+//
+// Work is laid out per (batch, head) "unit".  Workgroups are dealt to the eight
+// XCDs round-robin by the hardware, so workgroup id -> (unit, query tile) is
+// chosen such that all query tiles of a unit land on the same XCD and reuse
+// that unit's K/V through one L2; within a unit the longest (bottom) causal
+// query tiles are issued first.
+#include "common.hip.h"
+
+namespace en {
+
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+typedef _Float16 halfx8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+
+constexpr int kQTile = 128;  // query rows per workgroup
+
+// ---------------------------------------------------------------------------
+// per-dtype MFMA step on one 128-bit vector per lane of each operand.
+//   EPV  elements in a 128-bit vector
+//   KPV  contraction indices consumed per vector step by the two lane groups
+//   k_of contraction index held by element 0 of lane group g's vector at step vs
+// A and B use the same mapping, so any bijection gives the same sum.
+// ---------------------------------------------------------------------------
+template <int DT> struct Mma;
+
+template <> struct Mma<EN_F16> {
+  static constexpr int EPV = 8, KPV = 16;
+  __device__ static __forceinline__ int k_of(int vs, int g, int) { return vs * 16 + g * 8; }
+  __device__ static __forceinline__ void step(const uint4 &a, const uint4 &b, floatx16 &c) {
+    c = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(halfx8, a), __builtin_bit_cast(halfx8, b), c, 0, 0, 0);
+  }
+};
+template <> struct Mma<EN_BF16> {
+  static constexpr int EPV = 8, KPV = 16;
+  __device__ static __forceinline__ int k_of(int vs, int g, int) { return vs * 16 + g * 8; }
+  __device__ static __forceinline__ void step(const uint4 &a, const uint4 &b, floatx16 &c) {
+    c = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+  }
+};
+template <> struct Mma<EN_F32> {
+  static constexpr int EPV = 4, KPV = 8;
+  // lane group g owns the contiguous half [g*nvs*4, (g+1)*nvs*4) of the contraction range
+  __device__ static __forceinline__ int k_of(int vs, int g, int nvs) { return g * nvs * 4 + vs * 4; }
+  __device__ static __forceinline__ void step(const uint4 &a, const uint4 &b, floatx16 &c) {
+    c = __builtin_amdgcn_mfma_f32_32x32x2f32(__uint_as_float(a.x), __uint_as_float(b.x), c, 0, 0, 0);
+    c = __builtin_amdgcn_mfma_f32_32x32x2f32(__uint_as_float(a.y), __uint_as_float(b.y), c, 0, 0, 0);
+    c = __builtin_amdgcn_mfma_f32_32x32x2f32(__uint_as_float(a.z), __uint_as_float(b.z), c, 0, 0, 0);
+    c = __builtin_amdgcn_mfma_f32_32x32x2f32(__uint_as_float(a.w), __uint_as_float(b.w), c, 0, 0, 0);
+  }
+};
+
+__device__ __forceinline__ uint4 zero4() { return make_uint4(0u, 0u, 0u, 0u); }
+
+struct AttnArgs {
+  const void *a_ptr;   // q (QK) or p (PV)
+  const void *b_ptr;   // k (QK) or v (PV)
+  void *out;           // scores (QK) or ctx (PV)
+  const int32_t *k_lens;
+  const int32_t *q_lens;
+  int B, H, Sq, Sk, D;
+  int64_t q_sb, q_sh, q_ss;  // strides of q (QK) / ctx (PV), elements
+  int64_t k_sb, k_sh, k_ss;  // strides of k (QK) / v (PV), elements
+  float alpha;
+  int causal;
+  int zero_padding;
+  int vec_out;   // output rows may be written with 128-bit stores
+  int ntq;       // query tiles per unit
+  int units;     // B * H
+};
+
+// workgroup id -> (unit, query tile): see the header comment.
+__device__ __forceinline__ bool map_block(const AttnArgs &a, int &unit, int &qi) {
+  const int bid = blockIdx.x;
+  const int xcd = bid % kXcds;
+  const int slot = bid / kXcds;
+  unit = (slot / a.ntq) * kXcds + xcd;
+  qi = a.ntq - 1 - (slot % a.ntq);
+  return unit < a.units;
+}
+
+__device__ __forceinline__ void seq_extents(const AttnArgs &a, int b, int &kl, int &ql) {
+  kl = min(a.k_lens[b], a.Sk);
+  ql = a.q_lens ? a.q_lens[b] : min(kl, a.Sq);
+  ql = min(ql, a.Sq);
+}
+
+// keys the last valid query row of a tile may see
+__device__ __forceinline__ int tile_key_extent(const AttnArgs &a, int q_last, int kl, int ql) {
+  int n = a.causal ? min(kl, q_last + (kl - ql) + 1) : kl;
+  return max(n, 0);
+}
+
+// ===========================================================================
+// scores = alpha * Q K^T
+// ===========================================================================
+template <int DT, int DP>
+__global__ __launch_bounds__(kBlock) void attn_qk_kernel(AttnArgs a) {
+  typedef Elem<DT> E;
+  typedef typename E::T T;
+  typedef Mma<DT> M;
+  constexpr int EPV = M::EPV;
+  constexpr int BN = (DT == EN_F32) ? 64 : 128;  // keys per tile
+  constexpr int MT = BN / 64;                    // 32-key MFMA tiles per wave
+  constexpr int NT = 2;                          // 32-query MFMA tiles per wave
+  constexpr int NVS = DP / M::KPV;               // vector steps over the head dim
+  constexpr int KPITCH = DP + EPV;               // LDS pitch of a K row, elements
+  constexpr int CPITCH = BN + EPV;               // LDS pitch of a score row, elements
+  constexpr int KVEC_ROW = DP / EPV;             // 128-bit vectors per K row
+  constexpr int KLOADS = BN * KVEC_ROW / kBlock; // K vectors each lane stages per tile
+  constexpr int CVEC_ROW = BN / EPV;
+  constexpr int CSTORES = kQTile * CVEC_ROW / kBlock;
+  constexpr int LDS_ELEMS = (BN * KPITCH > kQTile * CPITCH) ? BN * KPITCH : kQTile * CPITCH;
+  static_assert(BN * KVEC_ROW % kBlock == 0 && kQTile * CVEC_ROW % kBlock == 0, "tile must divide over the block");
+  __shared__ __attribute__((aligned(16))) T lds[LDS_ELEMS];
+
+  int unit, qi;
+  if (!map_block(a, unit, qi)) return;
+  const int b = unit / a.H, h = unit % a.H;
+  int kl, ql;
+  seq_extents(a, b, kl, ql);
+  const int q0 = qi * kQTile;
+  if (q0 >= ql) return;
+  const int nk = tile_key_extent(a, min(q0 + kQTile, ql) - 1, kl, ql);
+  if (nk <= 0) return;
+  const int nkt = (nk + BN - 1) / BN;
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63, wave = tid >> 6;
+  const int r = lane & 31, g = lane >> 5;
+  const int wq = wave & 1, wk = wave >> 1;
+
+  const T *qbase = reinterpret_cast<const T *>(a.a_ptr) + (int64_t)b * a.q_sb + (int64_t)h * a.q_sh;
+  const T *kbase = reinterpret_cast<const T *>(a.b_ptr) + (int64_t)b * a.k_sb + (int64_t)h * a.k_sh;
+  T *sbase = reinterpret_cast<T *>(a.out) + ((int64_t)unit * a.Sq) * a.Sk;
+
+  // Q fragments stay in registers for the whole key loop.
+  uint4 qf[NT][NVS];
+#pragma unroll
+  for (int nt = 0; nt < NT; ++nt) {
+    const int row = min(q0 + wq * 64 + nt * 32 + r, a.Sq - 1);
+    const T *qrow = qbase + (int64_t)row * a.q_ss;
+#pragma unroll
+    for (int vs = 0; vs < NVS; ++vs) {
+      const int d = M::k_of(vs, g, NVS);
+      qf[nt][vs] = (d < a.D) ? *reinterpret_cast<const uint4 *>(qrow + d) : zero4();
+    }
+  }
+
+  uint4 kreg[KLOADS];
+  auto fetch_k = [&](int kt) {
+    const int k0 = kt * BN;
+#pragma unroll
+    for (int i = 0; i < KLOADS; ++i) {
+      const int v = tid + i * kBlock;
+      const int row = v / KVEC_ROW, c = v % KVEC_ROW;
+      const int key = k0 + row;
+      kreg[i] = (key < kl && c * EPV < a.D) ? *reinterpret_cast<const uint4 *>(kbase + (int64_t)key * a.k_ss + c * EPV)
+                                            : zero4();
+    }
+  };
+  fetch_k(0);
+
+  for (int kt = 0; kt < nkt; ++kt) {
+    const int k0 = kt * BN;
+#pragma unroll
+    for (int i = 0; i < KLOADS; ++i) {
+      const int v = tid + i * kBlock;
+      const int row = v / KVEC_ROW, c = v % KVEC_ROW;
+      *reinterpret_cast<uint4 *>(&lds[row * KPITCH + c * EPV]) = kreg[i];
+    }
+    __syncthreads();
+    if (kt + 1 < nkt) fetch_k(kt + 1);
+
+    floatx16 acc[MT][NT];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+      for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+        for (int x = 0; x < 16; ++x) acc[mt][nt][x] = 0.f;
+
+#pragma unroll
+    for (int vs = 0; vs < NVS; ++vs) {
+      uint4 kf[MT];
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt)
+        kf[mt] = *reinterpret_cast<const uint4 *>(&lds[(wk * (BN / 2) + mt * 32 + r) * KPITCH + M::k_of(vs, g, NVS)]);
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt) M::step(kf[mt], qf[nt][vs], acc[mt][nt]);
+    }
+    __syncthreads();  // every wave is done reading K before the tile is reused for scores
+
+    // accumulators -> LDS as a row-major [query][key] tile
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+      for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          Pack<T, 4> pk;
+#pragma unroll
+          for (int i = 0; i < 4; ++i) pk.v[i] = E::from_float(acc[mt][nt][4 * j + i] * a.alpha);
+          const int qrow = wq * 64 + nt * 32 + r;
+          const int kcol = wk * (BN / 2) + mt * 32 + 8 * j + 4 * g;
+          store_pack<T, 4>(&lds[qrow * CPITCH + kcol], pk);
+        }
+    __syncthreads();
+
+    // LDS -> HBM, whole rows of the tile as 128-bit stores
+#pragma unroll
+    for (int i = 0; i < CSTORES; ++i) {
+      const int v = tid + i * kBlock;
+      const int row = v / CVEC_ROW, c = v % CVEC_ROW;
+      const int q = q0 + row, k = k0 + c * EPV;
+      if (q < ql && k < a.Sk) {
+        const T *sp = &lds[row * CPITCH + c * EPV];
+        T *gp = sbase + (int64_t)q * a.Sk + k;
+        if (a.vec_out) {
+          *reinterpret_cast<uint4 *>(gp) = *reinterpret_cast<const uint4 *>(sp);
+        } else {
+#pragma unroll
+          for (int e = 0; e < EPV; ++e)
+            if (k + e < a.Sk) gp[e] = sp[e];
+        }
+      }
+    }
+    __syncthreads();  // scores leave LDS before the next K tile lands
+  }
+}
+
+// ===========================================================================
+// ctx = P V
+// ===========================================================================
+template <int DT, int DP>
+__global__ __launch_bounds__(kBlock) void attn_pv_kernel(AttnArgs a) {
+  typedef Elem<DT> E;
+  typedef typename E::T T;
+  typedef Mma<DT> M;
+  constexpr int EPV = M::EPV;
+  constexpr int BK = (DT == EN_F32) ? 32 : 64;   // keys per tile
+  constexpr int MT = DP / 64;                    // 32-channel MFMA tiles per wave
+  constexpr int NT = 2;                          // 32-query MFMA tiles per wave
+  constexpr int NVS = BK / M::KPV;               // vector steps over a key tile
+  constexpr int PITCH = BK + EPV;                // LDS pitch of P rows and V^T rows, elements
+  constexpr int PVEC_ROW = BK / EPV;
+  constexpr int PLOADS = kQTile * PVEC_ROW / kBlock;
+  constexpr int NQUAD = BK / 4;                  // groups of four keys in a tile
+  constexpr int NCHUNK = DP / EPV;               // 128-bit channel chunks in a V row
+  constexpr int VUNITS = NQUAD * NCHUNK;         // (key quad, channel chunk) units per tile
+  constexpr int VLOADS = (VUNITS + kBlock - 1) / kBlock;
+  static_assert(kQTile * PVEC_ROW % kBlock == 0, "P tile must divide over the block");
+  __shared__ __attribute__((aligned(16))) T lds_p[kQTile * PITCH];
+  __shared__ __attribute__((aligned(16))) T lds_v[DP * PITCH];
+
+  int unit, qi;
+  if (!map_block(a, unit, qi)) return;
+  const int b = unit / a.H, h = unit % a.H;
+  int kl, ql;
+  seq_extents(a, b, kl, ql);
+  const int q0 = qi * kQTile;
+  const int tid = threadIdx.x;
+  T *cbase = reinterpret_cast<T *>(a.out) + (int64_t)b * a.q_sb + (int64_t)h * a.q_sh;
+
+  if (q0 >= ql) {
+    if (a.zero_padding) {  // whole tile is padding
+      const int rows = min(kQTile, a.Sq - q0);
+      for (int i = tid; i < rows * a.D; i += kBlock) {
+        const int row = i / a.D, d = i - row * a.D;
+        cbase[(int64_t)(q0 + row) * a.q_ss + d] = E::from_float(0.f);
+      }
+    }
+    return;
+  }
+  const int nk = tile_key_extent(a, min(q0 + kQTile, ql) - 1, kl, ql);
+  const int nkt = (nk + BK - 1) / BK;
+
+  const int lane = tid & 63, wave = tid >> 6;
+  const int r = lane & 31, g = lane >> 5;
+  const int wq = wave & 1, wd = wave >> 1;
+
+  const T *pbase = reinterpret_cast<const T *>(a.a_ptr) + ((int64_t)unit * a.Sq) * a.Sk;
+  const T *vbase = reinterpret_cast<const T *>(a.b_ptr) + (int64_t)b * a.k_sb + (int64_t)h * a.k_sh;
+
+  floatx16 acc[MT][NT];
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+      for (int x = 0; x < 16; ++x) acc[mt][nt][x] = 0.f;
+
+  uint4 preg[PLOADS];
+  uint4 vreg[VLOADS][4];
+  auto fetch = [&](int kt) {
+    const int k0 = kt * BK;
+#pragma unroll
+    for (int i = 0; i < PLOADS; ++i) {
+      const int v = tid + i * kBlock;
+      const int row = v / PVEC_ROW, c = v % PVEC_ROW;
+      const int q = q0 + row, k = k0 + c * EPV;
+      // rows of padded queries and columns past the visible extent contribute nothing
+      if (q < ql && k < nk) {
+        const T *gp = pbase + (int64_t)q * a.Sk + k;
+        if (a.vec_out) {
+          preg[i] = *reinterpret_cast<const uint4 *>(gp);
+        } else {
+          Pack<T, EPV> pk;
+#pragma unroll
+          for (int e = 0; e < EPV; ++e) pk.v[e] = (k + e < a.Sk) ? gp[e] : E::from_float(0.f);
+          preg[i] = __builtin_bit_cast(uint4, pk);
+        }
+      } else {
+        preg[i] = zero4();
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < VLOADS; ++i) {
+      const int u = tid + i * kBlock;
+      const int c = (u % 4) + 4 * ((u / (4 * NQUAD)) % (NCHUNK / 4 > 0 ? NCHUNK / 4 : 1));
+      const int kq = (u / 4) % NQUAD;
+#pragma unroll
+      for (int x = 0; x < 4; ++x) {
+        const int key = k0 + kq * 4 + x;
+        vreg[i][x] = (u < VUNITS && key < kl && c * EPV < a.D)
+                         ? *reinterpret_cast<const uint4 *>(vbase + (int64_t)key * a.k_ss + c * EPV)
+                         : zero4();
+      }
+    }
+  };
+  if (nkt > 0) fetch(0);
+
+  for (int kt = 0; kt < nkt; ++kt) {
+    // P tile: straight copy.  V tile: four keys x EPV channels per unit, written transposed
+    // so that a lane later reads consecutive keys of one channel with one 128-bit load.
+#pragma unroll
+    for (int i = 0; i < PLOADS; ++i) {
+      const int v = tid + i * kBlock;
+      const int row = v / PVEC_ROW, c = v % PVEC_ROW;
+      *reinterpret_cast<uint4 *>(&lds_p[row * PITCH + c * EPV]) = preg[i];
+    }
+#pragma unroll
+    for (int i = 0; i < VLOADS; ++i) {
+      const int u = tid + i * kBlock;
+      if (u < VUNITS) {
+        const int c = (u % 4) + 4 * ((u / (4 * NQUAD)) % (NCHUNK / 4 > 0 ? NCHUNK / 4 : 1));
+        const int kq = (u / 4) % NQUAD;
+        Pack<T, EPV> rows[4];
+#pragma unroll
+        for (int x = 0; x < 4; ++x) rows[x] = __builtin_bit_cast(Pack<T, EPV>, vreg[i][x]);
+#pragma unroll
+        for (int e = 0; e < EPV; ++e) {
+          Pack<T, 4> col;
+#pragma unroll
+          for (int x = 0; x < 4; ++x) col.v[x] = rows[x].v[e];
+          store_pack<T, 4>(&lds_v[(c * EPV + e) * PITCH + kq * 4], col);
+        }
+      }
+    }
+    __syncthreads();
+    if (kt + 1 < nkt) fetch(kt + 1);
+
+#pragma unroll
+    for (int vs = 0; vs < NVS; ++vs) {
+      const int kk = M::k_of(vs, g, NVS);
+      uint4 vf[MT], pf[NT];
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt)
+        vf[mt] = *reinterpret_cast<const uint4 *>(&lds_v[(wd * (DP / 2) + mt * 32 + r) * PITCH + kk]);
+#pragma unroll
+      for (int nt = 0; nt < NT; ++nt)
+        pf[nt] = *reinterpret_cast<const uint4 *>(&lds_p[(wq * 64 + nt * 32 + r) * PITCH + kk]);
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt) M::step(vf[mt], pf[nt], acc[mt][nt]);
+    }
+    __syncthreads();  // tiles are consumed before the next ones are written
+  }
+
+  // each lane owns four consecutive channels of one query row
+#pragma unroll
+  for (int nt = 0; nt < NT; ++nt) {
+    const int q = q0 + wq * 64 + nt * 32 + r;
+    if (q >= a.Sq) continue;
+    const bool valid = q < ql;
+    if (!valid && !a.zero_padding) continue;
+    T *crow = cbase + (int64_t)q * a.q_ss;
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int d = wd * (DP / 2) + mt * 32 + 8 * j + 4 * g;
+        if (d < a.D) {
+          Pack<T, 4> pk;
+#pragma unroll
+          for (int i = 0; i < 4; ++i) pk.v[i] = E::from_float(valid ? acc[mt][nt][4 * j + i] : 0.f);
+          store_pack<T, 4>(crow + d, pk);
+        }
+      }
+  }
+}
+
+// ---------------------------------------------------------------------------
+// host side
+// ---------------------------------------------------------------------------
+static bool strides_vec_ok(int64_t sb, int64_t sh, int64_t ss, int epv) {
+  return (sb % epv) == 0 && (sh % epv) == 0 && (ss % epv) == 0;
+}
+
+template <int DT>
+static int launch_qk(AttnArgs &a, hipStream_t s) {
+  const unsigned grid = (unsigned)(ceil_div(a.units, kXcds) * kXcds * a.ntq);
+  if (a.D <= 64) attn_qk_kernel<DT, 64><<<grid, kBlock, 0, s>>>(a);
+  else attn_qk_kernel<DT, 128><<<grid, kBlock, 0, s>>>(a);
+  EN_RETURN_IF_LAUNCH_FAILED();
+  return EN_OK;
+}
+
+template <int DT>
+static int launch_pv(AttnArgs &a, hipStream_t s) {
+  const unsigned grid = (unsigned)(ceil_div(a.units, kXcds) * kXcds * a.ntq);
+  if (a.D <= 64) attn_pv_kernel<DT, 64><<<grid, kBlock, 0, s>>>(a);
+  else attn_pv_kernel<DT, 128><<<grid, kBlock, 0, s>>>(a);
+  EN_RETURN_IF_LAUNCH_FAILED();
+  return EN_OK;
+}
+
+static int check_common(const void *x, const void *y, const void *z, const int32_t *k_lens, int batch, int head_num,
+                        int q_seq_len, int k_seq_len, int size_per_head, int dtype) {
+  if (!x || !y || !z || !k_lens) return EN_ERR_NULL;
+  if (batch < 1 || head_num < 1 || q_seq_len < 1 || k_seq_len < 1 || size_per_head < 1) return EN_ERR_SHAPE;
+  const int es = dtype_size(dtype);
+  if (!es) return EN_ERR_DTYPE;
+  const int epv = 16 / es;
+  if (size_per_head > 128 || (size_per_head % epv) != 0) return EN_ERR_UNSUPPORTED;
+  if ((int64_t)batch * head_num > INT32_MAX / 64) return EN_ERR_SHAPE;
+  return EN_OK;
+}
+
+}  // namespace en
+
+extern "C" {
+
+int en_attn_qk(const void *q, const void *k, void *scores, const int32_t *k_lens, const int32_t *q_lens, int batch,
+               int head_num, int q_seq_len, int k_seq_len, int size_per_head, int64_t q_stride_b,
+               int64_t q_stride_h, int64_t q_stride_s, int64_t k_stride_b, int64_t k_stride_h, int64_t k_stride_s,
+               float alpha, int causal, int dtype, en_stream_t stream) {
+  using namespace en;
+  int rc = check_common(q, k, scores, k_lens, batch, head_num, q_seq_len, k_seq_len, size_per_head, dtype);
+  if (rc) return rc;
+  const int es = dtype_size(dtype), epv = 16 / es;
+  if (!aligned_to(q, 16) || !aligned_to(k, 16) || !aligned_to(scores, es)) return EN_ERR_ALIGN;
+  if (!strides_vec_ok(q_stride_b, q_stride_h, q_stride_s, epv) ||
+      !strides_vec_ok(k_stride_b, k_stride_h, k_stride_s, epv))
+    return EN_ERR_ALIGN;
+  AttnArgs a{};
+  a.a_ptr = q; a.b_ptr = k; a.out = scores; a.k_lens = k_lens; a.q_lens = q_lens;
+  a.B = batch; a.H = head_num; a.Sq = q_seq_len; a.Sk = k_seq_len; a.D = size_per_head;
+  a.q_sb = q_stride_b; a.q_sh = q_stride_h; a.q_ss = q_stride_s;
+  a.k_sb = k_stride_b; a.k_sh = k_stride_h; a.k_ss = k_stride_s;
+  a.alpha = alpha; a.causal = causal ? 1 : 0; a.zero_padding = 0;
+  a.vec_out = ((k_seq_len % epv) == 0 && aligned_to(scores, 16)) ? 1 : 0;
+  a.ntq = (int)ceil_div(q_seq_len, kQTile);
+  a.units = batch * head_num;
+  hipStream_t s = (hipStream_t)stream;
+  switch (dtype) {
+    case EN_F32: return launch_qk<EN_F32>(a, s);
+    case EN_F16: return launch_qk<EN_F16>(a, s);
+    default: return launch_qk<EN_BF16>(a, s);
+  }
+}
+
+int en_attn_pv(const void *p, const void *v, void *ctx, const int32_t *k_lens, const int32_t *q_lens, int batch,
+               int head_num, int q_seq_len, int k_seq_len, int size_per_head, int64_t v_stride_b,
+               int64_t v_stride_h, int64_t v_stride_s, int64_t c_stride_b, int64_t c_stride_h, int64_t c_stride_s,
+               int causal, int zero_padding, int dtype, en_stream_t stream) {
+  using namespace en;
+  int rc = check_common(p, v, ctx, k_lens, batch, head_num, q_seq_len, k_seq_len, size_per_head, dtype);
+  if (rc) return rc;
+  const int es = dtype_size(dtype), epv = 16 / es;
+  if (!aligned_to(p, es) || !aligned_to(v, 16) || !aligned_to(ctx, 4 * es)) return EN_ERR_ALIGN;
+  if (!strides_vec_ok(v_stride_b, v_stride_h, v_stride_s, epv) ||
+      !strides_vec_ok(c_stride_b, c_stride_h, c_stride_s, 4))
+    return EN_ERR_ALIGN;
+  AttnArgs a{};
+  a.a_ptr = p; a.b_ptr = v; a.out = ctx; a.k_lens = k_lens; a.q_lens = q_lens;
+  a.B = batch; a.H = head_num; a.Sq = q_seq_len; a.Sk = k_seq_len; a.D = size_per_head;
+  a.q_sb = c_stride_b; a.q_sh = c_stride_h; a.q_ss = c_stride_s;
+  a.k_sb = v_stride_b; a.k_sh = v_stride_h; a.k_ss = v_stride_s;
+  a.alpha = 1.f; a.causal = causal ? 1 : 0; a.zero_padding = zero_padding ? 1 : 0;
+  a.vec_out = ((k_seq_len % epv) == 0 && aligned_to(p, 16)) ? 1 : 0;
+  a.ntq = (int)ceil_div(q_seq_len, kQTile);
+  a.units = batch * head_num;
+  hipStream_t s = (hipStream_t)stream;
+  switch (dtype) {
+    case EN_F32: return launch_pv<EN_F32>(a, s);
+    case EN_F16: return launch_pv<EN_F16>(a, s);
+    default: return launch_pv<EN_BF16>(a, s);
+  }
+}
+
+}  // extern "C"

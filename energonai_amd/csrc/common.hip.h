@@ -1,0 +1,118 @@
+// Shared host/device helpers for the gfx950 kernels: status bookkeeping,
+// element traits for fp32/fp16/bf16 storage, 128-bit vector access and
+// wave64 reductions built on DPP row operations.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "energon_hip.h"
+
+namespace en {
+
+constexpr int kWave = 64;       // gfx950 wavefront width
+constexpr int kBlock = 256;     // default workgroup: 4 waves, one per SIMD
+constexpr int kXcds = 8;        // MI355X: 8 XCDs, workgroups are dealt to them round-robin
+
+// ---- host side ------------------------------------------------------------
+
+int record_hip_error(hipError_t e);  // stores e for en_last_hip_error(), returns EN_ERR_HIP
+
+#define EN_RETURN_IF_LAUNCH_FAILED()                      \
+  do {                                                    \
+    hipError_t en_e_ = hipGetLastError();                 \
+    if (en_e_ != hipSuccess) return ::en::record_hip_error(en_e_); \
+  } while (0)
+
+inline bool aligned_to(const void *p, size_t a) { return (reinterpret_cast<uintptr_t>(p) % a) == 0; }
+inline int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
+inline int dtype_size(int dt) { return dt == EN_F32 ? 4 : ((dt == EN_F16 || dt == EN_BF16) ? 2 : 0); }
+
+// ---- element traits ---------------------------------------------------------
+
+typedef _Float16 half_t;
+
+__device__ __forceinline__ float bf16_bits_to_float(uint16_t v) { return __uint_as_float(((uint32_t)v) << 16); }
+__device__ __forceinline__ uint16_t float_to_bf16_bits(float f) {
+  uint32_t u = __float_as_uint(f);
+  if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x0040u);  // quiet NaN
+  u += 0x7fffu + ((u >> 16) & 1u);                                             // round to nearest even
+  return (uint16_t)(u >> 16);
+}
+
+template <int DT> struct Elem;
+template <> struct Elem<EN_F32> {
+  typedef float T;
+  static constexpr int kSize = 4;
+  __device__ static __forceinline__ float to_float(T v) { return v; }
+  __device__ static __forceinline__ T from_float(float f) { return f; }
+};
+template <> struct Elem<EN_F16> {
+  typedef half_t T;
+  static constexpr int kSize = 2;
+  __device__ static __forceinline__ float to_float(T v) { return (float)v; }
+  __device__ static __forceinline__ T from_float(float f) { return (T)f; }
+};
+template <> struct Elem<EN_BF16> {
+  typedef uint16_t T;
+  static constexpr int kSize = 2;
+  __device__ static __forceinline__ float to_float(T v) { return bf16_bits_to_float(v); }
+  __device__ static __forceinline__ T from_float(float f) { return float_to_bf16_bits(f); }
+};
+
+// N elements of T moved as one access (N * sizeof(T) is 4, 8 or 16 bytes).
+template <typename T, int N> struct alignas(sizeof(T) * N) Pack { T v[N]; };
+
+template <typename T, int N>
+__device__ __forceinline__ Pack<T, N> load_pack(const T *p) { return *reinterpret_cast<const Pack<T, N> *>(p); }
+template <typename T, int N>
+__device__ __forceinline__ void store_pack(T *p, const Pack<T, N> &x) { *reinterpret_cast<Pack<T, N> *>(p) = x; }
+
+// ---- wave64 reductions --------------------------------------------------------
+//
+// Steps inside a 16-lane DPP row use quad_perm / row_half_mirror / row_mirror
+// (no LDS traffic, full rate); the two steps that cross rows go through the
+// LDS crossbar (ds_bpermute via __shfl_xor).  Every lane ends with the result.
+// All lanes of the wave must be active at the call.
+
+template <int CTRL>
+__device__ __forceinline__ float dpp_move(float v) {
+  return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xF, 0xF, true));
+}
+
+struct OpSum { __device__ static __forceinline__ float apply(float a, float b) { return a + b; } };
+struct OpMax { __device__ static __forceinline__ float apply(float a, float b) { return fmaxf(a, b); } };
+
+// Reduce over aligned groups of WIDTH lanes (WIDTH = 2..64, power of two).
+template <typename Op, int WIDTH>
+__device__ __forceinline__ float group_allreduce(float v) {
+  static_assert(WIDTH >= 1 && WIDTH <= 64 && (WIDTH & (WIDTH - 1)) == 0, "WIDTH must be a power of two <= 64");
+  if (WIDTH >= 2) v = Op::apply(v, dpp_move<0xB1>(v));   // quad_perm [1,0,3,2]
+  if (WIDTH >= 4) v = Op::apply(v, dpp_move<0x4E>(v));   // quad_perm [2,3,0,1]
+  if (WIDTH >= 8) v = Op::apply(v, dpp_move<0x141>(v));  // row_half_mirror
+  if (WIDTH >= 16) v = Op::apply(v, dpp_move<0x140>(v)); // row_mirror
+  if (WIDTH >= 32) v = Op::apply(v, __shfl_xor(v, 16, kWave));
+  if (WIDTH >= 64) v = Op::apply(v, __shfl_xor(v, 32, kWave));
+  return v;
+}
+
+template <typename Op>
+__device__ __forceinline__ float wave_allreduce(float v) { return group_allreduce<Op, 64>(v); }
+
+// Reduce over a workgroup of NWAVES waves; `slots` is NWAVES floats of LDS
+// owned by this reduction (a second reduction needs its own slots or a barrier).
+template <typename Op, int NWAVES>
+__device__ __forceinline__ float block_allreduce(float v, float *slots) {
+  v = wave_allreduce<Op>(v);
+  if (NWAVES == 1) return v;
+  const int lane = threadIdx.x & (kWave - 1);
+  const int wave = threadIdx.x >> 6;
+  if (lane == 0) slots[wave] = v;
+  __syncthreads();
+  float r = slots[0];
+#pragma unroll
+  for (int w = 1; w < NWAVES; ++w) r = Op::apply(r, slots[w]);
+  return r;
+}
+
+}  // namespace en

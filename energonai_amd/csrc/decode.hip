@@ -1,0 +1,189 @@
+// Single-query attention contractions for cached decode: one new token per
+// sequence against a ragged K/V cache.  Both are matrix-vector products whose
+// cost is the K (or V) bytes streamed from HBM, so they are written as
+// streaming reductions with 128-bit loads, one workgroup per (batch, head):
+// LPK lanes cover one cached row of D elements, 256/LPK rows are in flight per
+// step, four steps are unrolled so each lane keeps 64 bytes outstanding.
+#include "common.hip.h"
+
+namespace en {
+
+struct DecodeArgs {
+  const void *x;    // q [B,H,D] (QK) or p [B,H,Smax] (PV)
+  const void *kv;   // cache [B,H,Smax,D], strided
+  void *out;        // scores [B,H,Smax] (QK) or ctx [B,H,D] (PV)
+  const int32_t *kv_lens;
+  int H, Sk, D;
+  int64_t sb, sh, ss;
+  float alpha;
+};
+
+template <int DT, int LPK>
+__global__ __launch_bounds__(kBlock) void decode_qk_kernel(DecodeArgs a) {
+  typedef Elem<DT> E;
+  typedef typename E::T T;
+  constexpr int EPV = 16 / E::kSize;
+  constexpr int KPS = kBlock / LPK;  // keys per step
+  constexpr int U = 4;
+  const int h = blockIdx.x, b = blockIdx.y;
+  const int tid = threadIdx.x;
+  const int c = tid % LPK, slot = tid / LPK;
+  const int kl = min(a.kv_lens[b], a.Sk);
+  const T *q = reinterpret_cast<const T *>(a.x) + ((int64_t)b * a.H + h) * a.D;
+  const T *kbase = reinterpret_cast<const T *>(a.kv) + (int64_t)b * a.sb + (int64_t)h * a.sh;
+  T *srow = reinterpret_cast<T *>(a.out) + ((int64_t)b * a.H + h) * a.Sk;
+
+  float qv[EPV];
+  {
+    const Pack<T, EPV> pk = load_pack<T, EPV>(q + c * EPV);
+#pragma unroll
+    for (int e = 0; e < EPV; ++e) qv[e] = E::to_float(pk.v[e]) * a.alpha;
+  }
+  for (int k0 = 0; k0 < kl; k0 += KPS * U) {  // uniform trip count: all lanes reach the reductions
+    Pack<T, EPV> kv[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int key = k0 + u * KPS + slot;
+      if (key < kl) kv[u] = load_pack<T, EPV>(kbase + (int64_t)key * a.ss + c * EPV);
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int key = k0 + u * KPS + slot;
+      float dot = 0.f;
+      if (key < kl) {
+#pragma unroll
+        for (int e = 0; e < EPV; ++e) dot += qv[e] * E::to_float(kv[u].v[e]);
+      }
+      dot = group_allreduce<OpSum, LPK>(dot);
+      if (c == 0 && key < kl) srow[key] = E::from_float(dot);
+    }
+  }
+}
+
+template <int DT, int LPK>
+__global__ __launch_bounds__(kBlock) void decode_pv_kernel(DecodeArgs a) {
+  typedef Elem<DT> E;
+  typedef typename E::T T;
+  constexpr int EPV = 16 / E::kSize;
+  constexpr int KPS = kBlock / LPK;
+  constexpr int U = 4;
+  __shared__ float s_acc[KPS][LPK * EPV + 1];
+  const int h = blockIdx.x, b = blockIdx.y;
+  const int tid = threadIdx.x;
+  const int c = tid % LPK, slot = tid / LPK;
+  const int kl = min(a.kv_lens[b], a.Sk);
+  const T *prow = reinterpret_cast<const T *>(a.x) + ((int64_t)b * a.H + h) * a.Sk;
+  const T *vbase = reinterpret_cast<const T *>(a.kv) + (int64_t)b * a.sb + (int64_t)h * a.sh;
+  T *ctx = reinterpret_cast<T *>(a.out) + ((int64_t)b * a.H + h) * a.D;
+
+  float acc[EPV];
+#pragma unroll
+  for (int e = 0; e < EPV; ++e) acc[e] = 0.f;
+  for (int k0 = slot; k0 < kl; k0 += KPS * U) {
+    Pack<T, EPV> vv[U];
+    float p[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int key = k0 + u * KPS;
+      p[u] = 0.f;
+      if (key < kl) {
+        vv[u] = load_pack<T, EPV>(vbase + (int64_t)key * a.ss + c * EPV);
+        p[u] = E::to_float(prow[key]);
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int key = k0 + u * KPS;
+      if (key < kl) {
+#pragma unroll
+        for (int e = 0; e < EPV; ++e) acc[e] += p[u] * E::to_float(vv[u].v[e]);
+      }
+    }
+  }
+#pragma unroll
+  for (int e = 0; e < EPV; ++e) s_acc[slot][c * EPV + e] = acc[e];
+  __syncthreads();
+  for (int d = tid; d < a.D; d += kBlock) {
+    float s = 0.f;
+#pragma unroll 4
+    for (int j = 0; j < KPS; ++j) s += s_acc[j][d];
+    ctx[d] = E::from_float(s);
+  }
+}
+
+template <int DT, template <int, int> class Launcher>
+static int dispatch_lpk(const DecodeArgs &a, int batch, hipStream_t s) {
+  constexpr int EPV = 16 / Elem<DT>::kSize;
+  const int lpk = a.D / EPV;
+  dim3 grid((unsigned)a.H, (unsigned)batch, 1);
+  switch (lpk) {
+    case 4: Launcher<DT, 4>::go(a, grid, s); break;
+    case 8: Launcher<DT, 8>::go(a, grid, s); break;
+    case 16: Launcher<DT, 16>::go(a, grid, s); break;
+    case 32: Launcher<DT, 32>::go(a, grid, s); break;
+    case 64: Launcher<DT, 64>::go(a, grid, s); break;
+    default: return EN_ERR_UNSUPPORTED;
+  }
+  EN_RETURN_IF_LAUNCH_FAILED();
+  return EN_OK;
+}
+
+template <int DT, int LPK> struct QkLauncher {
+  static void go(const DecodeArgs &a, dim3 grid, hipStream_t s) { decode_qk_kernel<DT, LPK><<<grid, kBlock, 0, s>>>(a); }
+};
+template <int DT, int LPK> struct PvLauncher {
+  static void go(const DecodeArgs &a, dim3 grid, hipStream_t s) { decode_pv_kernel<DT, LPK><<<grid, kBlock, 0, s>>>(a); }
+};
+
+static int check_decode(const void *x, const void *kv, const void *out, const int32_t *lens, int batch, int head_num,
+                        int k_seq_len, int size_per_head, int64_t sb, int64_t sh, int64_t ss, int dtype) {
+  if (!x || !kv || !out || !lens) return EN_ERR_NULL;
+  if (batch < 1 || batch > 65535 || head_num < 1 || k_seq_len < 1 || size_per_head < 1) return EN_ERR_SHAPE;
+  const int es = dtype_size(dtype);
+  if (!es) return EN_ERR_DTYPE;
+  const int epv = 16 / es;
+  if ((size_per_head % epv) != 0) return EN_ERR_UNSUPPORTED;
+  if (!aligned_to(kv, 16) || (sb % epv) || (sh % epv) || (ss % epv)) return EN_ERR_ALIGN;
+  return EN_OK;
+}
+
+}  // namespace en
+
+extern "C" {
+
+int en_decode_qk(const void *q, const void *k_cache, void *scores, const int32_t *kv_lens, int batch, int head_num,
+                 int k_seq_len, int size_per_head, int64_t k_stride_b, int64_t k_stride_h, int64_t k_stride_s,
+                 float alpha, int dtype, en_stream_t stream) {
+  using namespace en;
+  int rc = check_decode(q, k_cache, scores, kv_lens, batch, head_num, k_seq_len, size_per_head, k_stride_b,
+                        k_stride_h, k_stride_s, dtype);
+  if (rc) return rc;
+  if (!aligned_to(q, 16) || !aligned_to(scores, dtype_size(dtype))) return EN_ERR_ALIGN;
+  DecodeArgs a{q, k_cache, scores, kv_lens, head_num, k_seq_len, size_per_head, k_stride_b, k_stride_h, k_stride_s,
+               alpha};
+  hipStream_t s = (hipStream_t)stream;
+  switch (dtype) {
+    case EN_F32: return dispatch_lpk<EN_F32, QkLauncher>(a, batch, s);
+    case EN_F16: return dispatch_lpk<EN_F16, QkLauncher>(a, batch, s);
+    default: return dispatch_lpk<EN_BF16, QkLauncher>(a, batch, s);
+  }
+}
+
+int en_decode_pv(const void *p, const void *v_cache, void *ctx, const int32_t *kv_lens, int batch, int head_num,
+                 int k_seq_len, int size_per_head, int64_t v_stride_b, int64_t v_stride_h, int64_t v_stride_s,
+                 int dtype, en_stream_t stream) {
+  using namespace en;
+  int rc = check_decode(p, v_cache, ctx, kv_lens, batch, head_num, k_seq_len, size_per_head, v_stride_b, v_stride_h,
+                        v_stride_s, dtype);
+  if (rc) return rc;
+  if (!aligned_to(p, dtype_size(dtype)) || !aligned_to(ctx, dtype_size(dtype))) return EN_ERR_ALIGN;
+  DecodeArgs a{p, v_cache, ctx, kv_lens, head_num, k_seq_len, size_per_head, v_stride_b, v_stride_h, v_stride_s, 1.f};
+  hipStream_t s = (hipStream_t)stream;
+  switch (dtype) {
+    case EN_F32: return dispatch_lpk<EN_F32, PvLauncher>(a, batch, s);
+    case EN_F16: return dispatch_lpk<EN_F16, PvLauncher>(a, batch, s);
+    default: return dispatch_lpk<EN_BF16, PvLauncher>(a, batch, s);
+  }
+}
+
+}  // extern "C"

@@ -1,0 +1,224 @@
+// LayerNorm forward with an optional fused residual add.
+//
+// Single pass over HBM: each row is read once into VGPRs with 128-bit loads
+// (TPR lanes share a row, VPL vectors per lane), the mean and then the
+// centred sum of squares are reduced from the registers (two-pass statistics
+// without a second trip to memory: wave64 DPP reductions, LDS only to combine
+// waves), and the normalised row is written once.  All arithmetic is fp32 with
+// a single rounding at the store.  Rows that do not fit the register tiling,
+// or are not 16-byte aligned, take the three-pass workgroup-per-row kernel.
+#include "common.hip.h"
+
+#include <math.h>
+
+namespace en {
+
+struct LnArgs {
+  void *out;
+  float *mean;
+  float *invvar;
+  void *sum_out;
+  const void *in;
+  const void *residual;
+  const void *gamma;
+  const void *beta;
+  int64_t n1;
+  int n2;
+  float eps;
+};
+
+template <int DTI, int DTO, int VPL, int TPR>
+__global__ __launch_bounds__(TPR < kBlock ? kBlock : TPR) void layernorm_rows_kernel(LnArgs a) {
+  typedef Elem<DTI> EI;
+  typedef Elem<DTO> EO;
+  typedef typename EI::T TI;
+  typedef typename EO::T TO;
+  constexpr int BLOCK = TPR < kBlock ? kBlock : TPR;
+  constexpr int EPV = 16 / EI::kSize;  // elements per 128-bit input vector
+  constexpr int NW = TPR / kWave;      // waves sharing a row
+  constexpr int ROWS_PER_BLOCK = BLOCK / TPR;
+  __shared__ float s_a[NW > 1 ? NW : 1];
+  __shared__ float s_b[NW > 1 ? NW : 1];
+
+  const int t = threadIdx.x % TPR;
+  const int64_t row = (int64_t)blockIdx.x * ROWS_PER_BLOCK + threadIdx.x / TPR;
+  const bool active = row < a.n1;  // uniform per wave (TPR is a multiple of 64)
+  if (!active) return;             // ROWS_PER_BLOCK > 1 only when a row is one wave: no barrier follows
+
+  const int nvec = a.n2 / EPV;
+  const TI *in = reinterpret_cast<const TI *>(a.in) + row * a.n2;
+  const TI *res = a.residual ? reinterpret_cast<const TI *>(a.residual) + row * a.n2 : nullptr;
+  TI *sum_out = a.sum_out ? reinterpret_cast<TI *>(a.sum_out) + row * a.n2 : nullptr;
+
+  float x[VPL][EPV];
+  float s = 0.f;
+#pragma unroll
+  for (int j = 0; j < VPL; ++j) {
+    const int v = t + TPR * j;
+    if (v < nvec) {
+      const Pack<TI, EPV> pk = load_pack<TI, EPV>(in + v * EPV);
+#pragma unroll
+      for (int e = 0; e < EPV; ++e) x[j][e] = EI::to_float(pk.v[e]);
+      if (res) {
+        const Pack<TI, EPV> rk = load_pack<TI, EPV>(res + v * EPV);
+#pragma unroll
+        for (int e = 0; e < EPV; ++e) x[j][e] += EI::to_float(rk.v[e]);
+      }
+      if (sum_out) {
+        Pack<TI, EPV> sk;
+#pragma unroll
+        for (int e = 0; e < EPV; ++e) sk.v[e] = EI::from_float(x[j][e]);
+        store_pack<TI, EPV>(sum_out + v * EPV, sk);
+      }
+#pragma unroll
+      for (int e = 0; e < EPV; ++e) s += x[j][e];
+    } else {
+#pragma unroll
+      for (int e = 0; e < EPV; ++e) x[j][e] = 0.f;
+    }
+  }
+  s = block_allreduce<OpSum, NW>(s, s_a);
+  const float mu = s / (float)a.n2;
+  float d2 = 0.f;
+#pragma unroll
+  for (int j = 0; j < VPL; ++j) {
+    const int v = t + TPR * j;
+    if (v < nvec) {
+#pragma unroll
+      for (int e = 0; e < EPV; ++e) {
+        const float d = x[j][e] - mu;
+        d2 += d * d;
+      }
+    }
+  }
+  d2 = block_allreduce<OpSum, NW>(d2, s_b);
+  const float var = d2 / (float)a.n2;
+  const float inv = 1.0f / sqrtf(var + a.eps);
+
+  const TO *gamma = reinterpret_cast<const TO *>(a.gamma);
+  const TO *beta = reinterpret_cast<const TO *>(a.beta);
+  TO *out = reinterpret_cast<TO *>(a.out) + row * a.n2;
+#pragma unroll
+  for (int j = 0; j < VPL; ++j) {
+    const int v = t + TPR * j;
+    if (v < nvec) {
+      const Pack<TO, EPV> g = load_pack<TO, EPV>(gamma + v * EPV);
+      const Pack<TO, EPV> bt = load_pack<TO, EPV>(beta + v * EPV);
+      Pack<TO, EPV> o;
+#pragma unroll
+      for (int e = 0; e < EPV; ++e)
+        o.v[e] = EO::from_float((x[j][e] - mu) * inv * EO::to_float(g.v[e]) + EO::to_float(bt.v[e]));
+      store_pack<TO, EPV>(out + v * EPV, o);
+    }
+  }
+  if (t == 0) {
+    if (a.mean) a.mean[row] = mu;
+    if (a.invvar) a.invvar[row] = inv;
+  }
+}
+
+// Any n2, any alignment: one workgroup per row, three strided passes.
+template <int DTI, int DTO>
+__global__ __launch_bounds__(kBlock) void layernorm_generic_kernel(LnArgs a) {
+  typedef Elem<DTI> EI;
+  typedef Elem<DTO> EO;
+  typedef typename EI::T TI;
+  typedef typename EO::T TO;
+  __shared__ float s_a[kBlock / kWave];
+  __shared__ float s_b[kBlock / kWave];
+  const int64_t row = blockIdx.x;
+  const TI *in = reinterpret_cast<const TI *>(a.in) + row * a.n2;
+  const TI *res = a.residual ? reinterpret_cast<const TI *>(a.residual) + row * a.n2 : nullptr;
+  TI *sum_out = a.sum_out ? reinterpret_cast<TI *>(a.sum_out) + row * a.n2 : nullptr;
+  float s = 0.f;
+  for (int i = threadIdx.x; i < a.n2; i += kBlock) {
+    float v = EI::to_float(in[i]);
+    if (res) v += EI::to_float(res[i]);
+    s += v;
+  }
+  s = block_allreduce<OpSum, kBlock / kWave>(s, s_a);
+  const float mu = s / (float)a.n2;
+  float d2 = 0.f;
+  for (int i = threadIdx.x; i < a.n2; i += kBlock) {
+    float v = EI::to_float(in[i]);
+    if (res) v += EI::to_float(res[i]);
+    d2 += (v - mu) * (v - mu);
+  }
+  d2 = block_allreduce<OpSum, kBlock / kWave>(d2, s_b);
+  const float inv = 1.0f / sqrtf(d2 / (float)a.n2 + a.eps);
+  const TO *gamma = reinterpret_cast<const TO *>(a.gamma);
+  const TO *beta = reinterpret_cast<const TO *>(a.beta);
+  TO *out = reinterpret_cast<TO *>(a.out) + row * a.n2;
+  for (int i = threadIdx.x; i < a.n2; i += kBlock) {
+    float v = EI::to_float(in[i]);
+    if (res) v += EI::to_float(res[i]);
+    if (sum_out) sum_out[i] = EI::from_float(v);
+    out[i] = EO::from_float((v - mu) * inv * EO::to_float(gamma[i]) + EO::to_float(beta[i]));
+  }
+  if (threadIdx.x == 0) {
+    if (a.mean) a.mean[row] = mu;
+    if (a.invvar) a.invvar[row] = inv;
+  }
+}
+
+template <int DTI, int DTO, int VPL, int TPR>
+static void launch_rows(const LnArgs &a, hipStream_t s) {
+  constexpr int BLOCK = TPR < kBlock ? kBlock : TPR;
+  constexpr int ROWS_PER_BLOCK = BLOCK / TPR;
+  layernorm_rows_kernel<DTI, DTO, VPL, TPR><<<(unsigned)ceil_div(a.n1, ROWS_PER_BLOCK), BLOCK, 0, s>>>(a);
+}
+
+template <int DTI, int DTO, int TPR>
+static bool launch_vpl(const LnArgs &a, int vpl, hipStream_t s) {
+  if (vpl <= 1) launch_rows<DTI, DTO, 1, TPR>(a, s);
+  else if (vpl <= 2) launch_rows<DTI, DTO, 2, TPR>(a, s);
+  else if (vpl <= 4) launch_rows<DTI, DTO, 4, TPR>(a, s);
+  else if (vpl <= 6) launch_rows<DTI, DTO, 6, TPR>(a, s);
+  else if (vpl <= 8) launch_rows<DTI, DTO, 8, TPR>(a, s);
+  else return false;
+  return true;
+}
+
+template <int DTI, int DTO>
+static int dispatch(const LnArgs &a, hipStream_t s) {
+  constexpr int EPV = 16 / Elem<DTI>::kSize;
+  constexpr int OUT_VEC_BYTES = EPV * Elem<DTO>::kSize;
+  if (a.n1 > (int64_t)INT32_MAX) return EN_ERR_SHAPE;
+  const bool vec_ok = (a.n2 % EPV) == 0 && aligned_to(a.in, 16) && aligned_to(a.out, OUT_VEC_BYTES) &&
+                      aligned_to(a.gamma, OUT_VEC_BYTES) && aligned_to(a.beta, OUT_VEC_BYTES) &&
+                      (!a.residual || aligned_to(a.residual, 16)) && (!a.sum_out || aligned_to(a.sum_out, 16));
+  const int nvec = vec_ok ? a.n2 / EPV : 0;
+  bool done = false;
+  if (vec_ok) {
+    if (nvec <= 2 * 64) done = launch_vpl<DTI, DTO, 64>(a, (nvec + 63) / 64, s);
+    else if (nvec <= 8 * 256) done = launch_vpl<DTI, DTO, 256>(a, (nvec + 255) / 256, s);
+    else if (nvec <= 8 * 1024) done = launch_vpl<DTI, DTO, 1024>(a, (nvec + 1023) / 1024, s);
+  }
+  if (!done) layernorm_generic_kernel<DTI, DTO><<<(unsigned)a.n1, kBlock, 0, s>>>(a);
+  EN_RETURN_IF_LAUNCH_FAILED();
+  return EN_OK;
+}
+
+}  // namespace en
+
+extern "C" int en_layernorm_fwd(void *out, float *mean, float *invvar, void *sum_out, const void *in,
+                                const void *residual, const void *gamma, const void *beta, int64_t n1, int64_t n2,
+                                float eps, int in_dtype, int out_dtype, en_stream_t stream) {
+  using namespace en;
+  if (!out || !in || !gamma || !beta) return EN_ERR_NULL;
+  if (n1 < 0 || n2 < 1 || n2 > (int64_t)INT32_MAX) return EN_ERR_SHAPE;
+  if (n1 == 0) return EN_OK;
+  const int esi = dtype_size(in_dtype), eso = dtype_size(out_dtype);
+  if (!esi || !eso) return EN_ERR_DTYPE;
+  if (!aligned_to(in, esi) || !aligned_to(out, eso) || !aligned_to(gamma, eso) || !aligned_to(beta, eso) ||
+      (residual && !aligned_to(residual, esi)) || (sum_out && !aligned_to(sum_out, esi)))
+    return EN_ERR_ALIGN;
+  LnArgs a{out, mean, invvar, sum_out, in, residual, gamma, beta, n1, (int)n2, eps};
+  hipStream_t s = (hipStream_t)stream;
+  if (in_dtype == EN_F32 && out_dtype == EN_F32) return dispatch<EN_F32, EN_F32>(a, s);
+  if (in_dtype == EN_F32 && out_dtype == EN_F16) return dispatch<EN_F32, EN_F16>(a, s);
+  if (in_dtype == EN_F32 && out_dtype == EN_BF16) return dispatch<EN_F32, EN_BF16>(a, s);
+  if (in_dtype == EN_F16 && out_dtype == EN_F16) return dispatch<EN_F16, EN_F16>(a, s);
+  if (in_dtype == EN_BF16 && out_dtype == EN_BF16) return dispatch<EN_BF16, EN_BF16>(a, s);
+  return EN_ERR_DTYPE;
+}

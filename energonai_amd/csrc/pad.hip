@@ -1,0 +1,423 @@
+// Packing / unpacking kernels: depad, transpose_pad, transpose_depad and the
+// ft_* offset family.  All of them are row gathers: an output row of `vpr`
+// vectors is either a copy of one input row or zero.  One kernel body does the
+// moving; a small "map" object per operation says, for each row of a block's
+// tile, where it comes from and where it goes.  The map is evaluated once per
+// row by the first lanes of the block and parked in LDS, so the per-sequence
+// offsets are looked up once per tile instead of once per element, and the
+// streaming loop is pure 128-bit loads and stores.
+//
+// Payloads are moved as raw bytes (vector type picked from row size and
+// pointer alignment), so every 2- and 4-byte dtype is bit-exact by
+// construction.
+#include "common.hip.h"
+
+namespace en {
+
+constexpr int kMaxTileRows = 64;     // rows a block may own
+constexpr int kTileVecs = 2048;      // target vectors (32 KiB at 16 B) per block
+constexpr int64_t kZeroRow = -1;     // source: write zeros
+constexpr int64_t kSkipRow = -1;     // destination: leave untouched
+
+struct Ptrs3 {
+  const void *src[3];
+  void *dst[3];
+};
+
+// ---------------------------------------------------------------------------
+// maps: operator()(tile_x, tile_y, r, &src_row, &dst_row) in units of rows of
+// the respective tensor; active(tile_x, tile_y) is a block-uniform early out.
+// ---------------------------------------------------------------------------
+
+// transpose_pad: grid.x = head + H * s_tile (heads fastest so that blocks in
+// flight together read neighbouring pieces of the same packed token rows).
+struct PadMap {
+  const int32_t *cu;
+  int H, S, R;
+  __device__ bool active(int, int) const { return true; }
+  __device__ void operator()(int tx, int b, int r, int64_t &src, int64_t &dst) const {
+    const int h = tx % H;
+    const int s = (tx / H) * R + r;
+    const int start = cu[b];
+    const int len = cu[b + 1] - start;
+    dst = (s < S) ? ((int64_t)b * H + h) * S + s : kSkipRow;
+    src = (s < len) ? ((int64_t)(start + s)) * H + h : kZeroRow;
+  }
+};
+
+// transpose_depad: same tiling, opposite direction; tiles past the sequence end exit.
+struct DepadHeadsMap {
+  const int32_t *cu;
+  int H, S, R;
+  __device__ bool active(int tx, int b) const { return (tx / H) * R < cu[b + 1] - cu[b]; }
+  __device__ void operator()(int tx, int b, int r, int64_t &src, int64_t &dst) const {
+    const int h = tx % H;
+    const int s = (tx / H) * R + r;
+    const int start = cu[b];
+    const int len = cu[b + 1] - start;
+    src = ((int64_t)b * H + h) * S + s;
+    dst = (s < len) ? ((int64_t)(start + s)) * H + h : kSkipRow;
+  }
+};
+
+// depad: rows of the whole hidden width; grid.x = s_tile, grid.y = b.
+struct DepadRowsMap {
+  const int32_t *cu;
+  int S, R, left;
+  __device__ bool active(int tx, int b) const { return tx * R < cu[b + 1] - cu[b]; }
+  __device__ void operator()(int tx, int b, int r, int64_t &src, int64_t &dst) const {
+    const int s = tx * R + r;
+    const int start = cu[b];
+    const int len = cu[b + 1] - start;
+    src = (int64_t)b * S + s + (left ? S - len : 0);
+    dst = (s < len) ? (int64_t)start + s : kSkipRow;
+  }
+};
+
+// ft_remove_padding: tgt[t] = src[t + off[t]]; also publishes mask_offset[t].
+struct FtRemoveMap {
+  const int32_t *tmp_off;
+  int32_t *mask_off;
+  int valid, R;
+  __device__ bool active(int, int) const { return true; }
+  __device__ void operator()(int tx, int, int r, int64_t &src, int64_t &dst) const {
+    const int t = tx * R + r;
+    if (t < valid) {
+      const int off = tmp_off[t];
+      mask_off[t] = off;
+      src = (int64_t)t + off;
+      dst = t;
+    } else {
+      src = kZeroRow;
+      dst = kSkipRow;
+    }
+  }
+};
+
+// ft_rebuild_padding: for each output row find the token t with t + off[t] == row
+// (t + off[t] is strictly increasing in t), else the row is padding -> zero.
+struct FtRebuildMap {
+  const int32_t *off;
+  int valid, rows_out, R;
+  __device__ bool active(int, int) const { return true; }
+  __device__ void operator()(int tx, int, int r, int64_t &src, int64_t &dst) const {
+    const int row = tx * R + r;
+    if (row >= rows_out) {
+      src = kZeroRow;
+      dst = kSkipRow;
+      return;
+    }
+    int lo = 0, hi = valid;  // first t with t + off[t] >= row
+    while (lo < hi) {
+      const int mid = (lo + hi) >> 1;
+      if (mid + off[mid] < row) lo = mid + 1; else hi = mid;
+    }
+    dst = row;
+    src = (lo < valid && lo + off[lo] == row) ? (int64_t)lo : kZeroRow;
+  }
+};
+
+// ft_transpose_rebuild_padding: [T,H,D] -> [B,H,S,D]; grid.x = head + H * t_tile.
+struct FtTransposeRebuildMap {
+  const int32_t *off;
+  int valid, H, S, R;
+  __device__ bool active(int, int) const { return true; }
+  __device__ void operator()(int tx, int, int r, int64_t &src, int64_t &dst) const {
+    const int h = tx % H;
+    const int t = (tx / H) * R + r;
+    if (t < valid) {
+      const int pos = t + off[t];
+      const int b = pos / S, s = pos - b * S;
+      src = (int64_t)t * H + h;
+      dst = ((int64_t)b * H + h) * S + s;
+    } else {
+      src = kZeroRow;
+      dst = kSkipRow;
+    }
+  }
+};
+
+// ft_transpose_remove_padding: the inverse gather.
+struct FtTransposeRemoveMap {
+  const int32_t *off;
+  int valid, H, S, R;
+  __device__ bool active(int, int) const { return true; }
+  __device__ void operator()(int tx, int, int r, int64_t &src, int64_t &dst) const {
+    const int h = tx % H;
+    const int t = (tx / H) * R + r;
+    if (t < valid) {
+      const int pos = t + off[t];
+      const int b = pos / S, s = pos - b * S;
+      src = ((int64_t)b * H + h) * S + s;
+      dst = (int64_t)t * H + h;
+    } else {
+      src = kZeroRow;
+      dst = kSkipRow;
+    }
+  }
+};
+
+// ---------------------------------------------------------------------------
+// the mover
+// ---------------------------------------------------------------------------
+template <typename Vec> __device__ __forceinline__ Vec zero_vec();
+template <> __device__ __forceinline__ uint4 zero_vec<uint4>() { return make_uint4(0, 0, 0, 0); }
+template <> __device__ __forceinline__ uint2 zero_vec<uint2>() { return make_uint2(0, 0); }
+template <> __device__ __forceinline__ uint32_t zero_vec<uint32_t>() { return 0u; }
+template <> __device__ __forceinline__ uint16_t zero_vec<uint16_t>() { return (uint16_t)0; }
+
+template <typename Vec, typename Map, int NT>
+__global__ __launch_bounds__(kBlock) void row_gather_kernel(Map map, Ptrs3 p, int vpr, int rows_per_block) {
+  __shared__ int64_t s_src[kMaxTileRows];
+  __shared__ int64_t s_dst[kMaxTileRows];
+  const int tid = threadIdx.x;
+  const int tx = blockIdx.x, ty = blockIdx.y;
+  if (!map.active(tx, ty)) return;
+  if (tid < rows_per_block) {
+    int64_t so, dn;
+    map(tx, ty, tid, so, dn);
+    s_src[tid] = so < 0 ? so : so * vpr;
+    s_dst[tid] = dn < 0 ? dn : dn * vpr;
+  }
+  __syncthreads();
+  constexpr int U = 4;
+  const int n = rows_per_block * vpr;
+#pragma unroll
+  for (int t = 0; t < NT; ++t) {
+    const Vec *__restrict__ src = reinterpret_cast<const Vec *>(p.src[t]);
+    Vec *__restrict__ dst = reinterpret_cast<Vec *>(p.dst[t]);
+    for (int i0 = tid; i0 < n; i0 += kBlock * U) {
+      Vec v[U];
+      int64_t d[U];
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const int i = i0 + u * kBlock;
+        d[u] = kSkipRow;
+        if (i < n) {
+          const int r = i / vpr;
+          const int c = i - r * vpr;
+          const int64_t so = s_src[r];
+          const int64_t dn = s_dst[r];
+          if (dn >= 0) {
+            d[u] = dn + c;
+            v[u] = (so >= 0) ? src[so + c] : zero_vec<Vec>();
+          }
+        }
+      }
+#pragma unroll
+      for (int u = 0; u < U; ++u)
+        if (d[u] >= 0) dst[d[u]] = v[u];
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------
+// host-side launch helpers
+// ---------------------------------------------------------------------------
+static int pick_vec_bytes(int64_t row_bytes, const Ptrs3 &p, int nt) {
+  int vb = 16;
+  while (vb > 2) {
+    bool ok = (row_bytes % vb) == 0;
+    for (int t = 0; t < nt && ok; ++t) ok = aligned_to(p.src[t], vb) && aligned_to(p.dst[t], vb);
+    if (ok) break;
+    vb >>= 1;
+  }
+  return vb;
+}
+
+static int tile_rows(int64_t vpr, int64_t total_rows) {
+  int64_t r = kTileVecs / (vpr > 0 ? vpr : 1);
+  if (r < 1) r = 1;
+  if (r > kMaxTileRows) r = kMaxTileRows;
+  if (r > total_rows) r = total_rows > 0 ? total_rows : 1;
+  return (int)r;
+}
+
+template <typename Map, int NT, typename MakeMap>
+static int launch_row_gather(int64_t row_bytes, int64_t tile_dim_rows, const Ptrs3 &p, MakeMap make_map,
+                             hipStream_t stream) {
+  const int vb = pick_vec_bytes(row_bytes, p, NT);
+  const int64_t vpr64 = row_bytes / vb;
+  if (vpr64 > (int64_t)INT32_MAX / kMaxTileRows) return EN_ERR_SHAPE;
+  const int vpr = (int)vpr64;
+  const int R = tile_rows(vpr, tile_dim_rows);
+  dim3 grid;
+  const Map map = make_map(R, grid);
+  if (grid.x == 0 || grid.y == 0) return EN_OK;
+  if (grid.y > 65535u) return EN_ERR_SHAPE;
+  switch (vb) {
+    case 16: row_gather_kernel<uint4, Map, NT><<<grid, kBlock, 0, stream>>>(map, p, vpr, R); break;
+    case 8: row_gather_kernel<uint2, Map, NT><<<grid, kBlock, 0, stream>>>(map, p, vpr, R); break;
+    case 4: row_gather_kernel<uint32_t, Map, NT><<<grid, kBlock, 0, stream>>>(map, p, vpr, R); break;
+    default: row_gather_kernel<uint16_t, Map, NT><<<grid, kBlock, 0, stream>>>(map, p, vpr, R); break;
+  }
+  EN_RETURN_IF_LAUNCH_FAILED();
+  return EN_OK;
+}
+
+// ---------------------------------------------------------------------------
+// ft_build_padding_offsets: one workgroup per sequence writes that sequence's
+// run of offsets; the exclusive prefix of (S - len) is recomputed per block from
+// the (short) length vector, 64 lengths per wave step.
+// ---------------------------------------------------------------------------
+__global__ __launch_bounds__(kBlock) void ft_build_offsets_kernel(const int32_t *__restrict__ lens, int batch,
+                                                                  int max_seq_len, int32_t *__restrict__ valid,
+                                                                  int32_t *__restrict__ tmp_off) {
+  __shared__ int32_t s_tok[kBlock / kWave];
+  __shared__ int32_t s_pad[kBlock / kWave];
+  const int b = blockIdx.x;
+  const int tid = threadIdx.x;
+  // tokens and padding before sequence b (block 0 of the tail also totals everything)
+  const int upto = (b == 0) ? batch : b;
+  int32_t tok = 0, pad = 0;
+  for (int i = tid; i < upto; i += kBlock) {
+    const int32_t n = lens[i];
+    tok += n;
+    pad += max_seq_len - n;
+  }
+  for (int off = 32; off > 0; off >>= 1) {
+    tok += __shfl_xor(tok, off, kWave);
+    pad += __shfl_xor(pad, off, kWave);
+  }
+  if ((tid & 63) == 0) {
+    s_tok[tid >> 6] = tok;
+    s_pad[tid >> 6] = pad;
+  }
+  __syncthreads();
+  tok = s_tok[0] + s_tok[1] + s_tok[2] + s_tok[3];
+  pad = s_pad[0] + s_pad[1] + s_pad[2] + s_pad[3];
+  if (b == 0) {
+    if (tid == 0) valid[0] = tok;
+    tok = 0;
+    pad = 0;
+  }
+  const int32_t n = lens[b];
+  for (int j = tid; j < n; j += kBlock) tmp_off[tok + j] = pad;
+}
+
+}  // namespace en
+
+using namespace en;
+
+static int check_elem(int elem_size) { return (elem_size == 2 || elem_size == 4) ? EN_OK : EN_ERR_DTYPE; }
+
+extern "C" {
+
+int en_depad(const void *src, void *dst, const int32_t *cu_seqlens, int batch, int max_seq_len, int64_t hidden,
+             int elem_size, int left_padded, en_stream_t stream) {
+  if (!src || !dst || !cu_seqlens) return EN_ERR_NULL;
+  if (check_elem(elem_size)) return EN_ERR_DTYPE;
+  if (batch < 1 || max_seq_len < 1 || hidden < 1) return EN_ERR_SHAPE;
+  if (!aligned_to(src, elem_size) || !aligned_to(dst, elem_size)) return EN_ERR_ALIGN;
+  Ptrs3 p = {{src, nullptr, nullptr}, {dst, nullptr, nullptr}};
+  return launch_row_gather<DepadRowsMap, 1>(hidden * elem_size, max_seq_len, p, [&](int R, dim3 &grid) {
+    grid = dim3((unsigned)ceil_div(max_seq_len, R), (unsigned)batch, 1);
+    return DepadRowsMap{cu_seqlens, max_seq_len, R, left_padded ? 1 : 0};
+  }, (hipStream_t)stream);
+}
+
+int en_transpose_pad(const void *src, void *dst, const int32_t *cu_seqlens, int batch, int max_seq_len, int head_num,
+                     int size_per_head, int elem_size, en_stream_t stream) {
+  if (!src || !dst || !cu_seqlens) return EN_ERR_NULL;
+  if (check_elem(elem_size)) return EN_ERR_DTYPE;
+  if (batch < 1 || max_seq_len < 1 || head_num < 1 || size_per_head < 1) return EN_ERR_SHAPE;
+  if (!aligned_to(src, elem_size) || !aligned_to(dst, elem_size)) return EN_ERR_ALIGN;
+  Ptrs3 p = {{src, nullptr, nullptr}, {dst, nullptr, nullptr}};
+  return launch_row_gather<PadMap, 1>((int64_t)size_per_head * elem_size, max_seq_len, p, [&](int R, dim3 &grid) {
+    grid = dim3((unsigned)(ceil_div(max_seq_len, R) * head_num), (unsigned)batch, 1);
+    return PadMap{cu_seqlens, head_num, max_seq_len, R};
+  }, (hipStream_t)stream);
+}
+
+int en_transpose_depad(const void *src, void *dst, const int32_t *cu_seqlens, int batch, int max_seq_len,
+                       int head_num, int size_per_head, int elem_size, en_stream_t stream) {
+  if (!src || !dst || !cu_seqlens) return EN_ERR_NULL;
+  if (check_elem(elem_size)) return EN_ERR_DTYPE;
+  if (batch < 1 || max_seq_len < 1 || head_num < 1 || size_per_head < 1) return EN_ERR_SHAPE;
+  if (!aligned_to(src, elem_size) || !aligned_to(dst, elem_size)) return EN_ERR_ALIGN;
+  Ptrs3 p = {{src, nullptr, nullptr}, {dst, nullptr, nullptr}};
+  return launch_row_gather<DepadHeadsMap, 1>((int64_t)size_per_head * elem_size, max_seq_len, p,
+                                             [&](int R, dim3 &grid) {
+    grid = dim3((unsigned)(ceil_div(max_seq_len, R) * head_num), (unsigned)batch, 1);
+    return DepadHeadsMap{cu_seqlens, head_num, max_seq_len, R};
+  }, (hipStream_t)stream);
+}
+
+int en_ft_build_offsets(const int32_t *seq_lens, int batch, int max_seq_len, int32_t *valid_word_num,
+                        int32_t *tmp_mask_offset, en_stream_t stream) {
+  if (!seq_lens || !valid_word_num || !tmp_mask_offset) return EN_ERR_NULL;
+  if (batch < 1 || max_seq_len < 1) return EN_ERR_SHAPE;
+  ft_build_offsets_kernel<<<batch, kBlock, 0, (hipStream_t)stream>>>(seq_lens, batch, max_seq_len, valid_word_num,
+                                                                      tmp_mask_offset);
+  EN_RETURN_IF_LAUNCH_FAILED();
+  return EN_OK;
+}
+
+int en_ft_remove_padding(const void *src, void *tgt, const int32_t *tmp_mask_offset, int32_t *mask_offset,
+                         int valid_word_num, int64_t hidden, int elem_size, en_stream_t stream) {
+  if (!src || !tgt || !tmp_mask_offset || !mask_offset) return EN_ERR_NULL;
+  if (check_elem(elem_size)) return EN_ERR_DTYPE;
+  if (valid_word_num < 0 || hidden < 1) return EN_ERR_SHAPE;
+  if (valid_word_num == 0) return EN_OK;
+  if (!aligned_to(src, elem_size) || !aligned_to(tgt, elem_size)) return EN_ERR_ALIGN;
+  Ptrs3 p = {{src, nullptr, nullptr}, {tgt, nullptr, nullptr}};
+  return launch_row_gather<FtRemoveMap, 1>(hidden * elem_size, valid_word_num, p, [&](int R, dim3 &grid) {
+    grid = dim3((unsigned)ceil_div(valid_word_num, R), 1, 1);
+    return FtRemoveMap{tmp_mask_offset, mask_offset, valid_word_num, R};
+  }, (hipStream_t)stream);
+}
+
+int en_ft_rebuild_padding(const void *src, void *tgt, const int32_t *mask_offset, int valid_word_num,
+                          int64_t hidden, int batch, int max_seq_len, int elem_size, en_stream_t stream) {
+  if (!src || !tgt || !mask_offset) return EN_ERR_NULL;
+  if (check_elem(elem_size)) return EN_ERR_DTYPE;
+  if (valid_word_num < 0 || hidden < 1 || batch < 1 || max_seq_len < 1) return EN_ERR_SHAPE;
+  const int64_t rows_out = (int64_t)batch * max_seq_len;
+  if (rows_out > INT32_MAX || valid_word_num > rows_out) return EN_ERR_SHAPE;
+  if (!aligned_to(src, elem_size) || !aligned_to(tgt, elem_size)) return EN_ERR_ALIGN;
+  Ptrs3 p = {{src, nullptr, nullptr}, {tgt, nullptr, nullptr}};
+  return launch_row_gather<FtRebuildMap, 1>(hidden * elem_size, rows_out, p, [&](int R, dim3 &grid) {
+    grid = dim3((unsigned)ceil_div(rows_out, R), 1, 1);
+    return FtRebuildMap{mask_offset, valid_word_num, (int)rows_out, R};
+  }, (hipStream_t)stream);
+}
+
+int en_ft_transpose_rebuild(const void *Q, const void *K, const void *V, void *q_buf, void *k_buf, void *v_buf,
+                            int batch, int seq_len, int head_num, int size_per_head, int valid_word_num,
+                            const int32_t *mask_offset, int elem_size, en_stream_t stream) {
+  if (!Q || !q_buf || !mask_offset) return EN_ERR_NULL;
+  if ((K == nullptr) != (k_buf == nullptr) || (V == nullptr) != (v_buf == nullptr)) return EN_ERR_NULL;
+  if (V && !K) return EN_ERR_NULL;
+  if (check_elem(elem_size)) return EN_ERR_DTYPE;
+  if (batch < 1 || seq_len < 1 || head_num < 1 || size_per_head < 1 || valid_word_num < 0) return EN_ERR_SHAPE;
+  if (valid_word_num == 0) return EN_OK;
+  Ptrs3 p = {{Q, K, V}, {q_buf, k_buf, v_buf}};
+  const int nt = V ? 3 : (K ? 2 : 1);
+  for (int t = 0; t < nt; ++t)
+    if (!aligned_to(p.src[t], elem_size) || !aligned_to(p.dst[t], elem_size)) return EN_ERR_ALIGN;
+  auto mk = [&](int R, dim3 &grid) {
+    grid = dim3((unsigned)(ceil_div(valid_word_num, R) * head_num), 1, 1);
+    return FtTransposeRebuildMap{mask_offset, valid_word_num, head_num, seq_len, R};
+  };
+  const int64_t row_bytes = (int64_t)size_per_head * elem_size;
+  if (nt == 3) return launch_row_gather<FtTransposeRebuildMap, 3>(row_bytes, valid_word_num, p, mk, (hipStream_t)stream);
+  if (nt == 2) return launch_row_gather<FtTransposeRebuildMap, 2>(row_bytes, valid_word_num, p, mk, (hipStream_t)stream);
+  return launch_row_gather<FtTransposeRebuildMap, 1>(row_bytes, valid_word_num, p, mk, (hipStream_t)stream);
+}
+
+int en_ft_transpose_remove(const void *src, void *dst, int valid_word_num, int batch, int seq_len, int head_num,
+                           int size_per_head, const int32_t *mask_offset, int elem_size, en_stream_t stream) {
+  if (!src || !dst || !mask_offset) return EN_ERR_NULL;
+  if (check_elem(elem_size)) return EN_ERR_DTYPE;
+  if (batch < 1 || seq_len < 1 || head_num < 1 || size_per_head < 1 || valid_word_num < 0) return EN_ERR_SHAPE;
+  if (valid_word_num == 0) return EN_OK;
+  if (!aligned_to(src, elem_size) || !aligned_to(dst, elem_size)) return EN_ERR_ALIGN;
+  Ptrs3 p = {{src, nullptr, nullptr}, {dst, nullptr, nullptr}};
+  return launch_row_gather<FtTransposeRemoveMap, 1>((int64_t)size_per_head * elem_size, valid_word_num, p,
+                                                    [&](int R, dim3 &grid) {
+    grid = dim3((unsigned)(ceil_div(valid_word_num, R) * head_num), 1, 1);
+    return FtTransposeRemoveMap{mask_offset, valid_word_num, head_num, seq_len, R};
+  }, (hipStream_t)stream);
+}
+
+}  // extern "C"

@@ -1,0 +1,127 @@
+"""The two attention contractions of the padding-removal path.
+
+The reference callers use ``torch.matmul`` on the padded ``[B,H,S,*]`` tensors
+(examples/bert/bert.py:108-119, examples/gpt/gpt.py:108-125) and therefore pay
+for every padded row and every masked key.  ``attn_qk`` / ``attn_pv`` compute
+only what the softmax uses: valid query rows and, under a causal mask, the keys
+at or left of the diagonal.  ``q``, ``k`` and ``v`` may be the strided
+``chunk(3, -1)`` views of the fused ``[B,H,S,3D]`` buffer; no copy is made.
+``decode_qk`` / ``decode_pv`` are the single-query forms for cached decode.
+"""
+from __future__ import annotations
+
+from typing import Optional
+
+import torch
+
+from .. import _lib
+from ..seqinfo import seq_info
+
+
+def _bhsd(t: torch.Tensor, name: str):
+    _lib.require_gpu(t, name, contiguous=False)
+    if t.dim() != 4:
+        raise RuntimeError(f"{name} must be [batch, head, seq, size_per_head]")
+    if t.stride(3) != 1:
+        raise RuntimeError(f"{name}: the last dimension must be contiguous")
+    return t.stride(0), t.stride(1), t.stride(2)
+
+
+def _lens_ptrs(seq_len_list, q_len_list, batch_size, device):
+    k_info = seq_info(seq_len_list, batch_size, device)
+    q_ptr = 0
+    if q_len_list is not None:
+        q_ptr = seq_info(q_len_list, batch_size, device).lens.data_ptr()
+    return k_info, q_ptr
+
+
+def attn_qk(q, k, seq_len_list, *, alpha: float = 1.0, causal: bool = True, q_len_list=None,
+            out: Optional[torch.Tensor] = None):
+    """scores[b,h,i,j] = alpha * <q[b,h,i,:], k[b,h,j,:]> as a new ``[B,H,Sq,Sk]`` tensor.
+
+    Only rows of valid queries and (rounded up to the 128-key tile) the keys
+    they can see are written; the rest of ``scores`` is uninitialised, exactly
+    the region ``scale_mask_softmax`` never reads.
+    """
+    qs = _bhsd(q, "q")
+    ks = _bhsd(k, "k")
+    B, H, Sq, D = q.shape
+    if k.shape[0] != B or k.shape[1] != H or k.shape[3] != D or k.dtype != q.dtype:
+        raise RuntimeError("attn_qk: q and k disagree in batch, heads, size_per_head or dtype")
+    Sk = k.shape[2]
+    k_info, q_ptr = _lens_ptrs(seq_len_list, q_len_list, B, q.device)
+    if out is None:
+        out = torch.empty((B, H, Sq, Sk), dtype=q.dtype, device=q.device)
+    else:
+        _lib.require_gpu(out, "out")
+        if out.shape != (B, H, Sq, Sk) or out.dtype != q.dtype:
+            raise RuntimeError("attn_qk: out must be a contiguous [B,H,Sq,Sk] tensor of q's dtype")
+    with torch.cuda.device(q.device):
+        _lib.check(_lib.load().en_attn_qk(q.data_ptr(), k.data_ptr(), out.data_ptr(), k_info.lens.data_ptr(), q_ptr,
+                                          B, H, Sq, Sk, D, *qs, *ks, float(alpha), int(bool(causal)),
+                                          _lib.dtype_tag(q, "attn_qk"), _lib.stream_of(q)), "attn_qk")
+    return out
+
+
+def attn_pv(p, v, seq_len_list, *, causal: bool = True, q_len_list=None, zero_padding: bool = False,
+            out: Optional[torch.Tensor] = None):
+    """ctx[b,h,i,:] = sum_j p[b,h,i,j] v[b,h,j,:] as ``[B,H,Sq,D]``; ``p`` as left by scale_mask_softmax.
+
+    Rows of padded queries are left uninitialised unless ``zero_padding``.
+    """
+    _lib.require_gpu(p, "p")
+    vs = _bhsd(v, "v")
+    if p.dim() != 4:
+        raise RuntimeError("p must be [batch, head, q_seq, k_seq]")
+    B, H, Sq, Sk = p.shape
+    D = v.shape[3]
+    if v.shape[0] != B or v.shape[1] != H or v.shape[2] != Sk or v.dtype != p.dtype:
+        raise RuntimeError("attn_pv: p and v disagree in batch, heads, key length or dtype")
+    k_info, q_ptr = _lens_ptrs(seq_len_list, q_len_list, B, p.device)
+    if out is None:
+        out = torch.empty((B, H, Sq, D), dtype=p.dtype, device=p.device)
+    else:
+        _bhsd(out, "out")
+        if out.shape != (B, H, Sq, D) or out.dtype != p.dtype:
+            raise RuntimeError("attn_pv: out must be [B,H,Sq,D] of p's dtype")
+    cs = (out.stride(0), out.stride(1), out.stride(2))
+    with torch.cuda.device(p.device):
+        _lib.check(_lib.load().en_attn_pv(p.data_ptr(), v.data_ptr(), out.data_ptr(), k_info.lens.data_ptr(), q_ptr,
+                                          B, H, Sq, Sk, D, *vs, *cs, int(bool(causal)), int(bool(zero_padding)),
+                                          _lib.dtype_tag(p, "attn_pv"), _lib.stream_of(p)), "attn_pv")
+    return out
+
+
+def decode_qk(q, k_cache, kv_len_list, *, alpha: float = 1.0, out: Optional[torch.Tensor] = None):
+    """scores[b,h,0,j] = alpha * <q[b,h,0,:], k_cache[b,h,j,:]> for j < kv_len[b]; ``[B,H,1,Smax]``."""
+    _lib.require_gpu(q, "q", contiguous=False)
+    ks = _bhsd(k_cache, "k_cache")
+    B, H, Smax, D = k_cache.shape
+    q_ = q.reshape(B, H, D).contiguous()
+    if q_.dtype != k_cache.dtype:
+        raise RuntimeError("decode_qk: q and k_cache must share one dtype")
+    info = seq_info(kv_len_list, B, q.device)
+    if out is None:
+        out = torch.empty((B, H, 1, Smax), dtype=q.dtype, device=q.device)
+    with torch.cuda.device(q.device):
+        _lib.check(_lib.load().en_decode_qk(q_.data_ptr(), k_cache.data_ptr(), out.data_ptr(), info.lens.data_ptr(),
+                                            B, H, Smax, D, *ks, float(alpha), _lib.dtype_tag(q, "decode_qk"),
+                                            _lib.stream_of(q)), "decode_qk")
+    return out
+
+
+def decode_pv(p, v_cache, kv_len_list, *, out: Optional[torch.Tensor] = None):
+    """ctx[b,h,0,:] = sum_{j<kv_len[b]} p[b,h,0,j] v_cache[b,h,j,:]; ``[B,H,1,D]``."""
+    _lib.require_gpu(p, "p")
+    vs = _bhsd(v_cache, "v_cache")
+    B, H, Smax, D = v_cache.shape
+    if p.numel() != B * H * Smax or p.dtype != v_cache.dtype:
+        raise RuntimeError("decode_pv: p must be [B,H,1,Smax] of v_cache's dtype")
+    info = seq_info(kv_len_list, B, p.device)
+    if out is None:
+        out = torch.empty((B, H, 1, D), dtype=p.dtype, device=p.device)
+    with torch.cuda.device(p.device):
+        _lib.check(_lib.load().en_decode_pv(p.data_ptr(), v_cache.data_ptr(), out.data_ptr(), info.lens.data_ptr(),
+                                            B, H, Smax, D, *vs, _lib.dtype_tag(p, "decode_pv"), _lib.stream_of(p)),
+                   "decode_pv")
+    return out

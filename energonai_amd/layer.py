@@ -1,0 +1,89 @@
+"""One transformer layer's padding-removal hot path, composed from the kernel API.
+
+    depad -> transpose_pad -> QK^T -> scale_mask_softmax -> PV -> transpose_depad
+          -> residual + LayerNorm
+
+This is the call sequence of the reference's BERT/GPT blocks
+(examples/bert/bert.py:54-62,91-134, examples/gpt/gpt.py:93-137) with the dense
+projections left to the caller: ``qkv_packed`` is what ``query_key_value``
+returns, and the residual + LayerNorm consumes either the attention output
+itself (when heads*size_per_head equals the LayerNorm width) or ``dense_out``,
+the output of the row-parallel ``dense``.
+"""
+from __future__ import annotations
+
+from typing import Dict, Optional
+
+import torch
+
+from .kernel import (attn_pv, attn_qk, decode_pv, decode_qk, depad, layer_norm_forward, scale_mask_softmax,
+                     transpose_depad, transpose_pad)
+from .seqinfo import SeqInfo, seq_info
+
+
+def padding_removal_layer(hidden_padded: torch.Tensor, qkv_packed: torch.Tensor, seq_lens, head_num: int,
+                          size_per_head: int, gamma: torch.Tensor, beta: torch.Tensor, eps: float = 1e-5,
+                          scale: Optional[float] = None, causal: bool = True, left_padded: bool = False,
+                          dense_out: Optional[torch.Tensor] = None, sum_seq: Optional[int] = None,
+                          keep: bool = False):
+    """Runs the seven ops on ``hidden_padded`` [B,S,hid] and ``qkv_packed`` [1,T,H,3D].
+
+    Returns the normalised ``[1,T,hid]`` output, or a dict of every
+    intermediate when ``keep`` is set.
+    """
+    B, S, hid = hidden_padded.shape
+    H, D = head_num, size_per_head
+    info = seq_info(seq_lens, B, hidden_padded.device)
+    T = info.total if sum_seq is None else int(sum_seq)
+    scale = float(D) ** -0.5 if scale is None else scale
+
+    x = depad(hidden_padded, B, info, left_padded=left_padded, sum_seq=T)
+    qkv = transpose_pad(qkv_packed, B, S, info, H, 3 * D)
+    q, k, v = torch.chunk(qkv, 3, dim=-1)
+    scores = attn_qk(q, k, info, causal=causal)
+    probs = scale_mask_softmax(B, S, H, scores, info, scale=scale, causal=causal)
+    ctx = attn_pv(probs, v, info, causal=causal)
+    ctx_packed = transpose_depad(ctx, B, T, S, info, H, D)
+    attn_out = ctx_packed.view(1, T, H * D) if dense_out is None else dense_out
+    y = layer_norm_forward(attn_out, gamma, beta, (hid,), eps, residual=x)
+    if keep:
+        return dict(x=x, qkv=qkv, probs=probs, ctx=ctx, ctx_packed=ctx_packed, y=y)
+    return y
+
+
+def decode_layer(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, kv_lens, residual: torch.Tensor,
+                 gamma: torch.Tensor, beta: torch.Tensor, eps: float = 1e-5, scale: Optional[float] = None,
+                 dense_out: Optional[torch.Tensor] = None, keep: bool = False):
+    """One cached decode step: a single new query per sequence against a ragged
+    cache, then transpose_depad and residual + LayerNorm on the B new tokens.
+
+    q [B,H,1,D]; caches [B,H,Smax,D]; residual [1,B,hid].
+    """
+    B, H, _, D = q.shape
+    Smax = k_cache.shape[2]
+    hid = gamma.numel()
+    info = seq_info(kv_lens, B, q.device)
+    scale = float(D) ** -0.5 if scale is None else scale
+    ones = _ones_info(B, q.device)
+
+    scores = decode_qk(q, k_cache, info)
+    probs = scale_mask_softmax(B, 1, H, scores, info, scale=scale, causal=True, k_seq_len=Smax, q_len_list=ones)
+    ctx = decode_pv(probs, v_cache, info)
+    ctx_packed = transpose_depad(ctx, B, B, 1, ones, H, D)
+    attn_out = ctx_packed.view(1, B, H * D) if dense_out is None else dense_out
+    y = layer_norm_forward(attn_out, gamma, beta, (hid,), eps, residual=residual)
+    if keep:
+        return dict(scores_probs=probs, ctx=ctx, ctx_packed=ctx_packed, y=y)
+    return y
+
+
+_ones_cache: Dict[tuple, SeqInfo] = {}
+
+
+def _ones_info(batch: int, device) -> SeqInfo:
+    key = (batch, str(device))
+    info = _ones_cache.get(key)
+    if info is None:
+        info = seq_info(torch.ones(batch, dtype=torch.int32), batch, device)
+        _ones_cache[key] = info
+    return info

@@ -1,0 +1,104 @@
+"""Per-batch sequence bookkeeping shared by every kernel call of a forward pass.
+
+The reference recomputes the prefix of ``seq_lens`` inside every block of every
+kernel (csrc/transpose_pad_fusion_kernel.cu:24-27,70-73).  Here the prefix is
+computed once per batch by one small kernel and reused by every op of every
+layer; the public functions still accept the plain ``seq_lens`` tensor of the
+reference API (int32 or int64, examples/bert/bert.py:100-103) and find the
+cached offsets through :func:`seq_info`.
+"""
+from __future__ import annotations
+
+from collections import OrderedDict
+from typing import Optional
+
+import torch
+
+from . import _lib
+
+_CACHE_SIZE = 16
+
+
+class SeqInfo:
+    """Device-resident int32 lengths and exclusive prefix for one batch."""
+
+    __slots__ = ("lens", "cu_seqlens", "batch_size", "_total", "_source")
+
+    def __init__(self, lens: torch.Tensor, cu_seqlens: torch.Tensor, batch_size: int, total: Optional[int], source):
+        self.lens = lens                # int32 [B] on the device
+        self.cu_seqlens = cu_seqlens    # int32 [B+1] on the device
+        self.batch_size = batch_size
+        self._total = total
+        self._source = source           # keeps the caller's tensor alive while cached
+
+    @property
+    def device(self) -> torch.device:
+        return self.lens.device
+
+    @property
+    def total(self) -> int:
+        """Sum of the lengths as a Python int.  The first use copies one int from
+        the device (a sync), like ``valid_word_num[0].item()`` in the reference
+        callers (examples/gpt/gpt.py:303); later uses are free."""
+        if self._total is None:
+            self._total = int(self.cu_seqlens[self.batch_size].item())
+        return self._total
+
+
+_cache: "OrderedDict[tuple, SeqInfo]" = OrderedDict()
+
+
+def build_seq_info(seq_lens, batch_size: int, device=None, total: Optional[int] = None) -> SeqInfo:
+    """Runs the prefix-sum kernel.  ``seq_lens`` is a CUDA int32/int64 tensor, or
+    a CPU tensor / list (then the total is known without a sync)."""
+    if not isinstance(seq_lens, torch.Tensor):
+        seq_lens = torch.as_tensor(list(seq_lens), dtype=torch.int32)
+    if seq_lens.dtype not in (torch.int32, torch.int64):
+        raise RuntimeError(f"seq_lens must be int32 or int64, got {seq_lens.dtype}")
+    if seq_lens.numel() < batch_size:
+        raise RuntimeError(f"seq_lens has {seq_lens.numel()} entries, batch_size is {batch_size}")
+    source = seq_lens
+    if not seq_lens.is_cuda:
+        if total is None:
+            total = int(seq_lens[:batch_size].sum())
+        if device is None:
+            device = torch.device("cuda", torch.cuda.current_device())
+        seq_lens = seq_lens.to(device, non_blocking=False)
+    seq_lens = seq_lens.contiguous()
+    lib = _lib.load()
+    with torch.cuda.device(seq_lens.device):
+        cu = torch.empty(batch_size + 1, dtype=torch.int32, device=seq_lens.device)
+        lens32 = torch.empty(batch_size, dtype=torch.int32, device=seq_lens.device)
+        _lib.check(lib.en_prefix_sum(seq_lens.data_ptr(), int(seq_lens.dtype == torch.int64), batch_size,
+                                     cu.data_ptr(), lens32.data_ptr(), _lib.stream_of(seq_lens)), "prefix_sum")
+    return SeqInfo(lens32, cu, batch_size, total, source)
+
+
+def seq_info(seq_lens, batch_size: int, device=None) -> SeqInfo:
+    """Returns the (cached) SeqInfo for ``seq_lens``.
+
+    A SeqInfo passes through unchanged.  Tensors are cached by identity and
+    version counter, and the cache holds a reference to the tensor so its
+    storage cannot be recycled under a stale entry; in-place edits through torch
+    bump the version and miss the cache.
+    """
+    if isinstance(seq_lens, SeqInfo):
+        if seq_lens.batch_size != batch_size:
+            raise RuntimeError(f"SeqInfo was built for batch {seq_lens.batch_size}, call passes {batch_size}")
+        return seq_lens
+    if not isinstance(seq_lens, torch.Tensor):
+        return build_seq_info(seq_lens, batch_size, device)
+    key = (id(seq_lens), seq_lens._version, seq_lens.data_ptr(), batch_size, str(device))
+    hit = _cache.get(key)
+    if hit is not None and hit._source is seq_lens:
+        _cache.move_to_end(key)
+        return hit
+    info = build_seq_info(seq_lens, batch_size, device)
+    _cache[key] = info
+    while len(_cache) > _CACHE_SIZE:
+        _cache.popitem(last=False)
+    return info
+
+
+def clear_cache() -> None:
+    _cache.clear()

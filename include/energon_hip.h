@@ -1,0 +1,179 @@
+/* energon_hip.h — C ABI of libenergon_hip.so (gfx950 / MI355X).
+ *
+ * One shared library replaces the reference's four pybind11 torch extensions
+ * for the padding-removal path (energonai_transpose_pad, energonai_scale_mask,
+ * energonai_layer_norm; reference setup.py:132-147).  Every entry point takes
+ * raw device pointers, plain integer extents, a dtype tag and the HIP stream
+ * to launch on; it never allocates, frees or retains device memory, never
+ * synchronises the host, and returns 0 on success or a negative en_status.
+ *
+ * Paths cited below are relative to the reference checkout,
+ * energonai/kernel/cuda_native/.
+ */
+#ifndef ENERGON_HIP_H
+#define ENERGON_HIP_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef void *en_stream_t; /* a hipStream_t; NULL = the legacy default stream */
+
+enum en_dtype { EN_F32 = 0, EN_F16 = 1, EN_BF16 = 2 };
+
+enum en_status {
+  EN_OK = 0,
+  EN_ERR_NULL = -1,        /* a required pointer is NULL */
+  EN_ERR_SHAPE = -2,       /* an extent is negative, zero where it may not be, or exceeds a kernel limit */
+  EN_ERR_DTYPE = -3,       /* dtype tag or element size not supported by this entry point */
+  EN_ERR_ALIGN = -4,       /* pointer or stride not aligned to the element size */
+  EN_ERR_UNSUPPORTED = -5, /* valid request this build has no kernel for (message names it) */
+  EN_ERR_HIP = -6          /* the HIP runtime reported an error; see en_last_hip_error() */
+};
+
+/* Library version (major*10000 + minor*100 + patch). */
+int en_version(void);
+/* Static description of an en_status value. */
+const char *en_status_string(int status);
+/* hipError_t (as int) recorded by the last EN_ERR_HIP on this thread, and its text. */
+int en_last_hip_error(void);
+const char *en_last_hip_error_string(void);
+
+/* ---- offsets ---------------------------------------------------------- */
+
+/* cu_seqlens[b] = sum_{b'<b} seq_lens[b'], cu_seqlens[batch] = total.
+ * Replaces the serial prefix loop every reference block runs
+ * (csrc/transpose_pad_fusion_kernel.cu:24-27,70-73).  seq_lens is int32, or
+ * int64 when lens_are_i64 != 0 (the reference test passes int64,
+ * tests/test_kernel/test_transpose_pad_fusion_kernel.py:6); lens32_out, if not
+ * NULL, receives the lengths as int32.  batch <= 65536. */
+int en_prefix_sum(const void *seq_lens, int lens_are_i64, int batch, int32_t *cu_seqlens, int32_t *lens32_out,
+                  en_stream_t stream);
+
+/* ---- packing / unpacking (bit-exact, any 2- or 4-byte element) ---------- */
+
+/* depad: [B,S,hid] -> [T,hid], valid rows only (transpose_pad.py:30-37).
+ * left_padded != 0 takes rows S-len..S of each sequence instead of 0..len. */
+int en_depad(const void *src, void *dst, const int32_t *cu_seqlens, int batch, int max_seq_len, int64_t hidden,
+             int elem_size, int left_padded, en_stream_t stream);
+
+/* transpose_pad_wrapper (csrc/transpose_pad_fusion_wrapper.cpp:33-57, kernel
+ * csrc/transpose_pad_fusion_kernel.cu:58-96): [T,H,Dk] -> [B,H,S,Dk]; every
+ * byte of dst is written, padding rows as zero. */
+int en_transpose_pad(const void *src, void *dst, const int32_t *cu_seqlens, int batch, int max_seq_len, int head_num,
+                     int size_per_head, int elem_size, en_stream_t stream);
+
+/* transpose_depad_wrapper (wrapper.cpp:59-83, kernel.cu:8-46):
+ * [B,H,S,D] -> [T,H,D]; every byte of dst is written when T = cu_seqlens[B]. */
+int en_transpose_depad(const void *src, void *dst, const int32_t *cu_seqlens, int batch, int max_seq_len,
+                       int head_num, int size_per_head, int elem_size, en_stream_t stream);
+
+/* ft_build_padding_offsets_wrapper (wrapper.cpp:96-107, kernel.cu:112-139):
+ * tmp_mask_offset[t] = sum_{b'<b(t)} (max_seq_len - len[b']) for each valid
+ * token t; valid_word_num[0] = T.  seq_lens int32. */
+int en_ft_build_offsets(const int32_t *seq_lens, int batch, int max_seq_len, int32_t *valid_word_num,
+                        int32_t *tmp_mask_offset, en_stream_t stream);
+
+/* ft_remove_padding_wrapper (wrapper.cpp:113-139, kernel.cu:142-166):
+ * tgt[t,:] = src[t + tmp_mask_offset[t],:]; also copies the offsets into
+ * mask_offset. */
+int en_ft_remove_padding(const void *src, void *tgt, const int32_t *tmp_mask_offset, int32_t *mask_offset,
+                         int valid_word_num, int64_t hidden, int elem_size, en_stream_t stream);
+
+/* ft_rebuild_padding_wrapper (wrapper.cpp:146-172, kernel.cu:178-199):
+ * tgt[B*S,hid]: row t + mask_offset[t] = src[t,:], all other rows zero; every
+ * byte of tgt is written (no separate memset). */
+int en_ft_rebuild_padding(const void *src, void *tgt, const int32_t *mask_offset, int valid_word_num,
+                          int64_t hidden, int batch, int max_seq_len, int elem_size, en_stream_t stream);
+
+/* ft_transpose_rebuild_padding_wrapper (wrapper.cpp:181-209, kernel.cu:213-255):
+ * Q,K,V [T,H,D] -> caller-owned q_buf,k_buf,v_buf [B,H,S,D]; padding rows of the
+ * buffers are not touched.  K/V (and their buffers) may be NULL to move one
+ * tensor only.  No limit on H*D. */
+int en_ft_transpose_rebuild(const void *Q, const void *K, const void *V, void *q_buf, void *k_buf, void *v_buf,
+                            int batch, int seq_len, int head_num, int size_per_head, int valid_word_num,
+                            const int32_t *mask_offset, int elem_size, en_stream_t stream);
+
+/* ft_transpose_remove_padding_wrapper (wrapper.cpp:218-244, kernel.cu:268-305):
+ * [B,H,S,D] -> [T,H*D]. */
+int en_ft_transpose_remove(const void *src, void *dst, int valid_word_num, int batch, int seq_len, int head_num,
+                           int size_per_head, const int32_t *mask_offset, int elem_size, en_stream_t stream);
+
+/* ---- scale + mask + softmax ------------------------------------------- */
+
+/* scale_mask_softmax_wrapper (csrc/scale_mask_softmax_wrapper.cpp:25-44, kernel
+ * csrc/scale_mask_softmax_kernel.cu:11-57), in place on src [B,H,Sq,Sk].
+ * For each b and each query row q < q_lens[b]: the first n visible entries
+ * become softmax(scale * src[..., :n]) and the remaining Sk-n entries zero;
+ * n = k_lens[b] when causal == 0, else min(k_lens[b], q + k_lens[b] - q_lens[b] + 1).
+ * Rows q >= q_lens[b] are not touched (as in the reference, kernel.cu:14-17).
+ * q_lens == NULL means q_lens[b] = min(k_lens[b], Sq).  The reference call is
+ * Sq == Sk, scale 1, causal 1, q_lens NULL.  No limit on Sk; fp32 math. */
+int en_scale_mask_softmax(void *src, const int32_t *k_lens, const int32_t *q_lens, int batch, int head_num,
+                          int q_seq_len, int k_seq_len, float scale, int causal, int dtype, en_stream_t stream);
+
+/* ---- LayerNorm forward -------------------------------------------------- */
+
+/* forward_affine (csrc/layer_norm_cuda.cpp:82-103, kernel
+ * csrc/layer_norm_cuda_kernel.cu:243-279,571-601): rows [n1,n2];
+ * x = in (+ residual, added in fp32, when residual != NULL);
+ * out = gamma * (x - mean) * rsqrt(var + eps) + beta, biased variance, fp32
+ * statistics, one rounding to out_dtype.  gamma/beta have out_dtype.
+ * mean/invvar (fp32 [n1]) and sum_out (x rounded to in_dtype, [n1,n2]) are
+ * optional (NULL to skip).  Supported (in,out): (f32,f32) (f32,f16) (f32,bf16)
+ * (f16,f16) (bf16,bf16), the pairs of csrc/type_shim.h:26-73. */
+int en_layernorm_fwd(void *out, float *mean, float *invvar, void *sum_out, const void *in, const void *residual,
+                     const void *gamma, const void *beta, int64_t n1, int64_t n2, float eps, int in_dtype,
+                     int out_dtype, en_stream_t stream);
+
+/* ---- attention contractions (torch.matmul in the reference callers) ----- */
+
+/* scores[b,h,i,j] = alpha * sum_d q[b,h,i,d] * k[b,h,j,d]
+ * (examples/bert/bert.py:110, examples/gpt/gpt.py:109).  q/k are addressed as
+ * base + b*stride_b + h*stride_h + s*stride_s + d (strides in elements), so
+ * the chunk views of the fused [B,H,S,3D] buffer are passed without a copy.
+ * scores is contiguous [B,H,Sq,Sk].  Only entries softmax will read are
+ * written: rows i < q_lens[b], columns j < visible(i) rounded up to the tile;
+ * everything else in scores is left untouched.  q_lens NULL as above.
+ * fp32 accumulation on MFMA; D a multiple of 8 (16-bit) / 4 (fp32), D <= 256. */
+int en_attn_qk(const void *q, const void *k, void *scores, const int32_t *k_lens, const int32_t *q_lens, int batch,
+               int head_num, int q_seq_len, int k_seq_len, int size_per_head, int64_t q_stride_b,
+               int64_t q_stride_h, int64_t q_stride_s, int64_t k_stride_b, int64_t k_stride_h, int64_t k_stride_s,
+               float alpha, int causal, int dtype, en_stream_t stream);
+
+/* ctx[b,h,i,:] = sum_j p[b,h,i,j] * v[b,h,j,:]  (examples/bert/bert.py:119,
+ * examples/gpt/gpt.py:125) over j < visible(i) only; p contiguous [B,H,Sq,Sk]
+ * as left by en_scale_mask_softmax, v strided like k above, ctx addressed with
+ * its own strides.  Rows i >= q_lens[b] of ctx are written as zero when
+ * zero_padding != 0 and left untouched otherwise. */
+int en_attn_pv(const void *p, const void *v, void *ctx, const int32_t *k_lens, const int32_t *q_lens, int batch,
+               int head_num, int q_seq_len, int k_seq_len, int size_per_head, int64_t v_stride_b,
+               int64_t v_stride_h, int64_t v_stride_s, int64_t c_stride_b, int64_t c_stride_h, int64_t c_stride_s,
+               int causal, int zero_padding, int dtype, en_stream_t stream);
+
+/* Single-query forms of the two contractions for cached decode (one new token
+ * per sequence against a ragged cache; the reference recomputes the whole
+ * square each step, energonai/model/attention.py:61-71,106-118).
+ * q [B,H,D] contiguous, k_cache/v_cache [B,H,Smax,D] with strides as above,
+ * scores/p [B,H,Smax] contiguous, ctx [B,H,D] contiguous.  Streaming kernels:
+ * bound by the K/V bytes read. */
+int en_decode_qk(const void *q, const void *k_cache, void *scores, const int32_t *kv_lens, int batch, int head_num,
+                 int k_seq_len, int size_per_head, int64_t k_stride_b, int64_t k_stride_h, int64_t k_stride_s,
+                 float alpha, int dtype, en_stream_t stream);
+int en_decode_pv(const void *p, const void *v_cache, void *ctx, const int32_t *kv_lens, int batch, int head_num,
+                 int k_seq_len, int size_per_head, int64_t v_stride_b, int64_t v_stride_h, int64_t v_stride_s,
+                 int dtype, en_stream_t stream);
+
+/* ---- measurement helper ------------------------------------------------- */
+
+/* Plain device-to-device copy of nbytes (multiple of 16, 16-byte aligned) with
+ * the same 128-bit access pattern the packing kernels use.  Used as the
+ * bandwidth yardstick and to calibrate hardware byte counters. */
+int en_copy_bytes(const void *src, void *dst, int64_t nbytes, en_stream_t stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* ENERGON_HIP_H */

@@ -1,0 +1,155 @@
+"""GPU parity: QK^T, PV and their single-query decode forms against the fp32/fp64 oracle.
+
+fp16: max-abs error <= 2e-3 on probabilities-weighted outputs (north-star
+tolerance); raw scores are compared relative to their fp16 rounding step.
+fp32: 1e-5 relative to the score scale.
+"""
+import pytest
+import torch
+
+from gpu_util import announce, max_abs, pad_bhsd, packed_randn
+from oracle import eager
+
+pytestmark = pytest.mark.gpu
+
+
+def _kernel():
+    from energonai_amd import kernel
+    return kernel
+
+
+def _visible_mask(B, H, Sq, Sk, k_lens, q_lens, causal):
+    m = torch.zeros(B, H, Sq, Sk, dtype=torch.bool)
+    for b in range(B):
+        for q in range(min(q_lens[b], Sq)):
+            n = eager.visible_keys(q, q_lens[b], k_lens[b], causal)
+            m[b, :, q, :n] = True
+    return m
+
+
+ATTN_CASES = [
+    # B, H, S, D, lens
+    (8, 12, 128, 64, [24, 127, 31, 65, 24, 127, 31, 65]),
+    (2, 3, 256, 128, [256, 129]),
+    (3, 2, 200, 64, [200, 0, 77]),       # S not a multiple of the tile, an empty sequence
+    (2, 2, 384, 32, [300, 1]),           # head dim below the tile's 64
+    (1, 2, 520, 80, [515]),              # OPT-2.7B head dim: padded to 128 inside the kernel
+    (9, 1, 130, 128, [130, 5, 64, 65, 127, 128, 129, 1, 33]),   # more units than XCDs, odd split
+]
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("causal", [True, False])
+@pytest.mark.parametrize("B,H,S,D,lens", ATTN_CASES)
+def test_attn_qk_pv_fused_layout(dtype, causal, B, H, S, D, lens):
+    """q/k/v are the strided chunk views of the fused [B,H,S,3D] buffer, as in the reference callers."""
+    k = _kernel()
+    announce("attn", dtype, causal, B, H, S, D, lens)
+    T = sum(lens)
+    qkv_packed = packed_randn(max(T, 1), H * 3 * D, dtype, 100 + S)[:T].reshape(T, H, 3 * D)
+    qkv = pad_bhsd(qkv_packed, lens, S, H, 3 * D)
+    q, kk, v = torch.chunk(qkv, 3, dim=-1)
+    lens_t = torch.tensor(lens, dtype=torch.int32).cuda()
+    qkv_g = qkv.cuda()
+    qg, kg, vg = torch.chunk(qkv_g, 3, dim=-1)
+    assert not qg.is_contiguous() or D * 3 == D
+
+    # ---- QK^T
+    sentinel = 777.0
+    out = torch.full((B, H, S, S), sentinel, dtype=dtype, device="cuda")
+    scores = k.attn_qk(qg, kg, lens_t, causal=causal, out=out).cpu()
+    want_scores = eager.attn_qk(q, kk, torch.float64)
+    vis = _visible_mask(B, H, S, S, lens, lens, causal)
+    step = {torch.float16: 2.0 ** -11, torch.bfloat16: 2.0 ** -8, torch.float32: 2.0 ** -16}[dtype]
+    if vis.any():
+        rel = ((scores.double() - want_scores).abs() / (want_scores.abs() + 1.0))[vis].max().item()
+        assert rel <= 1.5 * step, rel
+    # rows of padded queries are never written
+    rows_pad = torch.ones(B, H, S, dtype=torch.bool)
+    for b, n in enumerate(lens):
+        rows_pad[b, :, :n] = False
+    assert bool((scores[rows_pad] == sentinel).all())
+
+    # ---- PV on oracle probabilities (so the two kernels are checked independently)
+    probs64 = eager.scale_mask_softmax(B, S, H, want_scores, lens, scale=D ** -0.5, causal=causal,
+                                       acc_dtype=torch.float64, out_dtype=torch.float64)
+    probs = probs64.to(dtype)
+    for b, n in enumerate(lens):      # garbage in the rows of padded queries must not matter
+        probs[b, :, n:, :] = float("nan")
+    ctx_out = torch.full((B, H, S, D), sentinel, dtype=dtype, device="cuda")
+    ctx = k.attn_pv(probs.cuda(), vg, lens_t, causal=causal, out=ctx_out).cpu()
+    want_ctx = eager.attn_pv(torch.nan_to_num(probs, nan=0.0), v, torch.float64)
+    rows_ok = ~rows_pad
+    tol = {torch.float16: 2e-3, torch.bfloat16: 1.6e-2, torch.float32: 1e-5}[dtype]
+    if rows_ok.any():
+        err = max_abs(ctx[rows_ok], want_ctx[rows_ok])
+        assert err <= tol * max(1.0, float(want_ctx[rows_ok].abs().max())), err
+    assert bool((ctx[rows_pad] == sentinel).all())
+    # zero_padding writes zeros there instead
+    ctx0 = k.attn_pv(probs.cuda(), vg, lens_t, causal=causal, zero_padding=True).cpu()
+    assert bool((ctx0[rows_pad] == 0).all())
+    if rows_ok.any():
+        assert torch.equal(ctx0[rows_ok], ctx[rows_ok])
+
+
+def test_attn_nan_in_padding_of_v_is_ignored():
+    """Cache rows past the valid length may hold anything (torch.empty caches)."""
+    k = _kernel()
+    B, H, S, D = 2, 2, 192, 64
+    lens = [100, 192]
+    announce("attn nan padding")
+    g = torch.Generator().manual_seed(4)
+    q = torch.randn(B, H, S, D, generator=g).half()
+    kk = torch.randn(B, H, S, D, generator=g).half()
+    v = torch.randn(B, H, S, D, generator=g).half()
+    for b, n in enumerate(lens):
+        kk[b, :, n:] = float("nan")
+        v[b, :, n:] = float("nan")
+    lens_t = torch.tensor(lens, dtype=torch.int32).cuda()
+    scores = k.attn_qk(q.cuda(), kk.cuda(), lens_t, causal=True)
+    probs = k.scale_mask_softmax(B, S, H, scores, lens_t, scale=0.125)
+    ctx = k.attn_pv(probs, v.cuda(), lens_t, causal=True).cpu()
+    for b, n in enumerate(lens):
+        assert torch.isfinite(ctx[b, :, :n]).all()
+
+
+DECODE_CASES = [
+    # B, H, Smax, D, kv lens
+    (5, 4, 640, 128, [640, 1, 333, 64, 65]),
+    (3, 2, 100, 64, [100, 17, 2]),
+    (2, 3, 77, 32, [77, 40]),
+    (4, 72, 2048, 128, [2048, 3, 1024, 1989]),
+]
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("B,H,S,D,kv", DECODE_CASES)
+def test_decode_qk_pv(dtype, B, H, S, D, kv):
+    k = _kernel()
+    announce("decode", dtype, B, H, S, D, kv)
+    g = torch.Generator().manual_seed(S + D)
+    q = torch.randn(B, H, 1, D, generator=g).to(dtype)
+    kc = torch.randn(B, H, S, D, generator=g).to(dtype)
+    vc = torch.randn(B, H, S, D, generator=g).to(dtype)
+    for b, n in enumerate(kv):           # unused cache rows hold garbage
+        kc[b, :, n:] = float("nan")
+        vc[b, :, n:] = float("nan")
+    kv_t = torch.tensor(kv, dtype=torch.int32).cuda()
+    scale = D ** -0.5
+    want_scores, want_probs, want_ctx = eager.decode_attention(
+        q, torch.nan_to_num(kc, nan=0.0), torch.nan_to_num(vc, nan=0.0), kv, scale, acc_dtype=torch.float64)
+    scores = k.decode_qk(q.cuda(), kc.cuda(), kv_t)
+    assert scores.shape == (B, H, 1, S)
+    vis = torch.zeros(B, H, 1, S, dtype=torch.bool)
+    for b, n in enumerate(kv):
+        vis[b, :, :, :n] = True
+    step = {torch.float16: 2.0 ** -11, torch.bfloat16: 2.0 ** -8, torch.float32: 2.0 ** -16}[dtype]
+    rel = ((scores.cpu().double() - want_scores).abs() / (want_scores.abs() + 1.0))[vis].max().item()
+    assert rel <= 1.5 * step, rel
+    probs = k.scale_mask_softmax(B, 1, H, scores, kv_t, scale=scale, k_seq_len=S,
+                                 q_len_list=torch.ones(B, dtype=torch.int32).cuda())
+    tol = {torch.float16: 2e-3, torch.bfloat16: 1.6e-2, torch.float32: 1e-5}[dtype]
+    assert max_abs(probs.cpu(), want_probs) <= tol
+    ctx = k.decode_pv(probs, vc.cuda(), kv_t).cpu()
+    assert ctx.shape == (B, H, 1, D)
+    assert max_abs(ctx, want_ctx) <= tol * max(1.0, float(want_ctx.abs().max()))

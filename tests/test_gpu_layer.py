@@ -1,0 +1,163 @@
+"""GPU parity of the whole per-layer path on the benchmark workloads.
+
+c1 (fp32) is compared with the float64 oracle at 1e-5; the fp16 workloads are
+compared at the north-star tolerance (max-abs <= 2e-3 against the fp32 oracle
+on the attention context, and the LayerNorm output within one fp16 rounding
+step of it).  c2 runs at full size here; c3/c4 run at full size through
+size-independent properties (bit-exact pack round trips, rows of probabilities
+summing to one, LayerNorm row statistics) plus an oracle comparison on a
+subset of sequences, so the CPU side stays within seconds.
+"""
+import pytest
+import torch
+
+from gpu_util import announce, max_abs
+from oracle import eager
+
+pytestmark = pytest.mark.gpu
+
+
+def _mods():
+    from energonai_amd import layer, workloads
+    return layer, workloads
+
+
+def _run_and_compare(w, inp, acc_dtype, tol_ctx, tol_y):
+    layer, _ = _mods()
+    dev = {k: (v.cuda() if isinstance(v, torch.Tensor) else v) for k, v in inp.items()}
+    got = layer.padding_removal_layer(dev["hidden_padded"], dev["qkv_packed"], dev["lens"], w.heads, w.head_dim,
+                                      dev["gamma"], dev["beta"], 1e-5, w.scale, w.causal, w.left_padded,
+                                      dense_out=dev["dense_out"], keep=True)
+    want = eager.layer_unpadded(inp["hidden_padded"], inp["qkv_packed"], inp["lens_list"], w.heads, w.head_dim,
+                                inp["gamma"], inp["beta"], 1e-5, w.scale, w.causal, w.left_padded,
+                                dense_out=inp["dense_out"], acc_dtype=acc_dtype)
+    assert torch.equal(got["x"].cpu(), want["x"].to(w.dtype)), "depad must be bit-exact"
+    assert torch.equal(got["qkv"].cpu(), want["qkv"].to(w.dtype)), "transpose_pad must be bit-exact"
+    err_ctx = max_abs(got["ctx_packed"].cpu(), want["ctx_packed"])
+    assert err_ctx <= tol_ctx, err_ctx
+    err_y = max_abs(got["y"].cpu(), want["y"])
+    assert err_y <= tol_y, err_y
+    return got, want
+
+
+def test_layer_c1_fp32_full():
+    _, wl = _mods()
+    w = wl.BY_NAME["c1"]
+    announce("layer c1")
+    inp = wl.make_inputs(w)
+    assert inp["total"] == 698
+    _run_and_compare(w, inp, torch.float64, 1e-5, 2e-5)
+
+
+def test_layer_c1_matches_padded_layer():
+    """The unpadded path equals the ordinary padded layer on valid tokens (examples/bert/bert.py:100-126)."""
+    layer, wl = _mods()
+    w = wl.BY_NAME["c1"]
+    announce("layer c1 vs padded")
+    inp = wl.make_inputs(w)
+    got = layer.padding_removal_layer(inp["hidden_padded"].cuda(), inp["qkv_packed"].cuda(), inp["lens"].cuda(),
+                                      w.heads, w.head_dim, inp["gamma"].cuda(), inp["beta"].cuda(), 1e-5, w.scale,
+                                      w.causal, w.left_padded).cpu()
+    lens = inp["lens_list"]
+    qkv_padded = torch.zeros(w.batch, w.seq, w.heads, 3 * w.head_dim)
+    t = 0
+    for b, n in enumerate(lens):
+        qkv_padded[b, :n] = inp["qkv_packed"][0, t:t + n]
+        t += n
+    y_pad = eager.layer_padded(inp["hidden_padded"], qkv_padded, lens, w.heads, w.head_dim, inp["gamma"],
+                               inp["beta"], 1e-5, w.scale, w.causal, acc_dtype=torch.float64)
+    want = eager.depad(y_pad, w.batch, lens)
+    assert max_abs(got, want) <= 2e-5
+
+
+def test_layer_c2_fp16_full():
+    _, wl = _mods()
+    w = wl.BY_NAME["c2"]
+    announce("layer c2")
+    inp = wl.make_inputs(w)
+    assert inp["total"] == 8538
+    # LayerNorm output |y| reaches ~5: one fp16 rounding there is 3.9e-3/2, on top of the 2e-3 budget of its input
+    _run_and_compare(w, inp, torch.float32, 2e-3, 6e-3)
+
+
+@pytest.mark.parametrize("name,total", [("c3", 9244), ("c4", 20142)])
+def test_layer_large_fp16_properties(name, total):
+    layer, wl = _mods()
+    w = wl.BY_NAME[name]
+    announce("layer", name)
+    inp = wl.make_inputs(w)
+    assert inp["total"] == total
+    from energonai_amd import kernel as k
+    lens_l = inp["lens_list"]
+    lens_g = inp["lens"].cuda()
+    hp = inp["hidden_padded"].cuda()
+    qkvp = inp["qkv_packed"].cuda()
+    got = layer.padding_removal_layer(hp, qkvp, lens_g, w.heads, w.head_dim, inp["gamma"].cuda(), inp["beta"].cuda(),
+                                      1e-5, w.scale, w.causal, w.left_padded,
+                                      dense_out=None if inp["dense_out"] is None else inp["dense_out"].cuda(),
+                                      keep=True)
+    T, B, S, H, D = total, w.batch, w.seq, w.heads, w.head_dim
+    # pack round trips at full size, bit-exact
+    assert torch.equal(got["x"].cpu(), eager.depad(inp["hidden_padded"], B, lens_l, left_padded=w.left_padded))
+    back = k.transpose_depad(got["qkv"], B, T, S, lens_g, H, 3 * D)
+    assert torch.equal(back, qkvp)
+    # padding of the padded tensor is zero
+    for b in (0, B - 1):
+        assert bool((got["qkv"][b, :, lens_l[b]:, :] == 0).all())
+    # probabilities: valid rows sum to one, nothing above the diagonal
+    probs = got["probs"]
+    for b in (0, B // 2, B - 1):
+        n = lens_l[b]
+        sums = probs[b, :, :n].float().sum(-1)
+        assert float((sums - 1).abs().max()) < 5e-3
+        assert float(probs[b, :, :n].float().triu(1).abs().max()) == 0.0
+    # LayerNorm: rows of (y - beta) / gamma have zero mean and unit variance
+    y = got["y"].float()[0]
+    z = (y - inp["beta"].cuda().float()) / inp["gamma"].cuda().float()
+    assert float(z.mean(-1).abs().max()) < 2e-3
+    assert float((z.var(-1, unbiased=False) - 1).abs().max()) < 5e-3
+    # oracle on the two shortest sequences (keeps the CPU side small)
+    order = sorted(range(B), key=lambda b: lens_l[b])[:2]
+    cu = [0]
+    for n in lens_l:
+        cu.append(cu[-1] + n)
+    for b in order:
+        n = lens_l[b]
+        sl = slice(cu[b], cu[b] + n)
+        sub_qkv = inp["qkv_packed"][:, sl]
+        sub_hidden = inp["hidden_padded"][b:b + 1]
+        sub_dense = None if inp["dense_out"] is None else inp["dense_out"][:, sl]
+        want = eager.layer_unpadded(sub_hidden, sub_qkv, [n], H, D, inp["gamma"], inp["beta"], 1e-5, w.scale,
+                                    w.causal, w.left_padded, dense_out=sub_dense, acc_dtype=torch.float32)
+        assert max_abs(got["ctx_packed"][0, sl].cpu(), want["ctx_packed"][0]) <= 2e-3
+        assert max_abs(got["y"][0, sl].cpu(), want["y"][0]) <= 6e-3
+
+
+def test_decode_layer_c5_reduced_and_full():
+    layer, wl = _mods()
+    w = wl.BY_NAME["c5"]
+    announce("layer c5")
+    lens = wl.make_lens(w)
+    assert int(lens.sum()) == 70929
+    # full-size run: caches drawn on the device, oracle on a subset of sequences
+    inp = wl.make_decode_inputs(w, device="cuda", cache_on_device=True)
+    got = layer.decode_layer(inp["q"], inp["k_cache"], inp["v_cache"], inp["lens"].cuda(), inp["residual"],
+                             inp["gamma"], inp["beta"], 1e-5, w.scale, dense_out=inp["dense_out"], keep=True)
+    lens_l = inp["lens_list"]
+    pick = sorted(range(w.batch), key=lambda b: lens_l[b])
+    pick = [pick[0], pick[len(pick) // 2], pick[-1]]
+    for b in pick:
+        _, probs, ctx = eager.decode_attention(inp["q"][b:b + 1].cpu(), inp["k_cache"][b:b + 1].cpu(),
+                                               inp["v_cache"][b:b + 1].cpu(), [lens_l[b]], w.scale)
+        assert max_abs(got["ctx"][b:b + 1].cpu(), ctx) <= 2e-3
+        assert max_abs(got["scores_probs"][b:b + 1].cpu(), probs) <= 2e-3
+    want_y, _, _, _ = eager.layer_norm(inp["dense_out"].cpu(), inp["gamma"].cpu(), inp["beta"].cpu(), 1e-5,
+                                       residual=inp["residual"].cpu(), out_dtype=torch.float32)
+    assert max_abs(got["y"].cpu(), want_y) <= 6e-3
+    # the attention output feeds the residual directly when no dense output is given
+    got2 = layer.decode_layer(inp["q"], inp["k_cache"], inp["v_cache"], inp["lens"].cuda(), inp["residual"],
+                              inp["gamma"], inp["beta"], 1e-5, w.scale, keep=True)
+    want2, _, _, _ = eager.layer_norm(got2["ctx_packed"].reshape(1, w.batch, -1).cpu(), inp["gamma"].cpu(),
+                                      inp["beta"].cpu(), 1e-5, residual=inp["residual"].cpu(),
+                                      out_dtype=torch.float32)
+    assert max_abs(got2["y"].cpu(), want2) <= 6e-3
