@@ -1,0 +1,366 @@
+#!/usr/bin/env python3
+"""Benchmark of the per-layer padding-removal hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c2] [--no-cpu] [--no-extra]
+
+A step is one pass of
+    depad -> transpose_pad -> QK^T -> scale_mask_softmax -> PV -> transpose_depad -> residual + LayerNorm
+over one synthetic batch whose inputs are already resident in HBM.  The headline
+value is tokens/s of that pass on the workload named by --workload (default c2,
+the OPT-125M layer); the other workloads, the per-kernel bandwidths, the
+PyTorch-ROCm eager pipeline and the CPU oracle are reported beside it in the
+same JSON line.
+
+The line also carries
+  roofline      achieved vs peak for the kernel that takes the largest share of the step,
+                from algorithmic bytes (or FLOPs) per launch and the kernel's launch-to-launch
+                time measured with events on the launch stream;
+  cpu_baseline  the CPU oracle (a port of the reference's eager path) timed on
+                this box's host cores on a bounded sample of the same workload.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0          # MI355X HBM3E
+MFMA_PEAK_TFLOPS = {"f16": 2500.0, "bf16": 2500.0, "f32": 157.3}
+DTYPE_NAME = {"torch.float16": "f16", "torch.bfloat16": "bf16", "torch.float32": "f32"}
+
+
+def _event_time_ms(fn, iters, torch):
+    """Average time of fn() over iters back-to-back launches, events on the current stream."""
+    start = torch.cuda.Event(enable_timing=True)
+    stop = torch.cuda.Event(enable_timing=True)
+    start.record()
+    for _ in range(iters):
+        fn()
+    stop.record()
+    stop.synchronize()
+    return start.elapsed_time(stop) / iters
+
+
+def _median_step_ms(fn, iters, torch):
+    """Median of per-step event timings (used for the eager baseline, as its definition asks)."""
+    times = []
+    for _ in range(iters):
+        s = torch.cuda.Event(enable_timing=True)
+        e = torch.cuda.Event(enable_timing=True)
+        s.record()
+        fn()
+        e.record()
+        e.synchronize()
+        times.append(s.elapsed_time(e))
+    times.sort()
+    return times[len(times) // 2]
+
+
+# ---------------------------------------------------------------------------
+# PyTorch-ROCm eager pipeline: the same seven steps with stock torch ops
+# ---------------------------------------------------------------------------
+def eager_prefill_step(torch, w, d):
+    import torch.nn.functional as F
+    B, S, H, D = w.batch, w.seq, w.heads, w.head_dim
+    lens = d["lens_list"]
+    hp = d["hidden_padded"]
+    # depad: the reference's cat loop (energonai/kernel/cuda_native/transpose_pad.py:30-37)
+    if w.left_padded:
+        x = torch.cat([hp[i:i + 1, S - lens[i]:S, :] for i in range(B)], dim=1)
+    else:
+        x = torch.cat([hp[i:i + 1, 0:lens[i], :] for i in range(B)], dim=1)
+    # pad: zeros + index copy + permute
+    qkv = torch.zeros(B * S, H, 3 * D, dtype=hp.dtype, device=hp.device)
+    qkv.index_copy_(0, d["valid_rows"], d["qkv_packed"][0])
+    qkv = qkv.view(B, S, H, 3 * D).permute(0, 2, 1, 3).contiguous()
+    q, k, v = torch.chunk(qkv, 3, dim=-1)
+    s = torch.matmul(q, k.transpose(-1, -2)) * w.scale
+    if w.causal:
+        s = torch.where(d["tri"], s, d["neg"])
+    s = s + d["key_mask"]
+    p = torch.softmax(s, -1, dtype=torch.float).to(hp.dtype)
+    ctx = torch.matmul(p, v)
+    ctx = ctx.permute(0, 2, 1, 3).reshape(B * S, H * D).index_select(0, d["valid_rows"]).unsqueeze(0)
+    attn_out = ctx if d["dense_out"] is None else d["dense_out"]
+    return F.layer_norm(attn_out + x, (w.hidden,), d["gamma"], d["beta"], 1e-5)
+
+
+def eager_decode_step(torch, w, d):
+    import torch.nn.functional as F
+    s = torch.matmul(d["q"], d["k_cache"].transpose(-1, -2)) * w.scale
+    s = s + d["key_mask"]
+    p = torch.softmax(s, -1, dtype=torch.float).to(d["q"].dtype)
+    ctx = torch.matmul(p, d["v_cache_clean"])
+    ctx = ctx.permute(0, 2, 1, 3).reshape(1, w.batch, w.heads * w.head_dim)
+    return F.layer_norm(d["dense_out"] + d["residual"], (w.hidden,), d["gamma"], d["beta"], 1e-5), ctx
+
+
+def add_eager_aux(torch, w, d, device):
+    lens = d["lens_list"]
+    B, S = w.batch, w.seq
+    pos = torch.arange(S, device=device)
+    lens_t = torch.tensor(lens, device=device)
+    key_ok = pos.view(1, S) < lens_t.view(B, 1)
+    d["key_mask"] = ((~key_ok).to(w.dtype) * -10000.0).view(B, 1, 1, S)
+    if not w.decode:
+        rows = torch.cat([torch.arange(n, device=device) + b * S for b, n in enumerate(lens)])
+        d["valid_rows"] = rows
+        d["tri"] = torch.tril(torch.ones(S, S, dtype=torch.bool, device=device)).view(1, 1, S, S)
+        d["neg"] = torch.tensor(-1e4, dtype=w.dtype, device=device)
+    else:
+        d["v_cache_clean"] = d["v_cache"]
+
+
+# ---------------------------------------------------------------------------
+# one workload on the GPU
+# ---------------------------------------------------------------------------
+def run_workload(torch, w, steps, warmup, want_eager=True, want_kernels=True):
+    from energonai_amd import kernel as K
+    from energonai_amd import layer, workloads
+    from energonai_amd.seqinfo import seq_info
+    dev = torch.device("cuda", 0)
+    res = {"title": w.title, "dtype": DTYPE_NAME[str(w.dtype)]}
+    if w.decode:
+        d = workloads.make_decode_inputs(w, device=dev, cache_on_device=True)
+        info = seq_info(d["lens"], w.batch, dev)
+        tokens = w.batch
+
+        def step():
+            return layer.decode_layer(d["q"], d["k_cache"], d["v_cache"], info, d["residual"], d["gamma"], d["beta"],
+                                      workloads.EPS, w.scale, dense_out=d["dense_out"])
+    else:
+        d = workloads.make_inputs(w, device=dev)
+        info = seq_info(d["lens"], w.batch, dev)
+        tokens = d["total"]
+
+        def step():
+            return layer.padding_removal_layer(d["hidden_padded"], d["qkv_packed"], info, w.heads, w.head_dim,
+                                               d["gamma"], d["beta"], workloads.EPS, w.scale, w.causal,
+                                               w.left_padded, dense_out=d["dense_out"], sum_seq=tokens)
+    res["tokens"] = tokens
+    for _ in range(warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        step()
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3 / steps
+    res["ms_per_step"] = wall_ms
+    res["tokens_per_s"] = tokens / (wall_ms * 1e-3)
+
+    # the same step replayed from a HIP graph (launch overhead removed); reported, never the headline
+    try:
+        g = torch.cuda.CUDAGraph()
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            step()
+            with torch.cuda.graph(g, stream=side):
+                step()
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        for _ in range(3):
+            g.replay()
+        res["graph_ms_per_step"] = _event_time_ms(g.replay, steps, torch)
+        del g
+    except Exception as exc:  # graph capture is a convenience measurement only
+        res["graph_ms_per_step"] = None
+        res["graph_error"] = str(exc)[:200]
+    torch.cuda.synchronize()
+
+    if want_kernels:
+        res["kernels"] = kernel_table(torch, K, layer, workloads, w, d, info, steps)
+    if want_eager:
+        add_eager_aux(torch, w, d, dev)
+        fn = (lambda: eager_decode_step(torch, w, d)) if w.decode else (lambda: eager_prefill_step(torch, w, d))
+        try:
+            for _ in range(min(warmup, 10)):
+                fn()
+            torch.cuda.synchronize()
+            ms = _median_step_ms(fn, max(5, min(steps, 50)), torch)
+            res["eager_gpu_ms_per_step"] = ms
+            res["speedup_vs_eager_gpu"] = ms / wall_ms
+        except Exception as exc:
+            res["eager_gpu_ms_per_step"] = None
+            res["eager_error"] = str(exc)[:200]
+    del d
+    torch.cuda.empty_cache()
+    return res
+
+
+def kernel_table(torch, K, layer, workloads, w, d, info, steps):
+    """Launch-to-launch time of every kernel on its real operands -> GB/s, TFLOP/s, fraction of peak."""
+    dt = DTYPE_NAME[str(w.dtype)]
+    alg = workloads.algorithmic_bytes(w, d["lens_list"])
+    flops = workloads.algorithmic_flops(w, d["lens_list"])
+    H, D, S, B = w.heads, w.head_dim, w.seq, w.batch
+    fns = {}
+    if w.decode:
+        ones = layer._ones_info(B, d["q"].device)
+        keep = layer.decode_layer(d["q"], d["k_cache"], d["v_cache"], info, d["residual"], d["gamma"], d["beta"],
+                                  workloads.EPS, w.scale, dense_out=d["dense_out"], keep=True)
+        scores = torch.empty((B, H, 1, S), dtype=w.dtype, device=d["q"].device)
+        ctx = torch.empty((B, H, 1, D), dtype=w.dtype, device=d["q"].device)
+        probs = keep["scores_probs"]
+        fns["decode_qk"] = lambda: K.decode_qk(d["q"], d["k_cache"], info, out=scores)
+        fns["scale_mask_softmax"] = lambda: K.scale_mask_softmax(B, 1, H, probs, info, scale=w.scale, k_seq_len=S,
+                                                                 q_len_list=ones)
+        fns["decode_pv"] = lambda: K.decode_pv(probs, d["v_cache"], info, out=ctx)
+        fns["layernorm_residual"] = lambda: K.layer_norm_forward(d["dense_out"], d["gamma"], d["beta"], (w.hidden,),
+                                                                 workloads.EPS, residual=d["residual"])
+    else:
+        T = d["total"]
+        keep = layer.padding_removal_layer(d["hidden_padded"], d["qkv_packed"], info, H, D, d["gamma"], d["beta"],
+                                           workloads.EPS, w.scale, w.causal, w.left_padded, dense_out=d["dense_out"],
+                                           sum_seq=T, keep=True)
+        q, k, v = torch.chunk(keep["qkv"], 3, dim=-1)
+        scores = keep["probs"]
+        ctx = keep["ctx"]
+        attn_out = keep["ctx_packed"].view(1, T, H * D) if d["dense_out"] is None else d["dense_out"]
+        fns["depad"] = lambda: K.depad(d["hidden_padded"], B, info, left_padded=w.left_padded, sum_seq=T)
+        fns["transpose_pad"] = lambda: K.transpose_pad(d["qkv_packed"], B, S, info, H, 3 * D)
+        fns["attn_qk"] = lambda: K.attn_qk(q, k, info, causal=w.causal, out=scores)
+        fns["scale_mask_softmax"] = lambda: K.scale_mask_softmax(B, S, H, scores, info, scale=w.scale,
+                                                                 causal=w.causal)
+        fns["attn_pv"] = lambda: K.attn_pv(scores, v, info, causal=w.causal, out=ctx)
+        fns["transpose_depad"] = lambda: K.transpose_depad(ctx, B, T, S, info, H, D)
+        fns["layernorm_residual"] = lambda: K.layer_norm_forward(attn_out, d["gamma"], d["beta"], (w.hidden,),
+                                                                 workloads.EPS, residual=keep["x"])
+    table = {}
+    for name, fn in fns.items():
+        for _ in range(3):
+            fn()
+        torch.cuda.synchronize()
+        ms = _event_time_ms(fn, steps, torch)
+        row = {"us": ms * 1e3, "alg_MB": alg[name] / 1e6, "GBps": alg[name] / (ms * 1e-3) / 1e9}
+        row["hbm_frac"] = row["GBps"] / HBM_PEAK_GBS
+        if name in ("attn_qk", "attn_pv", "decode_qk", "decode_pv"):
+            row["TFLOPs"] = flops / (ms * 1e-3) / 1e12
+            row["mfma_frac"] = row["TFLOPs"] / MFMA_PEAK_TFLOPS[dt]
+        table[name] = row
+    return table
+
+
+# ---------------------------------------------------------------------------
+# CPU baseline: the oracle on this box's host cores, bounded sample
+# ---------------------------------------------------------------------------
+def cpu_baseline(torch, w, budget_s=12.0):
+    from energonai_amd import workloads
+    from oracle import eager
+    cores = min(os.cpu_count() or 1, 16)
+    torch.set_num_threads(cores)
+    if w.decode:
+        lens = workloads.make_lens(w)[:8]
+        sub = workloads.Workload(w.index, w.name, w.title, torch.float32, 8, w.seq, w.heads, w.head_dim, w.hidden,
+                                 w.len_lo, w.len_hi, w.causal, w.left_padded, decode=True)
+        d = workloads.make_decode_inputs(sub, dtype=torch.float32, lens=lens)
+        tokens = 8
+        sample = "first 8 of the 64 sequences, fp32 on the CPU"
+
+        def step():
+            eager.decode_attention(d["q"], d["k_cache"], d["v_cache"], d["lens_list"], w.scale)
+            eager.layer_norm(d["dense_out"], d["gamma"], d["beta"], workloads.EPS, residual=d["residual"])
+    else:
+        nb = w.batch if w.name in ("c1", "c2") else 2
+        lens = workloads.make_lens(w)[:nb]
+        sub = workloads.Workload(w.index, w.name, w.title, torch.float32, nb, w.seq, w.heads, w.head_dim, w.hidden,
+                                 w.len_lo, w.len_hi, w.causal, w.left_padded)
+        d = workloads.make_inputs(sub, dtype=torch.float32, lens=lens)
+        tokens = d["total"]
+        sample = (f"{'all' if nb == w.batch else 'first ' + str(nb) + ' of the'} {w.batch} sequences "
+                  f"({tokens} tokens), fp32 on the CPU")
+
+        def step():
+            eager.layer_unpadded(d["hidden_padded"], d["qkv_packed"], d["lens_list"], w.heads, w.head_dim, d["gamma"],
+                                 d["beta"], workloads.EPS, w.scale, w.causal, w.left_padded,
+                                 dense_out=d["dense_out"])
+    step()  # warm-up
+    times = []
+    t_begin = time.perf_counter()
+    while len(times) < 3 or (time.perf_counter() - t_begin < budget_s and len(times) < 50):
+        t0 = time.perf_counter()
+        step()
+        times.append(time.perf_counter() - t0)
+        if time.perf_counter() - t_begin > 3 * budget_s:
+            break
+    times.sort()
+    med = times[len(times) // 2]
+    return {"value": tokens / med, "unit": "tokens/s", "cores": cores, "kind": "port",
+            "sample": f"{sample}; median of {len(times)} passes, {med * 1e3:.1f} ms each; "
+                      f"oracle.eager.layer_unpadded (torch-eager restatement of the reference path)"}
+
+
+def main(argv=None) -> int:
+    ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--workload", default="c2", choices=["c1", "c2", "c3", "c4", "c5"])
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-extra", action="store_true", help="only the headline workload, no eager / other workloads")
+    ns = ap.parse_args(argv)
+    if ns.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py: this build measures one GPU's share of the path; --gpus must be 1 "
+              "(the path shards by head / by sequence with no exchange step, nothing here uses a second GPU)",
+              file=sys.stderr)
+        return 2
+
+    import torch
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU", file=sys.stderr)
+        return 2
+    torch.cuda.set_device(0)
+    from energonai_amd import workloads
+
+    w = workloads.BY_NAME[ns.workload]
+    torch.cuda.synchronize()
+    head = run_workload(torch, w, ns.steps, ns.warmup, want_eager=not ns.no_extra, want_kernels=True)
+    torch.cuda.synchronize()
+
+    # roofline of the kernel that takes the largest share of the step
+    kt = head["kernels"]
+    dom = max(kt, key=lambda n: kt[n]["us"])
+    row = kt[dom]
+    roofline = {"kernel": dom, "bound": "hbm", "achieved": row["GBps"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                "frac": row["GBps"] / HBM_PEAK_GBS, "traffic": None, "us_per_launch": row["us"],
+                "alg_bytes_per_launch": row["alg_MB"] * 1e6}
+
+    out = {
+        "metric": "per_layer_tokens_per_s", "value": head["tokens_per_s"], "unit": "tokens/s", "n_gpus": 1,
+        "steps": ns.steps, "warmup": ns.warmup, "ms_per_step": head["ms_per_step"], "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": head["dtype"], "data": "synthetic",
+        "config": {"workload": f"{w.name}: {w.title}; batch {w.batch}, bucket {w.seq}, {w.heads}x{w.head_dim} heads, "
+                               f"LayerNorm width {w.hidden}, {head['tokens']} valid tokens"},
+        "roofline": roofline,
+        "graph_ms_per_step": head.get("graph_ms_per_step"),
+        "eager_gpu_ms_per_step": head.get("eager_gpu_ms_per_step"),
+        "speedup_vs_eager_gpu": head.get("speedup_vs_eager_gpu"),
+        "kernels": kt,
+    }
+    if not ns.no_extra:
+        others = {}
+        for ow in workloads.WORKLOADS:
+            if ow.name == w.name:
+                continue
+            try:
+                others[ow.name] = run_workload(torch, ow, max(5, ns.steps // 2), max(2, ns.warmup // 2))
+            except Exception as exc:
+                others[ow.name] = {"error": str(exc)[:300]}
+        out["workloads"] = others
+    if not ns.no_cpu:
+        out["cpu_baseline"] = cpu_baseline(torch, w)
+    else:
+        out["cpu_baseline"] = None
+    print(json.dumps(out))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())
