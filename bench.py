@@ -229,6 +229,9 @@ def kernel_table(torch, K, layer, workloads, w, d, info, steps):
         fns["attn_qk"] = lambda: K.attn_qk(q, k, info, causal=w.causal, out=scores)
         fns["scale_mask_softmax"] = lambda: K.scale_mask_softmax(B, S, H, scores, info, scale=w.scale,
                                                                  causal=w.causal)
+        fns["scale_mask_softmax_tiled"] = lambda: K.scale_mask_softmax(B, S, H, scores, info, scale=w.scale,
+                                                                       causal=w.causal,
+                                                                       tail_rows=layer.PV_QUERY_TILE)
         fns["attn_pv"] = lambda: K.attn_pv(scores, v, info, causal=w.causal, out=ctx)
         fns["transpose_depad"] = lambda: K.transpose_depad(ctx, B, T, S, info, H, D)
         fns["layernorm_residual"] = lambda: K.layer_norm_forward(attn_out, d["gamma"], d["beta"], (w.hidden,),
@@ -326,7 +329,8 @@ def main(argv=None) -> int:
 
     # roofline of the kernel that takes the largest share of the step
     kt = head["kernels"]
-    dom = max(kt, key=lambda n: kt[n]["us"])
+    in_step = [n for n in kt if n != "scale_mask_softmax" or "scale_mask_softmax_tiled" not in kt]
+    dom = max(in_step, key=lambda n: kt[n]["us"])
     row = kt[dom]
     roofline = {"kernel": dom, "bound": "hbm", "achieved": row["GBps"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
                 "frac": row["GBps"] / HBM_PEAK_GBS, "traffic": None, "us_per_launch": row["us"],

@@ -35,7 +35,7 @@ SIGNATURES = {
     "en_ft_transpose_rebuild": (c_int, [c_void_p] * 6 + [c_int] * 5 + [c_void_p, c_int, c_void_p]),
     "en_ft_transpose_remove": (c_int, [c_void_p, c_void_p] + [c_int] * 5 + [c_void_p, c_int, c_void_p]),
     "en_scale_mask_softmax": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_float, c_int, c_int,
-                                      c_void_p]),
+                                      c_int, c_void_p]),
     "en_layernorm_fwd": (c_int, [c_void_p] * 8 + [c_int64, c_int64, c_float, c_int, c_int, c_void_p]),
     "en_attn_qk": (c_int, [c_void_p] * 5 + [c_int] * 5 + [c_int64] * 6 + [c_float, c_int, c_int, c_void_p]),
     "en_attn_pv": (c_int, [c_void_p] * 5 + [c_int] * 5 + [c_int64] * 6 + [c_int, c_int, c_int, c_void_p]),
@@ -99,4 +99,36 @@ def ptr(t) -> int:
 
 def stream_of(t: torch.Tensor) -> int:
     """Raw handle of torch's current stream on t's device (kernels launch there, never on the default stream)."""
-    return torch.cuda.current_stream(t.device).cuda_stream
+    return torch._C._cuda_getCurrentRawStream(t.device.index)
+
+
+class _NoGuard:
+    __slots__ = ()
+
+    def __enter__(self):
+        return None
+
+    def __exit__(self, *exc):
+        return False
+
+
+_NO_GUARD = _NoGuard()
+
+
+def device_guard(t: torch.Tensor):
+    """Context that makes t's device current for the launch; free when it already is."""
+    if t.device.index == torch.cuda.current_device():
+        return _NO_GUARD
+    return torch.cuda.device(t.device)
+
+
+class _Fns:
+    """Attribute access to the bound entry points: ``fn.en_depad(...)``; loads the library on first use."""
+
+    def __getattr__(self, name):
+        f = getattr(load(), name)
+        setattr(self, name, f)
+        return f
+
+
+fn = _Fns()

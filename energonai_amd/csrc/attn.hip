@@ -325,7 +325,7 @@ __global__ __launch_bounds__(kBlock) void attn_pv_kernel(AttnArgs a) {
         } else {
           Pack<T, EPV> pk;
 #pragma unroll
-          for (int e = 0; e < EPV; ++e) pk.v[e] = (k + e < a.Sk) ? gp[e] : E::from_float(0.f);
+          for (int e = 0; e < EPV; ++e) pk.v[e] = (k + e < nk) ? gp[e] : E::from_float(0.f);
           preg[i] = __builtin_bit_cast(uint4, pk);
         }
       } else {

@@ -68,6 +68,32 @@ __device__ __forceinline__ Pack<T, N> load_pack(const T *p) { return *reinterpre
 template <typename T, int N>
 __device__ __forceinline__ void store_pack(T *p, const Pack<T, N> &x) { *reinterpret_cast<Pack<T, N> *>(p) = x; }
 
+// Outputs at least this large cannot stay in the 256 MB memory-side cache for the
+// consumer kernel anyway, so they are written with non-temporal stores (measured:
+// +10..25 % on such tensors, -5 % when applied to small, cache-resident ones).
+constexpr int64_t kStreamStoreBytes = 96ll << 20;
+
+// 128-bit global accesses, optionally non-temporal (streamed once: do not keep in cache).
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+
+template <bool NT>
+__device__ __forceinline__ uint4 load16(const void *p) {
+  if (NT) {
+    const u32x4 v = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(p));
+    return make_uint4(v.x, v.y, v.z, v.w);
+  }
+  return *reinterpret_cast<const uint4 *>(p);
+}
+template <bool NT>
+__device__ __forceinline__ void store16(void *p, const uint4 &v) {
+  if (NT) {
+    u32x4 x = {v.x, v.y, v.z, v.w};
+    __builtin_nontemporal_store(x, reinterpret_cast<u32x4 *>(p));
+  } else {
+    *reinterpret_cast<uint4 *>(p) = v;
+  }
+}
+
 // ---- wave64 reductions --------------------------------------------------------
 //
 // Steps inside a 16-lane DPP row use quad_perm / row_half_mirror / row_mirror

@@ -27,7 +27,7 @@ struct LnArgs {
   float eps;
 };
 
-template <int DTI, int DTO, int VPL, int TPR>
+template <int DTI, int DTO, int VPL, int TPR, bool STREAM>
 __global__ __launch_bounds__(TPR < kBlock ? kBlock : TPR) void layernorm_rows_kernel(LnArgs a) {
   typedef Elem<DTI> EI;
   typedef Elem<DTO> EO;
@@ -56,11 +56,11 @@ __global__ __launch_bounds__(TPR < kBlock ? kBlock : TPR) void layernorm_rows_ke
   for (int j = 0; j < VPL; ++j) {
     const int v = t + TPR * j;
     if (v < nvec) {
-      const Pack<TI, EPV> pk = load_pack<TI, EPV>(in + v * EPV);
+      const Pack<TI, EPV> pk = __builtin_bit_cast(Pack<TI, EPV>, load16<false>(in + v * EPV));
 #pragma unroll
       for (int e = 0; e < EPV; ++e) x[j][e] = EI::to_float(pk.v[e]);
       if (res) {
-        const Pack<TI, EPV> rk = load_pack<TI, EPV>(res + v * EPV);
+        const Pack<TI, EPV> rk = __builtin_bit_cast(Pack<TI, EPV>, load16<false>(res + v * EPV));
 #pragma unroll
         for (int e = 0; e < EPV; ++e) x[j][e] += EI::to_float(rk.v[e]);
       }
@@ -108,7 +108,8 @@ __global__ __launch_bounds__(TPR < kBlock ? kBlock : TPR) void layernorm_rows_ke
 #pragma unroll
       for (int e = 0; e < EPV; ++e)
         o.v[e] = EO::from_float((x[j][e] - mu) * inv * EO::to_float(g.v[e]) + EO::to_float(bt.v[e]));
-      store_pack<TO, EPV>(out + v * EPV, o);
+      if constexpr (sizeof(TO) * EPV == 16) store16<STREAM>(out + v * EPV, __builtin_bit_cast(uint4, o));
+      else store_pack<TO, EPV>(out + v * EPV, o);
     }
   }
   if (t == 0) {
@@ -165,7 +166,10 @@ template <int DTI, int DTO, int VPL, int TPR>
 static void launch_rows(const LnArgs &a, hipStream_t s) {
   constexpr int BLOCK = TPR < kBlock ? kBlock : TPR;
   constexpr int ROWS_PER_BLOCK = BLOCK / TPR;
-  layernorm_rows_kernel<DTI, DTO, VPL, TPR><<<(unsigned)ceil_div(a.n1, ROWS_PER_BLOCK), BLOCK, 0, s>>>(a);
+  const unsigned grid = (unsigned)ceil_div(a.n1, ROWS_PER_BLOCK);
+  // outputs too large to stay in the memory-side cache are written with non-temporal stores
+  if (a.n1 * a.n2 * Elem<DTO>::kSize >= kStreamStoreBytes) layernorm_rows_kernel<DTI, DTO, VPL, TPR, true><<<grid, BLOCK, 0, s>>>(a);
+  else layernorm_rows_kernel<DTI, DTO, VPL, TPR, false><<<grid, BLOCK, 0, s>>>(a);
 }
 
 template <int DTI, int DTO, int TPR>

@@ -166,7 +166,13 @@ template <> __device__ __forceinline__ uint2 zero_vec<uint2>() { return make_uin
 template <> __device__ __forceinline__ uint32_t zero_vec<uint32_t>() { return 0u; }
 template <> __device__ __forceinline__ uint16_t zero_vec<uint16_t>() { return (uint16_t)0; }
 
-template <typename Vec, typename Map, int NT>
+// stores of the mover; the 16-byte path has a non-temporal form for outputs too large to stay cached
+template <typename Vec, bool STREAM> __device__ __forceinline__ void put(Vec *p, const Vec &v) {
+  if constexpr (sizeof(Vec) == 16) store16<STREAM>(p, v);
+  else *p = v;
+}
+
+template <typename Vec, typename Map, int NT, bool STREAM>
 __global__ __launch_bounds__(kBlock) void row_gather_kernel(Map map, Ptrs3 p, int vpr, int rows_per_block) {
   __shared__ int64_t s_src[kMaxTileRows];
   __shared__ int64_t s_dst[kMaxTileRows];
@@ -206,7 +212,7 @@ __global__ __launch_bounds__(kBlock) void row_gather_kernel(Map map, Ptrs3 p, in
       }
 #pragma unroll
       for (int u = 0; u < U; ++u)
-        if (d[u] >= 0) dst[d[u]] = v[u];
+        if (d[u] >= 0) put<Vec, STREAM>(dst + d[u], v[u]);
     }
   }
 }
@@ -234,8 +240,8 @@ static int tile_rows(int64_t vpr, int64_t total_rows) {
 }
 
 template <typename Map, int NT, typename MakeMap>
-static int launch_row_gather(int64_t row_bytes, int64_t tile_dim_rows, const Ptrs3 &p, MakeMap make_map,
-                             hipStream_t stream) {
+static int launch_row_gather(int64_t row_bytes, int64_t tile_dim_rows, int64_t out_bytes, const Ptrs3 &p,
+                             MakeMap make_map, hipStream_t stream) {
   const int vb = pick_vec_bytes(row_bytes, p, NT);
   const int64_t vpr64 = row_bytes / vb;
   if (vpr64 > (int64_t)INT32_MAX / kMaxTileRows) return EN_ERR_SHAPE;
@@ -246,10 +252,13 @@ static int launch_row_gather(int64_t row_bytes, int64_t tile_dim_rows, const Ptr
   if (grid.x == 0 || grid.y == 0) return EN_OK;
   if (grid.y > 65535u) return EN_ERR_SHAPE;
   switch (vb) {
-    case 16: row_gather_kernel<uint4, Map, NT><<<grid, kBlock, 0, stream>>>(map, p, vpr, R); break;
-    case 8: row_gather_kernel<uint2, Map, NT><<<grid, kBlock, 0, stream>>>(map, p, vpr, R); break;
-    case 4: row_gather_kernel<uint32_t, Map, NT><<<grid, kBlock, 0, stream>>>(map, p, vpr, R); break;
-    default: row_gather_kernel<uint16_t, Map, NT><<<grid, kBlock, 0, stream>>>(map, p, vpr, R); break;
+    case 16:
+      if (out_bytes >= kStreamStoreBytes) row_gather_kernel<uint4, Map, NT, true><<<grid, kBlock, 0, stream>>>(map, p, vpr, R);
+      else row_gather_kernel<uint4, Map, NT, false><<<grid, kBlock, 0, stream>>>(map, p, vpr, R);
+      break;
+    case 8: row_gather_kernel<uint2, Map, NT, false><<<grid, kBlock, 0, stream>>>(map, p, vpr, R); break;
+    case 4: row_gather_kernel<uint32_t, Map, NT, false><<<grid, kBlock, 0, stream>>>(map, p, vpr, R); break;
+    default: row_gather_kernel<uint16_t, Map, NT, false><<<grid, kBlock, 0, stream>>>(map, p, vpr, R); break;
   }
   EN_RETURN_IF_LAUNCH_FAILED();
   return EN_OK;
@@ -310,7 +319,8 @@ int en_depad(const void *src, void *dst, const int32_t *cu_seqlens, int batch, i
   if (batch < 1 || max_seq_len < 1 || hidden < 1) return EN_ERR_SHAPE;
   if (!aligned_to(src, elem_size) || !aligned_to(dst, elem_size)) return EN_ERR_ALIGN;
   Ptrs3 p = {{src, nullptr, nullptr}, {dst, nullptr, nullptr}};
-  return launch_row_gather<DepadRowsMap, 1>(hidden * elem_size, max_seq_len, p, [&](int R, dim3 &grid) {
+  return launch_row_gather<DepadRowsMap, 1>(hidden * elem_size, max_seq_len,
+                                            (int64_t)batch * max_seq_len * hidden * elem_size / 2, p, [&](int R, dim3 &grid) {
     grid = dim3((unsigned)ceil_div(max_seq_len, R), (unsigned)batch, 1);
     return DepadRowsMap{cu_seqlens, max_seq_len, R, left_padded ? 1 : 0};
   }, (hipStream_t)stream);
@@ -323,7 +333,8 @@ int en_transpose_pad(const void *src, void *dst, const int32_t *cu_seqlens, int 
   if (batch < 1 || max_seq_len < 1 || head_num < 1 || size_per_head < 1) return EN_ERR_SHAPE;
   if (!aligned_to(src, elem_size) || !aligned_to(dst, elem_size)) return EN_ERR_ALIGN;
   Ptrs3 p = {{src, nullptr, nullptr}, {dst, nullptr, nullptr}};
-  return launch_row_gather<PadMap, 1>((int64_t)size_per_head * elem_size, max_seq_len, p, [&](int R, dim3 &grid) {
+  return launch_row_gather<PadMap, 1>((int64_t)size_per_head * elem_size, max_seq_len,
+                                      (int64_t)batch * max_seq_len * head_num * size_per_head * elem_size, p, [&](int R, dim3 &grid) {
     grid = dim3((unsigned)(ceil_div(max_seq_len, R) * head_num), (unsigned)batch, 1);
     return PadMap{cu_seqlens, head_num, max_seq_len, R};
   }, (hipStream_t)stream);
@@ -336,7 +347,8 @@ int en_transpose_depad(const void *src, void *dst, const int32_t *cu_seqlens, in
   if (batch < 1 || max_seq_len < 1 || head_num < 1 || size_per_head < 1) return EN_ERR_SHAPE;
   if (!aligned_to(src, elem_size) || !aligned_to(dst, elem_size)) return EN_ERR_ALIGN;
   Ptrs3 p = {{src, nullptr, nullptr}, {dst, nullptr, nullptr}};
-  return launch_row_gather<DepadHeadsMap, 1>((int64_t)size_per_head * elem_size, max_seq_len, p,
+  return launch_row_gather<DepadHeadsMap, 1>((int64_t)size_per_head * elem_size, max_seq_len,
+                                             (int64_t)batch * max_seq_len * head_num * size_per_head * elem_size / 2, p,
                                              [&](int R, dim3 &grid) {
     grid = dim3((unsigned)(ceil_div(max_seq_len, R) * head_num), (unsigned)batch, 1);
     return DepadHeadsMap{cu_seqlens, head_num, max_seq_len, R};
@@ -361,7 +373,8 @@ int en_ft_remove_padding(const void *src, void *tgt, const int32_t *tmp_mask_off
   if (valid_word_num == 0) return EN_OK;
   if (!aligned_to(src, elem_size) || !aligned_to(tgt, elem_size)) return EN_ERR_ALIGN;
   Ptrs3 p = {{src, nullptr, nullptr}, {tgt, nullptr, nullptr}};
-  return launch_row_gather<FtRemoveMap, 1>(hidden * elem_size, valid_word_num, p, [&](int R, dim3 &grid) {
+  return launch_row_gather<FtRemoveMap, 1>(hidden * elem_size, valid_word_num,
+                                           (int64_t)valid_word_num * hidden * elem_size, p, [&](int R, dim3 &grid) {
     grid = dim3((unsigned)ceil_div(valid_word_num, R), 1, 1);
     return FtRemoveMap{tmp_mask_offset, mask_offset, valid_word_num, R};
   }, (hipStream_t)stream);
@@ -376,7 +389,7 @@ int en_ft_rebuild_padding(const void *src, void *tgt, const int32_t *mask_offset
   if (rows_out > INT32_MAX || valid_word_num > rows_out) return EN_ERR_SHAPE;
   if (!aligned_to(src, elem_size) || !aligned_to(tgt, elem_size)) return EN_ERR_ALIGN;
   Ptrs3 p = {{src, nullptr, nullptr}, {tgt, nullptr, nullptr}};
-  return launch_row_gather<FtRebuildMap, 1>(hidden * elem_size, rows_out, p, [&](int R, dim3 &grid) {
+  return launch_row_gather<FtRebuildMap, 1>(hidden * elem_size, rows_out, rows_out * hidden * elem_size, p, [&](int R, dim3 &grid) {
     grid = dim3((unsigned)ceil_div(rows_out, R), 1, 1);
     return FtRebuildMap{mask_offset, valid_word_num, (int)rows_out, R};
   }, (hipStream_t)stream);
@@ -400,9 +413,10 @@ int en_ft_transpose_rebuild(const void *Q, const void *K, const void *V, void *q
     return FtTransposeRebuildMap{mask_offset, valid_word_num, head_num, seq_len, R};
   };
   const int64_t row_bytes = (int64_t)size_per_head * elem_size;
-  if (nt == 3) return launch_row_gather<FtTransposeRebuildMap, 3>(row_bytes, valid_word_num, p, mk, (hipStream_t)stream);
-  if (nt == 2) return launch_row_gather<FtTransposeRebuildMap, 2>(row_bytes, valid_word_num, p, mk, (hipStream_t)stream);
-  return launch_row_gather<FtTransposeRebuildMap, 1>(row_bytes, valid_word_num, p, mk, (hipStream_t)stream);
+  const int64_t out_bytes = (int64_t)valid_word_num * head_num * row_bytes * nt;
+  if (nt == 3) return launch_row_gather<FtTransposeRebuildMap, 3>(row_bytes, valid_word_num, out_bytes, p, mk, (hipStream_t)stream);
+  if (nt == 2) return launch_row_gather<FtTransposeRebuildMap, 2>(row_bytes, valid_word_num, out_bytes, p, mk, (hipStream_t)stream);
+  return launch_row_gather<FtTransposeRebuildMap, 1>(row_bytes, valid_word_num, out_bytes, p, mk, (hipStream_t)stream);
 }
 
 int en_ft_transpose_remove(const void *src, void *dst, int valid_word_num, int batch, int seq_len, int head_num,
@@ -413,7 +427,8 @@ int en_ft_transpose_remove(const void *src, void *dst, int valid_word_num, int b
   if (valid_word_num == 0) return EN_OK;
   if (!aligned_to(src, elem_size) || !aligned_to(dst, elem_size)) return EN_ERR_ALIGN;
   Ptrs3 p = {{src, nullptr, nullptr}, {dst, nullptr, nullptr}};
-  return launch_row_gather<FtTransposeRemoveMap, 1>((int64_t)size_per_head * elem_size, valid_word_num, p,
+  return launch_row_gather<FtTransposeRemoveMap, 1>((int64_t)size_per_head * elem_size, valid_word_num,
+                                                    (int64_t)valid_word_num * head_num * size_per_head * elem_size, p,
                                                     [&](int R, dim3 &grid) {
     grid = dim3((unsigned)(ceil_div(valid_word_num, R) * head_num), 1, 1);
     return FtTransposeRemoveMap{mask_offset, valid_word_num, head_num, seq_len, R};

@@ -56,8 +56,8 @@ def attn_qk(q, k, seq_len_list, *, alpha: float = 1.0, causal: bool = True, q_le
         _lib.require_gpu(out, "out")
         if out.shape != (B, H, Sq, Sk) or out.dtype != q.dtype:
             raise RuntimeError("attn_qk: out must be a contiguous [B,H,Sq,Sk] tensor of q's dtype")
-    with torch.cuda.device(q.device):
-        _lib.check(_lib.load().en_attn_qk(q.data_ptr(), k.data_ptr(), out.data_ptr(), k_info.lens.data_ptr(), q_ptr,
+    with _lib.device_guard(q):
+        _lib.check(_lib.fn.en_attn_qk(q.data_ptr(), k.data_ptr(), out.data_ptr(), k_info.lens.data_ptr(), q_ptr,
                                           B, H, Sq, Sk, D, *qs, *ks, float(alpha), int(bool(causal)),
                                           _lib.dtype_tag(q, "attn_qk"), _lib.stream_of(q)), "attn_qk")
     return out
@@ -85,8 +85,8 @@ def attn_pv(p, v, seq_len_list, *, causal: bool = True, q_len_list=None, zero_pa
         if out.shape != (B, H, Sq, D) or out.dtype != p.dtype:
             raise RuntimeError("attn_pv: out must be [B,H,Sq,D] of p's dtype")
     cs = (out.stride(0), out.stride(1), out.stride(2))
-    with torch.cuda.device(p.device):
-        _lib.check(_lib.load().en_attn_pv(p.data_ptr(), v.data_ptr(), out.data_ptr(), k_info.lens.data_ptr(), q_ptr,
+    with _lib.device_guard(p):
+        _lib.check(_lib.fn.en_attn_pv(p.data_ptr(), v.data_ptr(), out.data_ptr(), k_info.lens.data_ptr(), q_ptr,
                                           B, H, Sq, Sk, D, *vs, *cs, int(bool(causal)), int(bool(zero_padding)),
                                           _lib.dtype_tag(p, "attn_pv"), _lib.stream_of(p)), "attn_pv")
     return out
@@ -103,8 +103,8 @@ def decode_qk(q, k_cache, kv_len_list, *, alpha: float = 1.0, out: Optional[torc
     info = seq_info(kv_len_list, B, q.device)
     if out is None:
         out = torch.empty((B, H, 1, Smax), dtype=q.dtype, device=q.device)
-    with torch.cuda.device(q.device):
-        _lib.check(_lib.load().en_decode_qk(q_.data_ptr(), k_cache.data_ptr(), out.data_ptr(), info.lens.data_ptr(),
+    with _lib.device_guard(q):
+        _lib.check(_lib.fn.en_decode_qk(q_.data_ptr(), k_cache.data_ptr(), out.data_ptr(), info.lens.data_ptr(),
                                             B, H, Smax, D, *ks, float(alpha), _lib.dtype_tag(q, "decode_qk"),
                                             _lib.stream_of(q)), "decode_qk")
     return out
@@ -120,8 +120,8 @@ def decode_pv(p, v_cache, kv_len_list, *, out: Optional[torch.Tensor] = None):
     info = seq_info(kv_len_list, B, p.device)
     if out is None:
         out = torch.empty((B, H, 1, D), dtype=p.dtype, device=p.device)
-    with torch.cuda.device(p.device):
-        _lib.check(_lib.load().en_decode_pv(p.data_ptr(), v_cache.data_ptr(), out.data_ptr(), info.lens.data_ptr(),
+    with _lib.device_guard(p):
+        _lib.check(_lib.fn.en_decode_pv(p.data_ptr(), v_cache.data_ptr(), out.data_ptr(), info.lens.data_ptr(),
                                             B, H, Smax, D, *vs, _lib.dtype_tag(p, "decode_pv"), _lib.stream_of(p)),
                    "decode_pv")
     return out

@@ -78,8 +78,8 @@ def layer_norm_forward(input, weight, bias, normalized_shape, eps=1e-5, residual
         invvar = torch.empty_like(mean)
     if return_sum:
         sum_out = torch.empty_like(input_)
-    with torch.cuda.device(input_.device):
-        _lib.check(_lib.load().en_layernorm_fwd(
+    with _lib.device_guard(input_):
+        _lib.check(_lib.fn.en_layernorm_fwd(
             output.data_ptr(), _lib.ptr(mean), _lib.ptr(invvar), _lib.ptr(sum_out), input_.data_ptr(),
             _lib.ptr(res_), weight_.data_ptr(), bias_.data_ptr(), n1, n2, float(eps),
             _lib.dtype_tag(input_, "layer_norm"), _lib.dtype_tag(weight_, "layer_norm"),

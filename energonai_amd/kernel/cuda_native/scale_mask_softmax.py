@@ -12,6 +12,9 @@ Keyword extensions (defaults preserve the reference behaviour):
 ``k_seq_len``  key extent when src is rectangular [B,H,batch_seq_len,k_seq_len]
 ``q_len_list`` valid query rows per sequence when they differ from the key
                lengths (decode: one query against a longer cache)
+``tail_rows``  0 zeroes the whole masked tail of each row (reference); 128 zeroes
+               only what ``attn_pv`` reads (the extent of the row's 128-row query
+               tile) and leaves the rest of the row untouched
 
 There is no limit on the sequence length (the reference cannot launch above
 1024) and offsets are 64-bit.
@@ -30,7 +33,7 @@ except RuntimeError as _exc:
 
 
 def scale_mask_softmax(batch_size, batch_seq_len, head_num, src, seq_len_list, *, scale=1.0, causal=True,
-                       k_seq_len=None, q_len_list=None):
+                       k_seq_len=None, q_len_list=None, tail_rows=0):
     _lib.require_gpu(src, "correlation", contiguous=False)
     if src.dtype not in (torch.float32, torch.float16, torch.bfloat16):
         raise RuntimeError("Datatype not implemented")
@@ -45,9 +48,9 @@ def scale_mask_softmax(batch_size, batch_seq_len, head_num, src, seq_len_list, *
     if q_len_list is not None:
         q_info = seq_info(q_len_list, batch_size, src.device)
         q_ptr = q_info.lens.data_ptr()
-    with torch.cuda.device(src.device):
-        _lib.check(_lib.load().en_scale_mask_softmax(src.data_ptr(), k_info.lens.data_ptr(), q_ptr, batch_size,
+    with _lib.device_guard(src):
+        _lib.check(_lib.fn.en_scale_mask_softmax(src.data_ptr(), k_info.lens.data_ptr(), q_ptr, batch_size,
                                                      head_num, batch_seq_len, k_seq_len, float(scale),
-                                                     int(bool(causal)), _lib.dtype_tag(src, "scale_mask_softmax"),
+                                                     int(bool(causal)), int(tail_rows), _lib.dtype_tag(src, "scale_mask_softmax"),
                                                      _lib.stream_of(src)), "scale_mask_softmax")
     return src

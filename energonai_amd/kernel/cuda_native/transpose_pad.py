@@ -55,8 +55,8 @@ def transpose_pad(src, batch_size, max_seq_len, seq_len_list, head_num, size_per
     if src.numel() % (head_num * size_per_head) != 0:
         raise RuntimeError("transpose_pad: src size is not a multiple of head_num * size_per_head")
     dst = torch.empty((batch_size, head_num, max_seq_len, size_per_head), dtype=src.dtype, device=src.device)
-    with torch.cuda.device(src.device):
-        _lib.check(_lib.load().en_transpose_pad(src.data_ptr(), dst.data_ptr(), info.cu_seqlens.data_ptr(),
+    with _lib.device_guard(src):
+        _lib.check(_lib.fn.en_transpose_pad(src.data_ptr(), dst.data_ptr(), info.cu_seqlens.data_ptr(),
                                                 batch_size, max_seq_len, head_num, size_per_head,
                                                 _elem_size(src, "transpose_pad"), _lib.stream_of(src)),
                    "transpose_pad")
@@ -72,8 +72,8 @@ def transpose_depad(src, batch_size, sum_seq, max_seq_len, seq_len_list, head_nu
     if src.numel() != batch_size * head_num * max_seq_len * size_per_head:
         raise RuntimeError("transpose_depad: src does not have batch*head*seq*size_per_head elements")
     dst = torch.empty((1, total, head_num, size_per_head), dtype=src.dtype, device=src.device)
-    with torch.cuda.device(src.device):
-        _lib.check(_lib.load().en_transpose_depad(src.data_ptr(), dst.data_ptr(), info.cu_seqlens.data_ptr(),
+    with _lib.device_guard(src):
+        _lib.check(_lib.fn.en_transpose_depad(src.data_ptr(), dst.data_ptr(), info.cu_seqlens.data_ptr(),
                                                   batch_size, max_seq_len, head_num, size_per_head,
                                                   _elem_size(src, "transpose_depad"), _lib.stream_of(src)),
                    "transpose_depad")
@@ -95,8 +95,8 @@ def depad(src, batch_size, seq_lens, left_padded=False, sum_seq=None):
     total = info.total if sum_seq is None else _as_int(sum_seq)
     S, hid = src.shape[1], src.shape[2]
     dst = torch.empty((1, total, hid), dtype=src.dtype, device=src.device)
-    with torch.cuda.device(src.device):
-        _lib.check(_lib.load().en_depad(src.data_ptr(), dst.data_ptr(), info.cu_seqlens.data_ptr(), batch_size, S,
+    with _lib.device_guard(src):
+        _lib.check(_lib.fn.en_depad(src.data_ptr(), dst.data_ptr(), info.cu_seqlens.data_ptr(), batch_size, S,
                                         hid, _elem_size(src, "depad"), int(bool(left_padded)), _lib.stream_of(src)),
                    "depad")
     return dst
@@ -117,8 +117,8 @@ def ft_build_padding_offsets(seq_lens, batch_size, max_seq_len, valid_word_num, 
         raise RuntimeError("sequence_length must be an int32 or int64 tensor")
     if tmp_mask_offset.numel() < batch_size * max_seq_len:
         raise RuntimeError("tmp_mask_offset must hold batch_size * max_seq_len entries")
-    with torch.cuda.device(seq_lens.device):
-        _lib.check(_lib.load().en_ft_build_offsets(seq_lens.data_ptr(), batch_size, max_seq_len,
+    with _lib.device_guard(seq_lens):
+        _lib.check(_lib.fn.en_ft_build_offsets(seq_lens.data_ptr(), batch_size, max_seq_len,
                                                    valid_word_num.data_ptr(), tmp_mask_offset.data_ptr(),
                                                    _lib.stream_of(seq_lens)), "ft_build_padding_offsets")
 
@@ -133,8 +133,8 @@ def ft_remove_padding(src, tmp_mask_offset, mask_offset, valid_word_num, hidden_
     if mask_offset.numel() < valid or tmp_mask_offset.numel() < valid:
         raise RuntimeError("ft_remove_padding: offset tensors are shorter than valid_word_num")
     tgt = torch.empty((1, valid, hidden_dim), dtype=src.dtype, device=src.device)
-    with torch.cuda.device(src.device):
-        _lib.check(_lib.load().en_ft_remove_padding(src.data_ptr(), tgt.data_ptr(), tmp_mask_offset.data_ptr(),
+    with _lib.device_guard(src):
+        _lib.check(_lib.fn.en_ft_remove_padding(src.data_ptr(), tgt.data_ptr(), tmp_mask_offset.data_ptr(),
                                                     mask_offset.data_ptr(), valid, hidden_dim,
                                                     _elem_size(src, "ft_remove_padding"), _lib.stream_of(src)),
                    "ft_remove_padding")
@@ -150,8 +150,8 @@ def ft_rebuild_padding(src, mask_offset, valid_word_num, hidden_dim, batch_size,
     if mask_offset.numel() < valid:
         raise RuntimeError("ft_rebuild_padding: mask_offset is shorter than valid_word_num")
     tgt = torch.empty((batch_size, max_seq_len, hidden_dim), dtype=src.dtype, device=src.device)
-    with torch.cuda.device(src.device):
-        _lib.check(_lib.load().en_ft_rebuild_padding(src.data_ptr(), tgt.data_ptr(), mask_offset.data_ptr(), valid,
+    with _lib.device_guard(src):
+        _lib.check(_lib.fn.en_ft_rebuild_padding(src.data_ptr(), tgt.data_ptr(), mask_offset.data_ptr(), valid,
                                                      hidden_dim, batch_size, max_seq_len,
                                                      _elem_size(src, "ft_rebuild_padding"), _lib.stream_of(src)),
                    "ft_rebuild_padding")
@@ -176,8 +176,8 @@ def ft_transpose_rebuild_padding(Q, K, V, q_buf, k_buf, v_buf, batch_size, seq_l
     need = batch_size * head_num * seq_len * size_per_head
     if min(q_buf.numel(), k_buf.numel(), v_buf.numel()) < need:
         raise RuntimeError("ft_transpose_rebuild_padding: buffers are smaller than [B,H,S,D]")
-    with torch.cuda.device(Q.device):
-        _lib.check(_lib.load().en_ft_transpose_rebuild(Q.data_ptr(), K.data_ptr(), V.data_ptr(), q_buf.data_ptr(),
+    with _lib.device_guard(Q):
+        _lib.check(_lib.fn.en_ft_transpose_rebuild(Q.data_ptr(), K.data_ptr(), V.data_ptr(), q_buf.data_ptr(),
                                                        k_buf.data_ptr(), v_buf.data_ptr(), batch_size, seq_len,
                                                        head_num, size_per_head, valid, mask_offset.data_ptr(),
                                                        _elem_size(Q, "ft_transpose_rebuild_padding"),
@@ -191,8 +191,8 @@ def ft_transpose_remove_padding(src, valid_word_num, batch_size, seq_len, head_n
     _int32_gpu(mask_offset, "mask_offset")
     valid = _as_int(valid_word_num)
     dst = torch.empty((1, valid, head_num * size_per_head), dtype=src.dtype, device=src.device)
-    with torch.cuda.device(src.device):
-        _lib.check(_lib.load().en_ft_transpose_remove(src.data_ptr(), dst.data_ptr(), valid, batch_size, seq_len,
+    with _lib.device_guard(src):
+        _lib.check(_lib.fn.en_ft_transpose_remove(src.data_ptr(), dst.data_ptr(), valid, batch_size, seq_len,
                                                       head_num, size_per_head, mask_offset.data_ptr(),
                                                       _elem_size(src, "ft_transpose_remove_padding"),
                                                       _lib.stream_of(src)), "ft_transpose_remove_padding")

@@ -21,6 +21,10 @@ from .kernel import (attn_pv, attn_qk, decode_pv, decode_qk, depad, layer_norm_f
 from .seqinfo import SeqInfo, seq_info
 
 
+# attn_pv reads a row of probabilities only up to the visible extent of its 128-row query tile
+PV_QUERY_TILE = 128
+
+
 def padding_removal_layer(hidden_padded: torch.Tensor, qkv_packed: torch.Tensor, seq_lens, head_num: int,
                           size_per_head: int, gamma: torch.Tensor, beta: torch.Tensor, eps: float = 1e-5,
                           scale: Optional[float] = None, causal: bool = True, left_padded: bool = False,
@@ -41,7 +45,7 @@ def padding_removal_layer(hidden_padded: torch.Tensor, qkv_packed: torch.Tensor,
     qkv = transpose_pad(qkv_packed, B, S, info, H, 3 * D)
     q, k, v = torch.chunk(qkv, 3, dim=-1)
     scores = attn_qk(q, k, info, causal=causal)
-    probs = scale_mask_softmax(B, S, H, scores, info, scale=scale, causal=causal)
+    probs = scale_mask_softmax(B, S, H, scores, info, scale=scale, causal=causal, tail_rows=PV_QUERY_TILE)
     ctx = attn_pv(probs, v, info, causal=causal)
     ctx_packed = transpose_depad(ctx, B, T, S, info, H, D)
     attn_out = ctx_packed.view(1, T, H * D) if dense_out is None else dense_out

@@ -66,7 +66,7 @@ def build_seq_info(seq_lens, batch_size: int, device=None, total: Optional[int] 
         seq_lens = seq_lens.to(device, non_blocking=False)
     seq_lens = seq_lens.contiguous()
     lib = _lib.load()
-    with torch.cuda.device(seq_lens.device):
+    with _lib.device_guard(seq_lens):
         cu = torch.empty(batch_size + 1, dtype=torch.int32, device=seq_lens.device)
         lens32 = torch.empty(batch_size, dtype=torch.int32, device=seq_lens.device)
         _lib.check(lib.en_prefix_sum(seq_lens.data_ptr(), int(seq_lens.dtype == torch.int64), batch_size,

@@ -109,10 +109,15 @@ int en_ft_transpose_remove(const void *src, void *dst, int valid_word_num, int b
  * become softmax(scale * src[..., :n]) and the remaining Sk-n entries zero;
  * n = k_lens[b] when causal == 0, else min(k_lens[b], q + k_lens[b] - q_lens[b] + 1).
  * Rows q >= q_lens[b] are not touched (as in the reference, kernel.cu:14-17).
- * q_lens == NULL means q_lens[b] = min(k_lens[b], Sq).  The reference call is
- * Sq == Sk, scale 1, causal 1, q_lens NULL.  No limit on Sk; fp32 math. */
+ * q_lens == NULL means q_lens[b] = min(k_lens[b], Sq).  tail_rows == 0 zeroes the
+ * whole tail of every row as the reference does; tail_rows == t > 0 zeroes a row
+ * only as far as the last row of its t-row query tile can see, which is all
+ * en_attn_pv (t = 128) reads -- the rest of the row is then left untouched.
+ * The reference call is Sq == Sk, scale 1, causal 1, q_lens NULL, tail_rows 0.
+ * No limit on Sk; fp32 math. */
 int en_scale_mask_softmax(void *src, const int32_t *k_lens, const int32_t *q_lens, int batch, int head_num,
-                          int q_seq_len, int k_seq_len, float scale, int causal, int dtype, en_stream_t stream);
+                          int q_seq_len, int k_seq_len, float scale, int causal, int tail_rows, int dtype,
+                          en_stream_t stream);
 
 /* ---- LayerNorm forward -------------------------------------------------- */
 
