@@ -110,7 +110,7 @@ __device__ __forceinline__ int tile_key_extent(const AttnArgs &a, int q_last, in
 // ===========================================================================
 // scores = alpha * Q K^T
 // ===========================================================================
-template <int DT, int DP>
+template <int DT, int DP, bool VEC>
 __global__ __launch_bounds__(kBlock) void attn_qk_kernel(AttnArgs a) {
   typedef Elem<DT> E;
   typedef typename E::T T;
@@ -163,6 +163,10 @@ __global__ __launch_bounds__(kBlock) void attn_qk_kernel(AttnArgs a) {
     }
   }
 
+  // K rows >= kl and channels >= D read as zero through the bounds check; a fetch past the
+  // last tile is all out of range and costs no traffic, so the loop body has no branches.
+  const rsrc_t k_rsrc = make_rsrc(kbase, (uint32_t)(((int64_t)(kl - 1) * a.k_ss + a.D) * E::kSize));
+  const rsrc_t s_rsrc = make_rsrc(sbase, (uint32_t)((int64_t)ql * a.Sk * E::kSize));
   uint4 kreg[KLOADS];
   auto fetch_k = [&](int kt) {
     const int k0 = kt * BN;
@@ -171,11 +175,20 @@ __global__ __launch_bounds__(kBlock) void attn_qk_kernel(AttnArgs a) {
       const int v = tid + i * kBlock;
       const int row = v / KVEC_ROW, c = v % KVEC_ROW;
       const int key = k0 + row;
-      kreg[i] = (key < kl && c * EPV < a.D) ? *reinterpret_cast<const uint4 *>(kbase + (int64_t)key * a.k_ss + c * EPV)
-                                            : zero4();
+      const uint32_t off = (uint32_t)(((int64_t)key * a.k_ss + c * EPV) * E::kSize);
+      kreg[i] = buffer_load16(k_rsrc, (kt < nkt && key < kl && c * EPV < a.D) ? off : kOutOfRange);
     }
   };
   fetch_k(0);
+  if constexpr (VEC) {
+    // Out-of-range (dropped) stores that put the queue of outstanding memory operations into the same
+    // shape on loop entry as on the back edge -- K loads, then score stores -- so the wait for the K
+    // tile at the top of the loop is "all but the last CSTORES operations" and never drains the stores.
+    asm volatile("" ::: "memory");  // keep the loads ahead of the stores in issue order
+#pragma unroll
+    for (int i = 0; i < CSTORES; ++i) buffer_store16(s_rsrc, kOutOfRange + 16u * i, zero4());  // distinct: not merged
+    asm volatile("" ::: "memory");
+  }
 
   for (int kt = 0; kt < nkt; ++kt) {
     const int k0 = kt * BN;
@@ -185,8 +198,8 @@ __global__ __launch_bounds__(kBlock) void attn_qk_kernel(AttnArgs a) {
       const int row = v / KVEC_ROW, c = v % KVEC_ROW;
       *reinterpret_cast<uint4 *>(&lds[row * KPITCH + c * EPV]) = kreg[i];
     }
-    __syncthreads();
-    if (kt + 1 < nkt) fetch_k(kt + 1);
+    lds_barrier();
+    fetch_k(kt + 1);
 
     floatx16 acc[MT][NT];
 #pragma unroll
@@ -207,7 +220,7 @@ __global__ __launch_bounds__(kBlock) void attn_qk_kernel(AttnArgs a) {
 #pragma unroll
         for (int nt = 0; nt < NT; ++nt) M::step(kf[mt], qf[nt][vs], acc[mt][nt]);
     }
-    __syncthreads();  // every wave is done reading K before the tile is reused for scores
+    lds_barrier();  // every wave is done reading K before the tile is reused for scores
 
     // accumulators -> LDS as a row-major [query][key] tile
 #pragma unroll
@@ -223,7 +236,7 @@ __global__ __launch_bounds__(kBlock) void attn_qk_kernel(AttnArgs a) {
           const int kcol = wk * (BN / 2) + mt * 32 + 8 * j + 4 * g;
           store_pack<T, 4>(&lds[qrow * CPITCH + kcol], pk);
         }
-    __syncthreads();
+    lds_barrier();
 
     // LDS -> HBM, whole rows of the tile as 128-bit stores
 #pragma unroll
@@ -231,26 +244,25 @@ __global__ __launch_bounds__(kBlock) void attn_qk_kernel(AttnArgs a) {
       const int v = tid + i * kBlock;
       const int row = v / CVEC_ROW, c = v % CVEC_ROW;
       const int q = q0 + row, k = k0 + c * EPV;
-      if (q < ql && k < a.Sk) {
-        const T *sp = &lds[row * CPITCH + c * EPV];
+      const T *sp = &lds[row * CPITCH + c * EPV];
+      if constexpr (VEC) {  // rows >= ql fall outside the resource and are dropped by the bounds check
+        const uint32_t off = (uint32_t)(((int64_t)q * a.Sk + k) * E::kSize);
+        buffer_store16(s_rsrc, (k < a.Sk) ? off : kOutOfRange, *reinterpret_cast<const uint4 *>(sp));
+      } else if (q < ql && k < a.Sk) {
         T *gp = sbase + (int64_t)q * a.Sk + k;
-        if (a.vec_out) {
-          *reinterpret_cast<uint4 *>(gp) = *reinterpret_cast<const uint4 *>(sp);
-        } else {
 #pragma unroll
-          for (int e = 0; e < EPV; ++e)
-            if (k + e < a.Sk) gp[e] = sp[e];
-        }
+        for (int e = 0; e < EPV; ++e)
+          if (k + e < a.Sk) gp[e] = sp[e];
       }
     }
-    __syncthreads();  // scores leave LDS before the next K tile lands
+    lds_barrier();  // scores leave LDS before the next K tile lands
   }
 }
 
 // ===========================================================================
 // ctx = P V
 // ===========================================================================
-template <int DT, int DP>
+template <int DT, int DP, bool VEC>
 __global__ __launch_bounds__(kBlock) void attn_pv_kernel(AttnArgs a) {
   typedef Elem<DT> E;
   typedef typename E::T T;
@@ -308,6 +320,10 @@ __global__ __launch_bounds__(kBlock) void attn_pv_kernel(AttnArgs a) {
 #pragma unroll
       for (int x = 0; x < 16; ++x) acc[mt][nt][x] = 0.f;
 
+  // rows of padded queries, columns past the visible extent and V rows >= kl read as zero
+  // through the bounds check; the loop body has no branches on the fast path.
+  const rsrc_t p_rsrc = make_rsrc(pbase, (uint32_t)((int64_t)ql * a.Sk * E::kSize));
+  const rsrc_t v_rsrc = make_rsrc(vbase, (uint32_t)(((int64_t)(max(kl, 1) - 1) * a.k_ss + a.D) * E::kSize));
   uint4 preg[PLOADS];
   uint4 vreg[VLOADS][4];
   auto fetch = [&](int kt) {
@@ -317,12 +333,12 @@ __global__ __launch_bounds__(kBlock) void attn_pv_kernel(AttnArgs a) {
       const int v = tid + i * kBlock;
       const int row = v / PVEC_ROW, c = v % PVEC_ROW;
       const int q = q0 + row, k = k0 + c * EPV;
-      // rows of padded queries and columns past the visible extent contribute nothing
-      if (q < ql && k < nk) {
+      if constexpr (VEC) {
+        const uint32_t off = (uint32_t)(((int64_t)q * a.Sk + k) * E::kSize);
+        preg[i] = buffer_load16(p_rsrc, (kt < nkt && k < nk) ? off : kOutOfRange);
+      } else if (kt < nkt && q < ql && k < nk) {
         const T *gp = pbase + (int64_t)q * a.Sk + k;
-        if (a.vec_out) {
-          preg[i] = *reinterpret_cast<const uint4 *>(gp);
-        } else {
+        {
           Pack<T, EPV> pk;
 #pragma unroll
           for (int e = 0; e < EPV; ++e) pk.v[e] = (k + e < nk) ? gp[e] : E::from_float(0.f);
@@ -340,9 +356,8 @@ __global__ __launch_bounds__(kBlock) void attn_pv_kernel(AttnArgs a) {
 #pragma unroll
       for (int x = 0; x < 4; ++x) {
         const int key = k0 + kq * 4 + x;
-        vreg[i][x] = (u < VUNITS && key < kl && c * EPV < a.D)
-                         ? *reinterpret_cast<const uint4 *>(vbase + (int64_t)key * a.k_ss + c * EPV)
-                         : zero4();
+        const uint32_t off = (uint32_t)(((int64_t)key * a.k_ss + c * EPV) * E::kSize);
+        vreg[i][x] = buffer_load16(v_rsrc, (kt < nkt && u < VUNITS && key < kl && c * EPV < a.D) ? off : kOutOfRange);
       }
     }
   };
@@ -360,7 +375,7 @@ __global__ __launch_bounds__(kBlock) void attn_pv_kernel(AttnArgs a) {
 #pragma unroll
     for (int i = 0; i < VLOADS; ++i) {
       const int u = tid + i * kBlock;
-      if (u < VUNITS) {
+      if (VUNITS % kBlock == 0 || u < VUNITS) {
         const int c = (u % 4) + 4 * ((u / (4 * NQUAD)) % (NCHUNK / 4 > 0 ? NCHUNK / 4 : 1));
         const int kq = (u / 4) % NQUAD;
         Pack<T, EPV> rows[4];
@@ -375,8 +390,8 @@ __global__ __launch_bounds__(kBlock) void attn_pv_kernel(AttnArgs a) {
         }
       }
     }
-    __syncthreads();
-    if (kt + 1 < nkt) fetch(kt + 1);
+    lds_barrier();
+    fetch(kt + 1);
 
 #pragma unroll
     for (int vs = 0; vs < NVS; ++vs) {
@@ -393,7 +408,7 @@ __global__ __launch_bounds__(kBlock) void attn_pv_kernel(AttnArgs a) {
 #pragma unroll
         for (int nt = 0; nt < NT; ++nt) M::step(vf[mt], pf[nt], acc[mt][nt]);
     }
-    __syncthreads();  // tiles are consumed before the next ones are written
+    lds_barrier();  // tiles are consumed before the next ones are written
   }
 
   // each lane owns four consecutive channels of one query row
@@ -429,8 +444,13 @@ static bool strides_vec_ok(int64_t sb, int64_t sh, int64_t ss, int epv) {
 template <int DT>
 static int launch_qk(AttnArgs &a, hipStream_t s) {
   const unsigned grid = (unsigned)(ceil_div(a.units, kXcds) * kXcds * a.ntq);
-  if (a.D <= 64) attn_qk_kernel<DT, 64><<<grid, kBlock, 0, s>>>(a);
-  else attn_qk_kernel<DT, 128><<<grid, kBlock, 0, s>>>(a);
+  if (a.vec_out) {
+    if (a.D <= 64) attn_qk_kernel<DT, 64, true><<<grid, kBlock, 0, s>>>(a);
+    else attn_qk_kernel<DT, 128, true><<<grid, kBlock, 0, s>>>(a);
+  } else {
+    if (a.D <= 64) attn_qk_kernel<DT, 64, false><<<grid, kBlock, 0, s>>>(a);
+    else attn_qk_kernel<DT, 128, false><<<grid, kBlock, 0, s>>>(a);
+  }
   EN_RETURN_IF_LAUNCH_FAILED();
   return EN_OK;
 }
@@ -438,8 +458,13 @@ static int launch_qk(AttnArgs &a, hipStream_t s) {
 template <int DT>
 static int launch_pv(AttnArgs &a, hipStream_t s) {
   const unsigned grid = (unsigned)(ceil_div(a.units, kXcds) * kXcds * a.ntq);
-  if (a.D <= 64) attn_pv_kernel<DT, 64><<<grid, kBlock, 0, s>>>(a);
-  else attn_pv_kernel<DT, 128><<<grid, kBlock, 0, s>>>(a);
+  if (a.vec_out) {
+    if (a.D <= 64) attn_pv_kernel<DT, 64, true><<<grid, kBlock, 0, s>>>(a);
+    else attn_pv_kernel<DT, 128, true><<<grid, kBlock, 0, s>>>(a);
+  } else {
+    if (a.D <= 64) attn_pv_kernel<DT, 64, false><<<grid, kBlock, 0, s>>>(a);
+    else attn_pv_kernel<DT, 128, false><<<grid, kBlock, 0, s>>>(a);
+  }
   EN_RETURN_IF_LAUNCH_FAILED();
   return EN_OK;
 }
@@ -453,6 +478,8 @@ static int check_common(const void *x, const void *y, const void *z, const int32
   const int epv = 16 / es;
   if (size_per_head > 128 || (size_per_head % epv) != 0) return EN_ERR_UNSUPPORTED;
   if ((int64_t)batch * head_num > INT32_MAX / 64) return EN_ERR_SHAPE;
+  // per-(batch, head) byte offsets are 32-bit buffer offsets
+  if ((int64_t)q_seq_len * k_seq_len * es >= (1ll << 31)) return EN_ERR_UNSUPPORTED;
   return EN_OK;
 }
 
@@ -472,6 +499,7 @@ int en_attn_qk(const void *q, const void *k, void *scores, const int32_t *k_lens
   if (!strides_vec_ok(q_stride_b, q_stride_h, q_stride_s, epv) ||
       !strides_vec_ok(k_stride_b, k_stride_h, k_stride_s, epv))
     return EN_ERR_ALIGN;
+  if (k_stride_s < 0 || (int64_t)k_seq_len * k_stride_s * es >= (1ll << 31)) return EN_ERR_UNSUPPORTED;
   AttnArgs a{};
   a.a_ptr = q; a.b_ptr = k; a.out = scores; a.k_lens = k_lens; a.q_lens = q_lens;
   a.B = batch; a.H = head_num; a.Sq = q_seq_len; a.Sk = k_seq_len; a.D = size_per_head;
@@ -501,6 +529,7 @@ int en_attn_pv(const void *p, const void *v, void *ctx, const int32_t *k_lens, c
   if (!strides_vec_ok(v_stride_b, v_stride_h, v_stride_s, epv) ||
       !strides_vec_ok(c_stride_b, c_stride_h, c_stride_s, 4))
     return EN_ERR_ALIGN;
+  if (v_stride_s < 0 || (int64_t)k_seq_len * v_stride_s * es >= (1ll << 31)) return EN_ERR_UNSUPPORTED;
   AttnArgs a{};
   a.a_ptr = p; a.b_ptr = v; a.out = ctx; a.k_lens = k_lens; a.q_lens = q_lens;
   a.B = batch; a.H = head_num; a.Sq = q_seq_len; a.Sk = k_seq_len; a.D = size_per_head;

@@ -94,6 +94,31 @@ __device__ __forceinline__ void store16(void *p, const uint4 &v) {
   }
 }
 
+// Buffer accesses with hardware bounds checking: a load whose offset lies outside
+// [0, bytes) returns zero and a store there is dropped, so ragged edges need no
+// branches and the compiler can count outstanding operations statically.
+typedef __amdgpu_buffer_rsrc_t rsrc_t;
+constexpr uint32_t kOutOfRange = 0x80000000u;  // any offset >= 2^31 is outside every resource built here
+
+__device__ __forceinline__ rsrc_t make_rsrc(const void *base, uint32_t bytes) {
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(base), 0, (int)bytes, 0x00020000);
+}
+__device__ __forceinline__ uint4 buffer_load16(rsrc_t r, uint32_t byte_offset) {
+  const u32x4 v = __builtin_amdgcn_raw_buffer_load_b128(r, (int)byte_offset, 0, 0);
+  return make_uint4(v.x, v.y, v.z, v.w);
+}
+__device__ __forceinline__ void buffer_store16(rsrc_t r, uint32_t byte_offset, const uint4 &v) {
+  const u32x4 x = {v.x, v.y, v.z, v.w};
+  __builtin_amdgcn_raw_buffer_store_b128(x, r, (int)byte_offset, 0, 0);
+}
+
+// Workgroup barrier that orders LDS traffic only.  __syncthreads() also waits
+// for every outstanding global load and store of the wave, which would cancel
+// any prefetch that is meant to stay in flight across the barrier.
+__device__ __forceinline__ void lds_barrier() {
+  asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+}
+
 // ---- wave64 reductions --------------------------------------------------------
 //
 // Steps inside a 16-lane DPP row use quad_perm / row_half_mirror / row_mirror
