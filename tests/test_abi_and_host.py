@@ -1,0 +1,156 @@
+"""CPU-only checks of the drop-in boundary: the C ABI library loads and exports
+exactly what include/energon_hip.h declares, the ctypes table matches the
+header, the Python mirror keeps the reference's names and signatures, and host
+argument checks fire before anything reaches the device."""
+import ctypes
+import inspect
+import os
+import re
+import sys
+
+import pytest
+import torch
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "energon_hip.h")
+
+
+def _declared_symbols():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(en_[a-z0-9_]+)\s*\(", text)))
+
+
+def _arg_count(name):
+    text = re.sub(r"/\*.*?\*/", "", open(HEADER).read(), flags=re.S)
+    m = re.search(r"\b%s\s*\((.*?)\)\s*;" % re.escape(name), text, flags=re.S)
+    args = m.group(1).strip()
+    return 0 if args in ("", "void") else len(args.split(","))
+
+
+def test_library_exports_every_declared_symbol():
+    from energonai_amd import _lib
+    lib = _lib.load()
+    declared = _declared_symbols()
+    assert len(declared) >= 20
+    for name in declared:
+        assert hasattr(lib, name), f"{name} is declared in the header but not exported"
+    assert sorted(_lib.SIGNATURES) == declared, "ctypes table and header disagree"
+    for name, (_, argtypes) in _lib.SIGNATURES.items():
+        assert len(argtypes) == _arg_count(name), f"{name}: ctypes arity differs from the header"
+    assert lib.en_version() >= 100
+    assert lib.en_status_string(0) == b"ok"
+    assert b"NULL" in lib.en_status_string(-1)
+
+
+def test_entry_points_validate_before_launch():
+    """NULL pointers and bad extents are refused on the host: no GPU is touched."""
+    from energonai_amd import _lib
+    lib = _lib.load()
+    assert lib.en_prefix_sum(None, 0, 4, None, None, None) == -1
+    assert lib.en_prefix_sum(1, 0, 0, 1, None, None) == -2
+    assert lib.en_depad(None, None, None, 1, 1, 1, 2, 0, None) == -1
+    assert lib.en_depad(16, 32, 48, 1, 1, 1, 3, 0, None) == -3          # element size 3
+    assert lib.en_transpose_pad(16, 32, 48, 0, 1, 1, 1, 2, None) == -2   # batch 0
+    assert lib.en_scale_mask_softmax(16, 32, None, 1, 1, 1, 1, 1.0, 1, 0, 7, None) == -3   # dtype tag 7
+    assert lib.en_scale_mask_softmax(16, 32, None, 1, 1, 1, 1, 1.0, 1, 96, 1, None) == -2  # tile not a power of two
+    assert lib.en_layernorm_fwd(16, None, None, None, 32, None, 48, 64, 1, 8, 1e-5, 1, 0, None) == -3  # (f16 -> f32)
+    assert lib.en_attn_qk(16, 32, 48, 64, None, 1, 1, 8, 8, 200, 0, 0, 200, 0, 0, 200, 1.0, 1, 1, None) == -5  # D > 128
+    assert lib.en_copy_bytes(16, 32, 24, None) == -2                     # not a multiple of 16
+
+
+def test_python_api_keeps_reference_names_and_signatures():
+    from energonai_amd import kernel
+    from energonai_amd.kernel import cuda_native
+    want = {   # energonai/kernel/cuda_native/transpose_pad.py:12-87, scale_mask_softmax.py:10
+        "transpose_pad": ["src", "batch_size", "max_seq_len", "seq_len_list", "head_num", "size_per_head"],
+        "transpose_depad": ["src", "batch_size", "sum_seq", "max_seq_len", "seq_len_list", "head_num",
+                            "size_per_head"],
+        "depad": ["src", "batch_size", "seq_lens"],
+        "scale_mask_softmax": ["batch_size", "batch_seq_len", "head_num", "src", "seq_len_list"],
+        "ft_build_padding_offsets": ["seq_lens", "batch_size", "max_seq_len", "valid_word_num", "tmp_mask_offset"],
+        "ft_remove_padding": ["src", "tmp_mask_offset", "mask_offset", "valid_word_num", "hidden_dim"],
+        "ft_rebuild_padding": ["src", "mask_offset", "valid_word_num", "hidden_dim", "batch_size", "max_seq_len"],
+        "ft_transpose_rebuild_padding": ["Q", "K", "V", "q_buf", "k_buf", "v_buf", "batch_size", "seq_len",
+                                         "head_num", "size_per_head", "valid_word_num", "mask_offset"],
+        "ft_transpose_remove_padding": ["src", "valid_word_num", "batch_size", "seq_len", "head_num",
+                                        "size_per_head", "mask_offset"],
+    }
+    for name, params in want.items():
+        fn = getattr(kernel, name)
+        got = [p.name for p in inspect.signature(fn).parameters.values()
+               if p.kind is p.POSITIONAL_OR_KEYWORD and p.default is p.empty]
+        assert got == params, (name, got)
+    for name in ("linear", "find_algo"):
+        assert callable(getattr(kernel, name))
+    assert cuda_native.LayerNorm is cuda_native.MixedFusedLayerNorm
+    sig = inspect.signature(cuda_native.LayerNorm.__init__)
+    assert list(sig.parameters)[1:] == ["normalized_shape", "eps", "device", "dtype"]
+
+
+def test_extension_name_shims_register_under_reference_names():
+    from energonai_amd import ext
+    ext.install()
+    import importlib
+    tp = importlib.import_module("energonai_transpose_pad")
+    for sym in ("transpose_pad_wrapper", "transpose_depad_wrapper", "ft_build_padding_offsets_wrapper",
+                "ft_remove_padding_wrapper", "ft_rebuild_padding_wrapper", "ft_transpose_remove_padding_wrapper",
+                "ft_transpose_rebuild_padding_wrapper"):
+        assert callable(getattr(tp, sym))    # csrc/transpose_pad_fusion_wrapper.cpp:246-263
+    assert callable(importlib.import_module("energonai_scale_mask").scale_mask_softmax_wrapper)
+    assert callable(importlib.import_module("energonai_layer_norm").forward_affine)
+    assert callable(importlib.import_module("energonai_linear_func").mlp_gemm)
+
+
+def test_host_side_argument_errors_without_gpu():
+    from energonai_amd import kernel
+    lens = torch.tensor([1, 2], dtype=torch.int32)
+    with pytest.raises(RuntimeError, match="must be a CUDA tensor"):
+        kernel.transpose_pad(torch.zeros(1, 3, 2, 4), 2, 4, lens, 2, 4)
+    with pytest.raises(RuntimeError, match="must be a CUDA tensor"):
+        kernel.scale_mask_softmax(2, 4, 1, torch.zeros(2, 1, 4, 4), lens)
+    with pytest.raises(RuntimeError, match="must be a CUDA tensor"):
+        kernel.layer_norm_forward(torch.zeros(2, 8), torch.ones(8), torch.zeros(8), (8,))
+    with pytest.raises(RuntimeError, match="must be a CUDA tensor"):
+        kernel.depad(torch.zeros(2, 4, 8), 2, lens)
+
+
+def test_missing_library_fails_loudly(tmp_path, monkeypatch):
+    """No CPU fallback: without the shared object the product refuses to load."""
+    from energonai_amd import _lib
+    monkeypatch.setattr(_lib, "_lib", None)
+    monkeypatch.setattr(_lib, "LIB_PATH", str(tmp_path / "libenergon_hip.so"))
+    with pytest.raises(RuntimeError, match="requires cuda extensions"):
+        _lib.load()
+
+
+def test_product_never_imports_the_oracle():
+    pkg = os.path.join(ROOT, "energonai_amd")
+    for base, _, files in os.walk(pkg):
+        for f in files:
+            if f.endswith((".py", ".hip", ".h")):
+                text = open(os.path.join(base, f)).read()
+                assert not re.search(r"^\s*(from|import)\s+oracle\b", text, flags=re.M), f
+
+
+def test_workload_definitions():
+    from energonai_amd import workloads as wl
+    totals = {"c1": 698, "c2": 8538, "c3": 9244, "c4": 20142, "c5": 70929}
+    for w in wl.WORKLOADS:
+        lens = wl.make_lens(w)
+        assert lens.dtype == torch.int32 and lens.numel() == w.batch
+        assert int(lens.sum()) == totals[w.name]
+        assert int(lens.min()) >= w.len_lo and int(lens.max()) <= w.len_hi
+    w = wl.BY_NAME["c1"]
+    inp = wl.make_inputs(w)
+    assert inp["hidden_padded"].shape == (8, 128, 768) and inp["qkv_packed"].shape == (1, 698, 12, 192)
+    for b, n in enumerate(inp["lens_list"]):
+        assert bool((inp["hidden_padded"][b, n:] == 0).all())        # right padded, zero padding
+    w2 = wl.BY_NAME["c2"]
+    small = wl.make_inputs(w2, lens=torch.tensor([3, 5], dtype=torch.int32)) if False else None
+    alg = wl.algorithmic_bytes(w, inp["lens_list"])
+    assert alg["depad"] == 2 * 698 * 768 * 4
+    assert alg["transpose_pad"] == 698 * 12 * 192 * 4 + 8 * 128 * 12 * 192 * 4
+    assert alg["layernorm_residual"] == 3 * 698 * 768 * 4
+    vis = sum(n * n for n in inp["lens_list"])
+    assert wl.algorithmic_flops(w, inp["lens_list"]) == 2.0 * 12 * 64 * vis
