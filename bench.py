@@ -300,6 +300,26 @@ def cpu_baseline(torch, w, budget_s=12.0):
                       f"oracle.eager.layer_unpadded (torch-eager restatement of the reference path)"}
 
 
+def copy_yardstick(torch, iters):
+    """en_copy_bytes at 64 MiB, 256 MiB and 1 GiB (read n + write n bytes per launch)."""
+    from energonai_amd import _lib
+    out = {"kernel": "copy_kernel", "unit": "GB/s", "sizes": {}}
+    stream = torch.cuda.current_stream().cuda_stream
+    for mib in (64, 256, 1024):
+        n = mib << 20
+        a = torch.empty(n, dtype=torch.uint8, device="cuda")
+        b = torch.empty_like(a)
+        a.fill_(1)
+        fn = lambda: _lib.check(_lib.fn.en_copy_bytes(a.data_ptr(), b.data_ptr(), n, stream), "copy")
+        for _ in range(3):
+            fn()
+        torch.cuda.synchronize()
+        ms = _event_time_ms(fn, max(5, iters), torch)
+        out["sizes"][f"{mib}MiB"] = {"bytes_read": n, "bytes_written": n, "us": ms * 1e3, "GBps": 2 * n / (ms * 1e-3) / 1e9}
+        del a, b
+    return out
+
+
 def main(argv=None) -> int:
     ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
     ap.add_argument("--gpus", type=int, default=1)
@@ -308,6 +328,9 @@ def main(argv=None) -> int:
     ap.add_argument("--workload", default="c2", choices=["c1", "c2", "c3", "c4", "c5"])
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-extra", action="store_true", help="only the headline workload, no eager / other workloads")
+    ap.add_argument("--copy-yardstick", action="store_true",
+                    help="instead of the benchmark, time en_copy_bytes (plain 128-bit copy) at known sizes; "
+                         "used as the bandwidth yardstick and to calibrate the FETCH_SIZE / WRITE_SIZE counters")
     ns = ap.parse_args(argv)
     if ns.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this build measures one GPU's share of the path; --gpus must be 1 "
@@ -321,6 +344,10 @@ def main(argv=None) -> int:
         return 2
     torch.cuda.set_device(0)
     from energonai_amd import workloads
+
+    if ns.copy_yardstick:
+        print(json.dumps(copy_yardstick(torch, ns.steps)))
+        return 0
 
     w = workloads.BY_NAME[ns.workload]
     torch.cuda.synchronize()
