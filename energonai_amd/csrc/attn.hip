@@ -30,6 +30,7 @@ typedef _Float16 halfx8 __attribute__((ext_vector_type(8)));
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 
 constexpr int kQTile = 128;  // query rows per workgroup
+constexpr int64_t kStreamScoreBytes = 512ll << 20;  // score tensors at least this large bypass the caches
 
 // ---------------------------------------------------------------------------
 // per-dtype MFMA step on one 128-bit vector per lane of each operand.
@@ -110,7 +111,7 @@ __device__ __forceinline__ int tile_key_extent(const AttnArgs &a, int q_last, in
 // ===========================================================================
 // scores = alpha * Q K^T
 // ===========================================================================
-template <int DT, int DP, bool VEC>
+template <int DT, int DP, bool VEC, bool STREAM>
 __global__ __launch_bounds__(kBlock) void attn_qk_kernel(AttnArgs a) {
   typedef Elem<DT> E;
   typedef typename E::T T;
@@ -247,7 +248,7 @@ __global__ __launch_bounds__(kBlock) void attn_qk_kernel(AttnArgs a) {
       const T *sp = &lds[row * CPITCH + c * EPV];
       if constexpr (VEC) {  // rows >= ql fall outside the resource and are dropped by the bounds check
         const uint32_t off = (uint32_t)(((int64_t)q * a.Sk + k) * E::kSize);
-        buffer_store16(s_rsrc, (k < a.Sk) ? off : kOutOfRange, *reinterpret_cast<const uint4 *>(sp));
+        buffer_store16<STREAM ? 2 : 0>(s_rsrc, (k < a.Sk) ? off : kOutOfRange, *reinterpret_cast<const uint4 *>(sp));
       } else if (q < ql && k < a.Sk) {
         T *gp = sbase + (int64_t)q * a.Sk + k;
 #pragma unroll
@@ -262,7 +263,7 @@ __global__ __launch_bounds__(kBlock) void attn_qk_kernel(AttnArgs a) {
 // ===========================================================================
 // ctx = P V
 // ===========================================================================
-template <int DT, int DP, bool VEC>
+template <int DT, int DP, bool VEC, bool STREAM>
 __global__ __launch_bounds__(kBlock) void attn_pv_kernel(AttnArgs a) {
   typedef Elem<DT> E;
   typedef typename E::T T;
@@ -335,7 +336,7 @@ __global__ __launch_bounds__(kBlock) void attn_pv_kernel(AttnArgs a) {
       const int q = q0 + row, k = k0 + c * EPV;
       if constexpr (VEC) {
         const uint32_t off = (uint32_t)(((int64_t)q * a.Sk + k) * E::kSize);
-        preg[i] = buffer_load16(p_rsrc, (kt < nkt && k < nk) ? off : kOutOfRange);
+        preg[i] = buffer_load16<STREAM ? 2 : 0>(p_rsrc, (kt < nkt && k < nk) ? off : kOutOfRange);
       } else if (kt < nkt && q < ql && k < nk) {
         const T *gp = pbase + (int64_t)q * a.Sk + k;
         {
@@ -444,12 +445,19 @@ static bool strides_vec_ok(int64_t sb, int64_t sh, int64_t ss, int epv) {
 template <int DT>
 static int launch_qk(AttnArgs &a, hipStream_t s) {
   const unsigned grid = (unsigned)(ceil_div(a.units, kXcds) * kXcds * a.ntq);
+  // a score tensor too large to stay in the memory-side cache is written with the non-temporal policy
+  const bool stream = (int64_t)a.units * a.Sq * a.Sk * Elem<DT>::kSize >= kStreamScoreBytes;
   if (a.vec_out) {
-    if (a.D <= 64) attn_qk_kernel<DT, 64, true><<<grid, kBlock, 0, s>>>(a);
-    else attn_qk_kernel<DT, 128, true><<<grid, kBlock, 0, s>>>(a);
+    if (a.D <= 64) {
+      if (stream) attn_qk_kernel<DT, 64, true, true><<<grid, kBlock, 0, s>>>(a);
+      else attn_qk_kernel<DT, 64, true, false><<<grid, kBlock, 0, s>>>(a);
+    } else {
+      if (stream) attn_qk_kernel<DT, 128, true, true><<<grid, kBlock, 0, s>>>(a);
+      else attn_qk_kernel<DT, 128, true, false><<<grid, kBlock, 0, s>>>(a);
+    }
   } else {
-    if (a.D <= 64) attn_qk_kernel<DT, 64, false><<<grid, kBlock, 0, s>>>(a);
-    else attn_qk_kernel<DT, 128, false><<<grid, kBlock, 0, s>>>(a);
+    if (a.D <= 64) attn_qk_kernel<DT, 64, false, false><<<grid, kBlock, 0, s>>>(a);
+    else attn_qk_kernel<DT, 128, false, false><<<grid, kBlock, 0, s>>>(a);
   }
   EN_RETURN_IF_LAUNCH_FAILED();
   return EN_OK;
@@ -458,12 +466,19 @@ static int launch_qk(AttnArgs &a, hipStream_t s) {
 template <int DT>
 static int launch_pv(AttnArgs &a, hipStream_t s) {
   const unsigned grid = (unsigned)(ceil_div(a.units, kXcds) * kXcds * a.ntq);
+  // probabilities of a tensor too large to stay cached are read with the non-temporal policy
+  const bool stream = (int64_t)a.units * a.Sq * a.Sk * Elem<DT>::kSize >= kStreamScoreBytes;
   if (a.vec_out) {
-    if (a.D <= 64) attn_pv_kernel<DT, 64, true><<<grid, kBlock, 0, s>>>(a);
-    else attn_pv_kernel<DT, 128, true><<<grid, kBlock, 0, s>>>(a);
+    if (a.D <= 64) {
+      if (stream) attn_pv_kernel<DT, 64, true, true><<<grid, kBlock, 0, s>>>(a);
+      else attn_pv_kernel<DT, 64, true, false><<<grid, kBlock, 0, s>>>(a);
+    } else {
+      if (stream) attn_pv_kernel<DT, 128, true, true><<<grid, kBlock, 0, s>>>(a);
+      else attn_pv_kernel<DT, 128, true, false><<<grid, kBlock, 0, s>>>(a);
+    }
   } else {
-    if (a.D <= 64) attn_pv_kernel<DT, 64, false><<<grid, kBlock, 0, s>>>(a);
-    else attn_pv_kernel<DT, 128, false><<<grid, kBlock, 0, s>>>(a);
+    if (a.D <= 64) attn_pv_kernel<DT, 64, false, false><<<grid, kBlock, 0, s>>>(a);
+    else attn_pv_kernel<DT, 128, false, false><<<grid, kBlock, 0, s>>>(a);
   }
   EN_RETURN_IF_LAUNCH_FAILED();
   return EN_OK;

@@ -103,13 +103,16 @@ constexpr uint32_t kOutOfRange = 0x80000000u;  // any offset >= 2^31 is outside 
 __device__ __forceinline__ rsrc_t make_rsrc(const void *base, uint32_t bytes) {
   return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(base), 0, (int)bytes, 0x00020000);
 }
+// AUX is the cache-policy immediate of the instruction; 2 = non-temporal (streamed once).
+template <int AUX = 0>
 __device__ __forceinline__ uint4 buffer_load16(rsrc_t r, uint32_t byte_offset) {
-  const u32x4 v = __builtin_amdgcn_raw_buffer_load_b128(r, (int)byte_offset, 0, 0);
+  const u32x4 v = __builtin_amdgcn_raw_buffer_load_b128(r, (int)byte_offset, 0, AUX);
   return make_uint4(v.x, v.y, v.z, v.w);
 }
+template <int AUX = 0>
 __device__ __forceinline__ void buffer_store16(rsrc_t r, uint32_t byte_offset, const uint4 &v) {
   const u32x4 x = {v.x, v.y, v.z, v.w};
-  __builtin_amdgcn_raw_buffer_store_b128(x, r, (int)byte_offset, 0, 0);
+  __builtin_amdgcn_raw_buffer_store_b128(x, r, (int)byte_offset, 0, AUX);
 }
 
 // Workgroup barrier that orders LDS traffic only.  __syncthreads() also waits
