@@ -10,10 +10,10 @@ from .cuda_native import (ft_build_padding_offsets, ft_remove_padding, ft_rebuil
                           ft_transpose_remove_padding, ft_transpose_rebuild_padding)
 from .cuda_native import linear, find_algo
 from .cuda_native import LayerNorm, layer_norm_forward
-from .attention import attn_qk, attn_pv, decode_qk, decode_pv
+from .attention import attn_qk, attn_pv, attn_fused, decode_qk, decode_pv
 
 __all__ = [
     "transpose_pad", "transpose_depad", "depad", "scale_mask_softmax", "ft_build_padding_offsets",
     "ft_remove_padding", "ft_rebuild_padding", "ft_transpose_remove_padding", "ft_transpose_rebuild_padding",
-    "linear", "find_algo", "LayerNorm", "layer_norm_forward", "attn_qk", "attn_pv", "decode_qk", "decode_pv",
+    "linear", "find_algo", "LayerNorm", "layer_norm_forward", "attn_qk", "attn_pv", "attn_fused", "decode_qk", "decode_pv",
 ]

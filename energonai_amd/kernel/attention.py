@@ -10,6 +10,7 @@ at or left of the diagonal.  ``q``, ``k`` and ``v`` may be the strided
 """
 from __future__ import annotations
 
+import ctypes
 from typing import Optional
 
 import torch
@@ -89,6 +90,41 @@ def attn_pv(p, v, seq_len_list, *, causal: bool = True, q_len_list=None, zero_pa
         _lib.check(_lib.fn.en_attn_pv(p.data_ptr(), v.data_ptr(), out.data_ptr(), k_info.lens.data_ptr(), q_ptr,
                                           B, H, Sq, Sk, D, *vs, *cs, int(bool(causal)), int(bool(zero_padding)),
                                           _lib.dtype_tag(p, "attn_pv"), _lib.stream_of(p)), "attn_pv")
+    return out
+
+
+def attn_fused(q, k, v, seq_len_list, *, scale: Optional[float] = None, causal: bool = True, q_len_list=None,
+               out: Optional[torch.Tensor] = None):
+    """ctx = softmax(scale * q k^T, mask) v in one kernel; the score tensor is never materialised.
+
+    Same masking rule as ``scale_mask_softmax`` (``causal``, key lengths, optional query lengths);
+    ``scale`` defaults to ``size_per_head ** -0.5``.  fp16 / bf16 only.  Returns ``[B,H,Sq,D]``; rows of
+    padded queries are left uninitialised.
+    """
+    qs = _bhsd(q, "q")
+    ks = _bhsd(k, "k")
+    vs = _bhsd(v, "v")
+    B, H, Sq, D = q.shape
+    Sk = k.shape[2]
+    if k.shape != (B, H, Sk, D) or v.shape != (B, H, Sk, D) or k.dtype != q.dtype or v.dtype != q.dtype:
+        raise RuntimeError("attn_fused: q, k, v disagree in batch, heads, size_per_head, key length or dtype")
+    if q.dtype not in (torch.float16, torch.bfloat16):
+        raise RuntimeError("attn_fused: Datatype not implemented (float16 and bfloat16 only)")
+    k_info, q_ptr = _lens_ptrs(seq_len_list, q_len_list, B, q.device)
+    if out is None:
+        out = torch.empty((B, H, Sq, D), dtype=q.dtype, device=q.device)
+    else:
+        _bhsd(out, "out")
+        if out.shape != (B, H, Sq, D) or out.dtype != q.dtype:
+            raise RuntimeError("attn_fused: out must be [B,H,Sq,D] of q's dtype")
+    cs = (out.stride(0), out.stride(1), out.stride(2))
+    arr = ctypes.c_int64 * 3
+    scale = float(D) ** -0.5 if scale is None else float(scale)
+    with _lib.device_guard(q):
+        _lib.check(_lib.fn.en_attn_fused(q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(),
+                                         k_info.lens.data_ptr(), q_ptr, B, H, Sq, Sk, D, arr(*qs), arr(*ks), arr(*vs),
+                                         arr(*cs), scale, int(bool(causal)), _lib.dtype_tag(q, "attn_fused"),
+                                         _lib.stream_of(q)), "attn_fused")
     return out
 
 

@@ -16,7 +16,7 @@ from typing import Dict, Optional
 
 import torch
 
-from .kernel import (attn_pv, attn_qk, decode_pv, decode_qk, depad, layer_norm_forward, scale_mask_softmax,
+from .kernel import (attn_fused, attn_pv, attn_qk, decode_pv, decode_qk, depad, layer_norm_forward, scale_mask_softmax,
                      transpose_depad, transpose_pad)
 from .seqinfo import SeqInfo, seq_info
 
@@ -29,11 +29,13 @@ def padding_removal_layer(hidden_padded: torch.Tensor, qkv_packed: torch.Tensor,
                           size_per_head: int, gamma: torch.Tensor, beta: torch.Tensor, eps: float = 1e-5,
                           scale: Optional[float] = None, causal: bool = True, left_padded: bool = False,
                           dense_out: Optional[torch.Tensor] = None, sum_seq: Optional[int] = None,
-                          keep: bool = False):
+                          keep: bool = False, fused_attention: bool = False):
     """Runs the seven ops on ``hidden_padded`` [B,S,hid] and ``qkv_packed`` [1,T,H,3D].
 
     Returns the normalised ``[1,T,hid]`` output, or a dict of every
-    intermediate when ``keep`` is set.
+    intermediate when ``keep`` is set.  ``fused_attention`` replaces the three
+    ops QK^T / scale_mask_softmax / PV by the single fused kernel (16-bit dtypes
+    only); the score tensor is then never written.
     """
     B, S, hid = hidden_padded.shape
     H, D = head_num, size_per_head
@@ -44,9 +46,13 @@ def padding_removal_layer(hidden_padded: torch.Tensor, qkv_packed: torch.Tensor,
     x = depad(hidden_padded, B, info, left_padded=left_padded, sum_seq=T)
     qkv = transpose_pad(qkv_packed, B, S, info, H, 3 * D)
     q, k, v = torch.chunk(qkv, 3, dim=-1)
-    scores = attn_qk(q, k, info, causal=causal)
-    probs = scale_mask_softmax(B, S, H, scores, info, scale=scale, causal=causal, tail_rows=PV_QUERY_TILE)
-    ctx = attn_pv(probs, v, info, causal=causal)
+    if fused_attention:
+        probs = None
+        ctx = attn_fused(q, k, v, info, scale=scale, causal=causal)
+    else:
+        scores = attn_qk(q, k, info, causal=causal)
+        probs = scale_mask_softmax(B, S, H, scores, info, scale=scale, causal=causal, tail_rows=PV_QUERY_TILE)
+        ctx = attn_pv(probs, v, info, causal=causal)
     ctx_packed = transpose_depad(ctx, B, T, S, info, H, D)
     attn_out = ctx_packed.view(1, T, H * D) if dense_out is None else dense_out
     y = layer_norm_forward(attn_out, gamma, beta, (hid,), eps, residual=x)

@@ -171,6 +171,18 @@ int en_decode_pv(const void *p, const void *v_cache, void *ctx, const int32_t *k
                  int k_seq_len, int size_per_head, int64_t v_stride_b, int64_t v_stride_h, int64_t v_stride_s,
                  int dtype, en_stream_t stream);
 
+/* Fused attention (an addition: the reference callers run matmul, softmax, matmul,
+ * examples/bert/bert.py:108-119): ctx[b,h,i,:] = sum_j softmax_j(scale * <q_i, k_j>) v[b,h,j,:]
+ * over the keys row i may see (same rule as en_scale_mask_softmax), without ever
+ * writing the [B,H,Sq,Sk] scores to memory.  q, k, v, ctx are addressed as
+ * base + b*strides[0] + h*strides[1] + s*strides[2] + d (elements; each *_strides
+ * points to three int64 in host memory).  Rows i >= q_lens[b] of ctx are left
+ * untouched.  fp16 / bf16, fp32 accumulation and statistics; D a multiple of 8, D <= 128. */
+int en_attn_fused(const void *q, const void *k, const void *v, void *ctx, const int32_t *k_lens,
+                  const int32_t *q_lens, int batch, int head_num, int q_seq_len, int k_seq_len, int size_per_head,
+                  const int64_t *q_strides, const int64_t *k_strides, const int64_t *v_strides,
+                  const int64_t *c_strides, float scale, int causal, int dtype, en_stream_t stream);
+
 /* ---- measurement helper ------------------------------------------------- */
 
 /* Plain device-to-device copy of nbytes (multiple of 16, 16-byte aligned) with

@@ -153,3 +153,56 @@ def test_decode_qk_pv(dtype, B, H, S, D, kv):
     ctx = k.decode_pv(probs, vc.cuda(), kv_t).cpu()
     assert ctx.shape == (B, H, 1, D)
     assert max_abs(ctx, want_ctx) <= tol * max(1.0, float(want_ctx.abs().max()))
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("causal", [True, False])
+@pytest.mark.parametrize("B,H,S,D,lens", ATTN_CASES)
+def test_attn_fused(dtype, causal, B, H, S, D, lens):
+    """One kernel for QK^T + mask/softmax + PV against the float64 oracle of the three steps."""
+    k = _kernel()
+    announce("attn fused", dtype, causal, B, H, S, D, lens)
+    T = sum(lens)
+    qkv_packed = packed_randn(max(T, 1), H * 3 * D, dtype, 300 + S)[:T].reshape(T, H, 3 * D)
+    qkv = pad_bhsd(qkv_packed, lens, S, H, 3 * D)
+    for b, n in enumerate(lens):              # whatever sits in the padding must not matter
+        qkv[b, :, n:] = float("nan")
+    q, kk, v = torch.chunk(qkv, 3, dim=-1)
+    lens_t = torch.tensor(lens, dtype=torch.int32).cuda()
+    qg, kg, vg = torch.chunk(qkv.cuda(), 3, dim=-1)
+    scale = D ** -0.5
+    sentinel = 777.0
+    out = torch.full((B, H, S, D), sentinel, dtype=dtype, device="cuda")
+    ctx = k.attn_fused(qg, kg, vg, lens_t, scale=scale, causal=causal, out=out).cpu()
+    qz, kz, vz = (torch.nan_to_num(t, nan=0.0) for t in (q, kk, v))
+    scores = eager.attn_qk(qz, kz, torch.float64)
+    probs = eager.scale_mask_softmax(B, S, H, scores, lens, scale=scale, causal=causal, acc_dtype=torch.float64,
+                                     out_dtype=torch.float64)
+    rows_pad = torch.ones(B, H, S, dtype=torch.bool)
+    for b, n in enumerate(lens):
+        rows_pad[b, :, :n] = False
+        probs[b, :, n:] = 0
+    want = eager.attn_pv(probs, vz, torch.float64)
+    tol = {torch.float16: 2e-3, torch.bfloat16: 1.6e-2}[dtype]
+    if (~rows_pad).any():
+        err = max_abs(ctx[~rows_pad], want[~rows_pad])
+        assert err <= tol * max(1.0, float(want[~rows_pad].abs().max())), err
+    assert bool((ctx[rows_pad] == sentinel).all())
+
+
+def test_attn_fused_matches_unfused_pipeline_on_c2_shape():
+    """Same inputs through the three separate kernels and through the fused one."""
+    k = _kernel()
+    B, H, S, D = 4, 12, 512, 64
+    lens = [512, 64, 301, 97]
+    announce("attn fused vs unfused")
+    g = torch.Generator().manual_seed(77)
+    qkv = torch.randn(B, H, S, 3 * D, generator=g).half().cuda()
+    q, kk, v = torch.chunk(qkv, 3, dim=-1)
+    lens_t = torch.tensor(lens, dtype=torch.int32).cuda()
+    scores = k.attn_qk(q, kk, lens_t, causal=True)
+    probs = k.scale_mask_softmax(B, S, H, scores, lens_t, scale=D ** -0.5, causal=True, tail_rows=128)
+    ctx_a = k.attn_pv(probs, v, lens_t, causal=True)
+    ctx_b = k.attn_fused(q, kk, v, lens_t, causal=True)
+    for b, n in enumerate(lens):
+        assert max_abs(ctx_a[b, :, :n].cpu(), ctx_b[b, :, :n].cpu()) <= 3e-3

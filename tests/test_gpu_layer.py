@@ -166,3 +166,20 @@ def test_decode_layer_c5_reduced_and_full():
                                       inp["beta"].cpu(), 1e-5, residual=inp["residual"].cpu(),
                                       out_dtype=torch.float32)
     assert max_abs(got2["y"].cpu(), want2) <= 6e-3
+
+
+def test_layer_c2_fused_attention():
+    """The optional fused-attention form of the step: no fp16 score tensor, so it meets the
+    north-star tolerance against the oracle that rounds nothing but the stored context."""
+    layer, wl = _mods()
+    w = wl.BY_NAME["c2"]
+    announce("layer c2 fused")
+    inp = wl.make_inputs(w)
+    got = layer.padding_removal_layer(inp["hidden_padded"].cuda(), inp["qkv_packed"].cuda(), inp["lens"].cuda(),
+                                      w.heads, w.head_dim, inp["gamma"].cuda(), inp["beta"].cuda(), 1e-5, w.scale,
+                                      w.causal, w.left_padded, keep=True, fused_attention=True)
+    want = eager.layer_unpadded(inp["hidden_padded"], inp["qkv_packed"], inp["lens_list"], w.heads, w.head_dim,
+                                inp["gamma"], inp["beta"], 1e-5, w.scale, w.causal, w.left_padded,
+                                acc_dtype=torch.float32)
+    assert max_abs(got["ctx_packed"].cpu(), want["ctx_packed"]) <= 2e-3
+    assert max_abs(got["y"].cpu(), want["y"]) <= 6e-3
