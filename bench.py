@@ -171,6 +171,20 @@ def run_workload(torch, w, steps, warmup, want_eager=True, want_kernels=True):
         torch.cuda.synchronize()
         res["fused_attention_ms_per_step"] = (time.perf_counter() - t0) * 1e3 / steps
 
+        def step_packed():
+            return layer.padding_removal_layer(d["hidden_padded"], d["qkv_packed"], info, w.heads, w.head_dim,
+                                               d["gamma"], d["beta"], workloads.EPS, w.scale, w.causal,
+                                               w.left_padded, dense_out=d["dense_out"], sum_seq=tokens,
+                                               fused_attention="packed")
+        for _ in range(max(2, warmup // 2)):
+            step_packed()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            step_packed()
+        torch.cuda.synchronize()
+        res["packed_fused_attention_ms_per_step"] = (time.perf_counter() - t0) * 1e3 / steps
+
     # the same step replayed from a HIP graph (launch overhead removed); reported, never the headline
     try:
         g = torch.cuda.CUDAGraph()
@@ -252,6 +266,10 @@ def kernel_table(torch, K, layer, workloads, w, d, info, steps):
         if w.dtype != torch.float32:
             alg["attn_fused"] = 4 * T * H * D * torch.empty(0, dtype=w.dtype).element_size()   # q, k, v in; ctx out
             fns["attn_fused"] = lambda: K.attn_fused(q, k, v, info, scale=w.scale, causal=w.causal, out=ctx)
+            alg["attn_fused_packed"] = alg["attn_fused"]
+            ctx_pk = torch.empty(1, T, H * D, dtype=w.dtype, device="cuda")
+            fns["attn_fused_packed"] = lambda: K.attn_fused_packed(d["qkv_packed"], B, S, info, H, D, scale=w.scale,
+                                                                   causal=w.causal, out=ctx_pk)
         fns["transpose_depad"] = lambda: K.transpose_depad(ctx, B, T, S, info, H, D)
         fns["layernorm_residual"] = lambda: K.layer_norm_forward(attn_out, d["gamma"], d["beta"], (w.hidden,),
                                                                  workloads.EPS, residual=keep["x"])
@@ -263,8 +281,8 @@ def kernel_table(torch, K, layer, workloads, w, d, info, steps):
         ms = _event_time_ms(fn, steps, torch)
         row = {"us": ms * 1e3, "alg_MB": alg[name] / 1e6, "GBps": alg[name] / (ms * 1e-3) / 1e9}
         row["hbm_frac"] = row["GBps"] / HBM_PEAK_GBS
-        if name in ("attn_qk", "attn_pv", "decode_qk", "decode_pv", "attn_fused"):
-            row["TFLOPs"] = (2 if name == "attn_fused" else 1) * flops / (ms * 1e-3) / 1e12
+        if name in ("attn_qk", "attn_pv", "decode_qk", "decode_pv", "attn_fused", "attn_fused_packed"):
+            row["TFLOPs"] = (2 if name.startswith("attn_fused") else 1) * flops / (ms * 1e-3) / 1e12
             row["mfma_frac"] = row["TFLOPs"] / MFMA_PEAK_TFLOPS[dt]
         table[name] = row
     return table
@@ -375,7 +393,7 @@ def main(argv=None) -> int:
 
     # roofline of the kernel that takes the largest share of the step
     kt = head["kernels"]
-    in_step = [n for n in kt if n != "attn_fused" and (n != "scale_mask_softmax" or "scale_mask_softmax_tiled" not in kt)]
+    in_step = [n for n in kt if not n.startswith("attn_fused") and (n != "scale_mask_softmax" or "scale_mask_softmax_tiled" not in kt)]
     dom = max(in_step, key=lambda n: kt[n]["us"])
     row = kt[dom]
     roofline = {"kernel": dom, "bound": "hbm", "achieved": row["GBps"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
@@ -391,6 +409,7 @@ def main(argv=None) -> int:
         "roofline": roofline,
         "graph_ms_per_step": head.get("graph_ms_per_step"),
         "fused_attention_ms_per_step": head.get("fused_attention_ms_per_step"),
+        "packed_fused_attention_ms_per_step": head.get("packed_fused_attention_ms_per_step"),
         "eager_gpu_ms_per_step": head.get("eager_gpu_ms_per_step"),
         "speedup_vs_eager_gpu": head.get("speedup_vs_eager_gpu"),
         "kernels": kt,

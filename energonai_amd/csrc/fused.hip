@@ -1,4 +1,5 @@
-// Fused attention for the padded [B,H,S,*] layout:
+// Fused attention for the padded [B,H,S,*] layout and for the packed layout
+// (all valid tokens back to back, no padding rows anywhere):
 //
 //   ctx = softmax(scale * Q K^T, causal / key-padding mask) V
 //
@@ -32,6 +33,8 @@ struct FusedArgs {
   const void *v;
   int64_t v_sb, v_sh, v_ss;
   int64_t c_sb, c_sh, c_ss;
+  const int32_t *q_row0;     // packed layout: first row of batch b in q / ctx (else null)
+  const int32_t *k_row0;     // packed layout: first row of batch b in k / v (else null)
   float scale;
 };
 
@@ -80,10 +83,12 @@ __global__ __launch_bounds__(kBlock, 2) void attn_fused_kernel(FusedArgs fa) {
   const int q_first = q0 + wave * 32;
   const int vis_min = (q_first + 31 < ql) ? (a.causal ? min(kl, q_first + (kl - ql) + 1) : kl) : 0;
 
-  const T *qbase = reinterpret_cast<const T *>(a.a_ptr) + (int64_t)b * a.q_sb + (int64_t)h * a.q_sh;
-  const T *kbase = reinterpret_cast<const T *>(a.b_ptr) + (int64_t)b * a.k_sb + (int64_t)h * a.k_sh;
-  const T *vbase = reinterpret_cast<const T *>(fa.v) + (int64_t)b * fa.v_sb + (int64_t)h * fa.v_sh;
-  T *cbase = reinterpret_cast<T *>(a.out) + (int64_t)b * fa.c_sb + (int64_t)h * fa.c_sh;
+  // batch base: b * batch stride (padded layout) or first-row * row stride (packed layout)
+  const int64_t qr = fa.q_row0 ? fa.q_row0[b] : 0, kr = fa.k_row0 ? fa.k_row0[b] : 0;
+  const T *qbase = reinterpret_cast<const T *>(a.a_ptr) + (int64_t)b * a.q_sb + qr * a.q_ss + (int64_t)h * a.q_sh;
+  const T *kbase = reinterpret_cast<const T *>(a.b_ptr) + (int64_t)b * a.k_sb + kr * a.k_ss + (int64_t)h * a.k_sh;
+  const T *vbase = reinterpret_cast<const T *>(fa.v) + (int64_t)b * fa.v_sb + kr * fa.v_ss + (int64_t)h * fa.v_sh;
+  T *cbase = reinterpret_cast<T *>(a.out) + (int64_t)b * fa.c_sb + qr * fa.c_ss + (int64_t)h * fa.c_sh;
 
   // Q fragments (B operand of S^T = K Q^T): this lane's query row, 8 channels per step
   uint4 qf[NVS];
@@ -272,8 +277,8 @@ static int launch_fused(FusedArgs &fa, hipStream_t s) {
 extern "C" int en_attn_fused(const void *q, const void *k, const void *v, void *ctx, const int32_t *k_lens,
                              const int32_t *q_lens, int batch, int head_num, int q_seq_len, int k_seq_len,
                              int size_per_head, const int64_t *q_strides, const int64_t *k_strides,
-                             const int64_t *v_strides, const int64_t *c_strides, float scale, int causal, int dtype,
-                             en_stream_t stream) {
+                             const int64_t *v_strides, const int64_t *c_strides, const int32_t *q_row_offsets,
+                             const int32_t *k_row_offsets, float scale, int causal, int dtype, en_stream_t stream) {
   using namespace en;
   if (!q || !k || !v || !ctx || !k_lens || !q_strides || !k_strides || !v_strides || !c_strides) return EN_ERR_NULL;
   if (batch < 1 || head_num < 1 || q_seq_len < 1 || k_seq_len < 1 || size_per_head < 1) return EN_ERR_SHAPE;
@@ -301,6 +306,7 @@ extern "C" int en_attn_fused(const void *q, const void *k, const void *v, void *
   fa.v = v;
   fa.v_sb = v_strides[0]; fa.v_sh = v_strides[1]; fa.v_ss = v_strides[2];
   fa.c_sb = c_strides[0]; fa.c_sh = c_strides[1]; fa.c_ss = c_strides[2];
+  fa.q_row0 = q_row_offsets; fa.k_row0 = k_row_offsets;
   fa.scale = scale;
   hipStream_t s = (hipStream_t)stream;
   return dtype == EN_F16 ? launch_fused<EN_F16>(fa, s) : launch_fused<EN_BF16>(fa, s);

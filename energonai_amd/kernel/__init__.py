@@ -3,17 +3,19 @@
 Same names, same positional signatures; every function runs hand-written
 gfx950 kernels through the C ABI of libenergon_hip.so.  ``attn_qk`` /
 ``attn_pv`` / ``decode_qk`` / ``decode_pv`` are additions: the reference
-callers use ``torch.matmul`` for the two contractions.
+callers use ``torch.matmul`` for the two contractions.  ``attn_fused`` and
+``attn_fused_packed`` run the contractions and the softmax in one kernel.
 """
 from .cuda_native import transpose_pad, transpose_depad, depad, scale_mask_softmax
 from .cuda_native import (ft_build_padding_offsets, ft_remove_padding, ft_rebuild_padding,
                           ft_transpose_remove_padding, ft_transpose_rebuild_padding)
 from .cuda_native import linear, find_algo
 from .cuda_native import LayerNorm, layer_norm_forward
-from .attention import attn_qk, attn_pv, attn_fused, decode_qk, decode_pv
+from .attention import attn_qk, attn_pv, attn_fused, attn_fused_packed, decode_qk, decode_pv
 
 __all__ = [
     "transpose_pad", "transpose_depad", "depad", "scale_mask_softmax", "ft_build_padding_offsets",
     "ft_remove_padding", "ft_rebuild_padding", "ft_transpose_remove_padding", "ft_transpose_rebuild_padding",
-    "linear", "find_algo", "LayerNorm", "layer_norm_forward", "attn_qk", "attn_pv", "attn_fused", "decode_qk", "decode_pv",
+    "linear", "find_algo", "LayerNorm", "layer_norm_forward", "attn_qk", "attn_pv", "attn_fused",
+    "attn_fused_packed", "decode_qk", "decode_pv",
 ]

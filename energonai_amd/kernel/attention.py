@@ -123,8 +123,43 @@ def attn_fused(q, k, v, seq_len_list, *, scale: Optional[float] = None, causal: 
     with _lib.device_guard(q):
         _lib.check(_lib.fn.en_attn_fused(q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(),
                                          k_info.lens.data_ptr(), q_ptr, B, H, Sq, Sk, D, arr(*qs), arr(*ks), arr(*vs),
-                                         arr(*cs), scale, int(bool(causal)), _lib.dtype_tag(q, "attn_fused"),
-                                         _lib.stream_of(q)), "attn_fused")
+                                         arr(*cs), None, None, scale, int(bool(causal)),
+                                         _lib.dtype_tag(q, "attn_fused"), _lib.stream_of(q)), "attn_fused")
+    return out
+
+
+def attn_fused_packed(qkv, batch_size: int, max_seq_len: int, seq_len_list, head_num: int, size_per_head: int, *,
+                      scale: Optional[float] = None, causal: bool = True, out: Optional[torch.Tensor] = None):
+    """Self-attention straight on the packed projection output: ``qkv`` is ``[1,T,H,3D]`` (or ``[T,H,3D]``,
+    the layout ``transpose_pad`` is fed with in examples/bert/bert.py:100-104), the result is the packed
+    context ``[1,T,H,D]`` that ``transpose_depad`` would return (bert.py:123).  No padded tensor is built:
+    batch ``b`` is addressed at row ``cu_seqlens[b]``.  fp16 / bf16 only.
+    """
+    _lib.require_gpu(qkv, "qkv")
+    H, D = int(head_num), int(size_per_head)
+    if qkv.dtype not in (torch.float16, torch.bfloat16):
+        raise RuntimeError("attn_fused_packed: Datatype not implemented (float16 and bfloat16 only)")
+    if qkv.numel() % (3 * H * D) != 0:
+        raise RuntimeError("attn_fused_packed: qkv must be [1,T,H,3D]")
+    T = qkv.numel() // (3 * H * D)
+    info = seq_info(seq_len_list, batch_size, qkv.device)
+    if out is None:
+        out = torch.empty((1, T, H, D), dtype=qkv.dtype, device=qkv.device)
+    elif out.numel() != T * H * D or out.dtype != qkv.dtype or not out.is_contiguous():
+        raise RuntimeError("attn_fused_packed: out must be contiguous [1,T,H,D] of qkv's dtype")
+    arr = ctypes.c_int64 * 3
+    es = qkv.element_size()
+    in_strides = arr(0, 3 * D, 3 * H * D)
+    out_strides = arr(0, D, H * D)
+    base = qkv.data_ptr()
+    cu = info.cu_seqlens.data_ptr()
+    scale = float(D) ** -0.5 if scale is None else float(scale)
+    with _lib.device_guard(qkv):
+        _lib.check(_lib.fn.en_attn_fused(base, base + D * es, base + 2 * D * es, out.data_ptr(), info.lens.data_ptr(),
+                                         None, batch_size, H, int(max_seq_len), int(max_seq_len), D, in_strides,
+                                         in_strides, in_strides, out_strides, cu, cu, scale, int(bool(causal)),
+                                         _lib.dtype_tag(qkv, "attn_fused_packed"), _lib.stream_of(qkv)),
+                   "attn_fused_packed")
     return out
 
 

@@ -16,7 +16,7 @@ from typing import Dict, Optional
 
 import torch
 
-from .kernel import (attn_fused, attn_pv, attn_qk, decode_pv, decode_qk, depad, layer_norm_forward, scale_mask_softmax,
+from .kernel import (attn_fused, attn_fused_packed, attn_pv, attn_qk, decode_pv, decode_qk, depad, layer_norm_forward, scale_mask_softmax,
                      transpose_depad, transpose_pad)
 from .seqinfo import SeqInfo, seq_info
 
@@ -29,13 +29,15 @@ def padding_removal_layer(hidden_padded: torch.Tensor, qkv_packed: torch.Tensor,
                           size_per_head: int, gamma: torch.Tensor, beta: torch.Tensor, eps: float = 1e-5,
                           scale: Optional[float] = None, causal: bool = True, left_padded: bool = False,
                           dense_out: Optional[torch.Tensor] = None, sum_seq: Optional[int] = None,
-                          keep: bool = False, fused_attention: bool = False):
+                          keep: bool = False, fused_attention=False):
     """Runs the seven ops on ``hidden_padded`` [B,S,hid] and ``qkv_packed`` [1,T,H,3D].
 
     Returns the normalised ``[1,T,hid]`` output, or a dict of every
-    intermediate when ``keep`` is set.  ``fused_attention`` replaces the three
-    ops QK^T / scale_mask_softmax / PV by the single fused kernel (16-bit dtypes
-    only); the score tensor is then never written.
+    intermediate when ``keep`` is set.  ``fused_attention=True`` replaces the
+    three ops QK^T / scale_mask_softmax / PV by the single fused kernel (16-bit
+    dtypes only); the score tensor is then never written.
+    ``fused_attention="packed"`` also drops transpose_pad and transpose_depad:
+    the fused kernel reads the packed projections and writes the packed context.
     """
     B, S, hid = hidden_padded.shape
     H, D = head_num, size_per_head
@@ -44,6 +46,13 @@ def padding_removal_layer(hidden_padded: torch.Tensor, qkv_packed: torch.Tensor,
     scale = float(D) ** -0.5 if scale is None else scale
 
     x = depad(hidden_padded, B, info, left_padded=left_padded, sum_seq=T)
+    if fused_attention == "packed":
+        ctx_packed = attn_fused_packed(qkv_packed, B, S, info, H, D, scale=scale, causal=causal)
+        attn_out = ctx_packed.view(1, T, H * D) if dense_out is None else dense_out
+        y = layer_norm_forward(attn_out, gamma, beta, (hid,), eps, residual=x)
+        if keep:
+            return dict(x=x, qkv=None, probs=None, ctx=None, ctx_packed=ctx_packed, y=y)
+        return y
     qkv = transpose_pad(qkv_packed, B, S, info, H, 3 * D)
     q, k, v = torch.chunk(qkv, 3, dim=-1)
     if fused_attention:

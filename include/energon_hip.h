@@ -176,12 +176,19 @@ int en_decode_pv(const void *p, const void *v_cache, void *ctx, const int32_t *k
  * over the keys row i may see (same rule as en_scale_mask_softmax), without ever
  * writing the [B,H,Sq,Sk] scores to memory.  q, k, v, ctx are addressed as
  * base + b*strides[0] + h*strides[1] + s*strides[2] + d (elements; each *_strides
- * points to three int64 in host memory).  Rows i >= q_lens[b] of ctx are left
- * untouched.  fp16 / bf16, fp32 accumulation and statistics; D a multiple of 8, D <= 128. */
+ * points to three int64 in host memory).  Packed operands (all valid rows back
+ * to back, as in the [1,T,H,3D] projection output of examples/bert/bert.py:100)
+ * are addressed by passing q_row_offsets (for q and ctx) and/or k_row_offsets
+ * (for k and v): device arrays of batch entries, the exclusive prefix of the
+ * lengths; batch b then starts at row offsets[b] (give stride[0] = 0), so neither
+ * transpose_pad before nor transpose_depad after is needed; q_seq_len / k_seq_len
+ * are then upper bounds of the lengths.  Null offsets select the padded layout.
+ * Rows i >= q_lens[b] of ctx are left untouched.  fp16 / bf16, fp32 accumulation and statistics; D a multiple of 8, D <= 128. */
 int en_attn_fused(const void *q, const void *k, const void *v, void *ctx, const int32_t *k_lens,
                   const int32_t *q_lens, int batch, int head_num, int q_seq_len, int k_seq_len, int size_per_head,
                   const int64_t *q_strides, const int64_t *k_strides, const int64_t *v_strides,
-                  const int64_t *c_strides, float scale, int causal, int dtype, en_stream_t stream);
+                  const int64_t *c_strides, const int32_t *q_row_offsets, const int32_t *k_row_offsets, float scale,
+                  int causal, int dtype, en_stream_t stream);
 
 /* ---- measurement helper ------------------------------------------------- */
 

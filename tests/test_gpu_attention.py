@@ -190,6 +190,39 @@ def test_attn_fused(dtype, causal, B, H, S, D, lens):
     assert bool((ctx[rows_pad] == sentinel).all())
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("causal", [True, False])
+@pytest.mark.parametrize("B,H,S,D,lens", ATTN_CASES)
+def test_attn_fused_packed(dtype, causal, B, H, S, D, lens):
+    """The fused kernel addressing the packed [T,H,3D] projections and the packed [T,H*D] context
+    directly: same result as pad -> attention -> depad, with no padded tensor in between."""
+    k = _kernel()
+    announce("attn fused packed", dtype, causal, B, H, S, D, lens)
+    T = sum(lens)
+    qkv_packed = packed_randn(max(T, 1), H * 3 * D, dtype, 400 + S)[:T].reshape(T, H, 3 * D)
+    qkv = pad_bhsd(qkv_packed, lens, S, H, 3 * D)
+    q, kk, v = torch.chunk(qkv, 3, dim=-1)
+    scale = D ** -0.5
+    scores = eager.attn_qk(q, kk, torch.float64)
+    probs = eager.scale_mask_softmax(B, S, H, scores, lens, scale=scale, causal=causal, acc_dtype=torch.float64,
+                                     out_dtype=torch.float64)
+    for b, n in enumerate(lens):
+        probs[b, :, n:] = 0
+    ctx = eager.attn_pv(probs, v, torch.float64)
+    want = torch.cat([ctx[b, :, :n].permute(1, 0, 2).reshape(n, H * D) for b, n in enumerate(lens)])
+    sentinel = 555.0
+    guard = torch.full((T + 2, H * D), sentinel, dtype=dtype, device="cuda")
+    lens_t = torch.tensor(lens, dtype=torch.int64).cuda()
+    got = k.attn_fused_packed(qkv_packed.reshape(1, T, H, 3 * D).cuda(), B, S, lens_t, H, D, scale=scale,
+                              causal=causal, out=guard[1:T + 1])
+    assert got.data_ptr() == guard[1:].data_ptr()
+    g = guard.cpu()
+    tol = {torch.float16: 2e-3, torch.bfloat16: 1.6e-2}[dtype]
+    err = max_abs(g[1:T + 1], want)
+    assert err <= tol * max(1.0, float(want.abs().max())), err
+    assert bool((g[0] == sentinel).all()) and bool((g[T + 1] == sentinel).all())
+
+
 def test_attn_fused_matches_unfused_pipeline_on_c2_shape():
     """Same inputs through the three separate kernels and through the fused one."""
     k = _kernel()

@@ -168,7 +168,8 @@ def test_decode_layer_c5_reduced_and_full():
     assert max_abs(got2["y"].cpu(), want2) <= 6e-3
 
 
-def test_layer_c2_fused_attention():
+@pytest.mark.parametrize("mode", [True, "packed"])
+def test_layer_c2_fused_attention(mode):
     """The optional fused-attention form of the step: no fp16 score tensor, so it meets the
     north-star tolerance against the oracle that rounds nothing but the stored context."""
     layer, wl = _mods()
@@ -177,7 +178,7 @@ def test_layer_c2_fused_attention():
     inp = wl.make_inputs(w)
     got = layer.padding_removal_layer(inp["hidden_padded"].cuda(), inp["qkv_packed"].cuda(), inp["lens"].cuda(),
                                       w.heads, w.head_dim, inp["gamma"].cuda(), inp["beta"].cuda(), 1e-5, w.scale,
-                                      w.causal, w.left_padded, keep=True, fused_attention=True)
+                                      w.causal, w.left_padded, keep=True, fused_attention=mode)
     want = eager.layer_unpadded(inp["hidden_padded"], inp["qkv_packed"], inp["lens_list"], w.heads, w.head_dim,
                                 inp["gamma"], inp["beta"], 1e-5, w.scale, w.causal, w.left_padded,
                                 acc_dtype=torch.float32)
