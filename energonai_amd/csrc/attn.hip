@@ -163,10 +163,12 @@ __global__ __launch_bounds__(kBlock) void attn_qk_kernel(AttnArgs a) {
       const int row = v / CVEC_ROW, c = v % CVEC_ROW;
       const int q = q0 + row, k = k0 + c * EPV;
       const T *sp = &lds[row * CPITCH + c * EPV];
+      // only vectors holding a key this row may see are written: nothing downstream reads the rest
+      const int k_end = min(a.causal ? min(kl, q + (kl - ql) + 1) : kl, a.Sk);
       if constexpr (VEC) {  // rows >= ql fall outside the resource and are dropped by the bounds check
         const uint32_t off = (uint32_t)(((int64_t)q * a.Sk + k) * E::kSize);
-        buffer_store16<STREAM ? 2 : 0>(s_rsrc, (k < a.Sk) ? off : kOutOfRange, *reinterpret_cast<const uint4 *>(sp));
-      } else if (q < ql && k < a.Sk) {
+        buffer_store16<STREAM ? 2 : 0>(s_rsrc, (k < k_end) ? off : kOutOfRange, *reinterpret_cast<const uint4 *>(sp));
+      } else if (q < ql && k < k_end) {
         T *gp = sbase + (int64_t)q * a.Sk + k;
 #pragma unroll
         for (int e = 0; e < EPV; ++e)

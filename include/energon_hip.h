@@ -140,7 +140,7 @@ int en_layernorm_fwd(void *out, float *mean, float *invvar, void *sum_out, const
  * base + b*stride_b + h*stride_h + s*stride_s + d (strides in elements), so
  * the chunk views of the fused [B,H,S,3D] buffer are passed without a copy.
  * scores is contiguous [B,H,Sq,Sk].  Only entries softmax will read are
- * written: rows i < q_lens[b], columns j < visible(i) rounded up to the tile;
+ * written: rows i < q_lens[b], columns j < visible(i) rounded up to 16 bytes;
  * everything else in scores is left untouched.  q_lens NULL as above.
  * fp32 accumulation on MFMA; D a multiple of 8 (16-bit) / 4 (fp32), D <= 256. */
 int en_attn_qk(const void *q, const void *k, void *scores, const int32_t *k_lens, const int32_t *q_lens, int batch,
