@@ -22,8 +22,8 @@
 //                    (j, i) hold keys 8j + 4g + i, and the A operand simply
 //                    reads V^T at those same keys, so P never touches LDS.
 //
-// K/V tiles are fetched with bounds-checked 128-bit buffer loads one tile
-// ahead and the barriers order LDS only, as in the unfused kernels.
+// K/V tiles are fetched with bounds-checked 128-bit buffer loads ahead of use
+// and the barriers order LDS only, as in the unfused kernels.
 #include "attn_common.hip.h"
 
 namespace en {
@@ -38,6 +38,13 @@ struct FusedArgs {
   float scale;
 };
 
+// Both halves of the wave get (x of lanes 0..31, x of lanes 32..63): one VALU swap, no LDS round trip.
+__device__ __forceinline__ void halves_of(float x, float &lo, float &hi) {
+  const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+  lo = __uint_as_float(r[0]);
+  hi = __uint_as_float(r[1]);
+}
+
 template <int DT, int DP>
 __global__ __launch_bounds__(kBlock, 2) void attn_fused_kernel(FusedArgs fa) {
   static_assert(DT != EN_F32, "the fused kernel is built for 16-bit storage");
@@ -51,7 +58,8 @@ __global__ __launch_bounds__(kBlock, 2) void attn_fused_kernel(FusedArgs fa) {
   constexpr int NVS = DP / 16;                   // MFMA steps over the head dim
   constexpr int DMT = DP / 32;                   // 32-channel MFMA tiles of the output
   constexpr int KPITCH = DP + EPV;               // LDS pitch of a K row
-  constexpr int VPITCH = BK + EPV;               // LDS pitch of a V^T row
+  constexpr int VPITCH = BK + 4;                 // LDS pitch of a V^T row: 34 dwords, so the 32 rows a 64-bit
+                                                 // fragment read touches fall into 32 distinct bank pairs
   constexpr int KVEC_ROW = DP / EPV;
   constexpr int KLOADS = BK * KVEC_ROW / kBlock;
   constexpr int NQUAD = BK / 4, NCHUNK = DP / EPV;
@@ -59,8 +67,8 @@ __global__ __launch_bounds__(kBlock, 2) void attn_fused_kernel(FusedArgs fa) {
   constexpr int VLOADS = (VUNITS + kBlock - 1) / kBlock;
   constexpr float kLog2e = 1.4426950408889634f;
   static_assert(BK * KVEC_ROW % kBlock == 0, "K tile must divide over the block");
-  __shared__ __attribute__((aligned(16))) T lds_k[BK * KPITCH];
-  __shared__ __attribute__((aligned(16))) T lds_v[DP * VPITCH];
+  __shared__ __attribute__((aligned(16))) T lds_k[2][BK * KPITCH];
+  __shared__ __attribute__((aligned(16))) T lds_v[2][DP * VPITCH];
 
   int unit, qi;
   if (!map_block(a, unit, qi)) return;
@@ -102,34 +110,48 @@ __global__ __launch_bounds__(kBlock, 2) void attn_fused_kernel(FusedArgs fa) {
     }
   }
 
-  const rsrc_t k_rsrc = make_rsrc(kbase, (uint32_t)(((int64_t)(max(kl, 1) - 1) * a.k_ss + a.D) * E::kSize));
-  const rsrc_t v_rsrc = make_rsrc(vbase, (uint32_t)(((int64_t)(max(kl, 1) - 1) * fa.v_ss + a.D) * E::kSize));
+  // K / V tiles: the resources end with the last valid key, so rows past it (and whole tiles
+  // past the last one) read as zeros with no traffic and no branches.  Each lane keeps one
+  // byte offset per operand and advances it by a tile per iteration; lanes whose channel
+  // chunk lies past the head size sit at an offset that stays out of range.
+  const uint32_t k_bytes = kl > 0 ? (uint32_t)(((int64_t)(kl - 1) * a.k_ss + a.D) * E::kSize) : 0u;
+  const uint32_t v_bytes = kl > 0 ? (uint32_t)(((int64_t)(kl - 1) * fa.v_ss + a.D) * E::kSize) : 0u;
+  const rsrc_t k_rsrc = make_rsrc(kbase, k_bytes);
+  const rsrc_t v_rsrc = make_rsrc(vbase, v_bytes);
+  const uint32_t k_row_bytes = (uint32_t)(a.k_ss * E::kSize), v_row_bytes = (uint32_t)(fa.v_ss * E::kSize);
+  const int k_row = tid / KVEC_ROW, k_c = tid % KVEC_ROW;                  // vector i sits kBlock / KVEC_ROW rows lower
+  const int v_c = (tid % 4) + 4 * (tid / (4 * NQUAD)), v_kq = (tid / 4) % NQUAD;
+  uint32_t k_off = (k_c * EPV < a.D) ? k_row * k_row_bytes + k_c * EPV * E::kSize : kOutOfRange;
+  uint32_t v_off = (tid < VUNITS && v_c * EPV < a.D) ? v_kq * 4 * v_row_bytes + v_c * EPV * E::kSize : kOutOfRange;
+  static_assert(VUNITS <= kBlock, "one V unit per lane");
   uint4 kreg[KLOADS];
-  uint4 vreg[VLOADS][4];
-  auto fetch = [&](int kt) {
-    const int k0 = kt * BK;
+  uint4 vreg[4];
+  auto fetch = [&]() {
 #pragma unroll
-    for (int i = 0; i < KLOADS; ++i) {
-      const int v = tid + i * kBlock;
-      const int row = v / KVEC_ROW, c = v % KVEC_ROW;
-      const int key = k0 + row;
-      const uint32_t off = (uint32_t)(((int64_t)key * a.k_ss + c * EPV) * E::kSize);
-      kreg[i] = buffer_load16(k_rsrc, (kt < nkt && key < kl && c * EPV < a.D) ? off : kOutOfRange);
-    }
+    for (int i = 0; i < KLOADS; ++i) kreg[i] = buffer_load16(k_rsrc, k_off + i * (kBlock / KVEC_ROW) * k_row_bytes);
 #pragma unroll
-    for (int i = 0; i < VLOADS; ++i) {
-      const int u = tid + i * kBlock;
-      const int c = (u % 4) + 4 * (u / (4 * NQUAD));
-      const int kq = (u / 4) % NQUAD;
+    for (int x = 0; x < 4; ++x) vreg[x] = buffer_load16(v_rsrc, v_off + x * v_row_bytes);
+    k_off += BK * k_row_bytes;
+    v_off += BK * v_row_bytes;
+  };
+  // registers -> LDS: K as is, V transposed (four keys of one channel per 64-bit store)
+  auto stage = [&](T *kdst, T *vdst) {
 #pragma unroll
-      for (int x = 0; x < 4; ++x) {
-        const int key = k0 + kq * 4 + x;
-        const uint32_t off = (uint32_t)(((int64_t)key * fa.v_ss + c * EPV) * E::kSize);
-        vreg[i][x] = buffer_load16(v_rsrc, (kt < nkt && u < VUNITS && key < kl && c * EPV < a.D) ? off : kOutOfRange);
+    for (int i = 0; i < KLOADS; ++i)
+      *reinterpret_cast<uint4 *>(&kdst[(k_row + i * (kBlock / KVEC_ROW)) * KPITCH + k_c * EPV]) = kreg[i];
+    if (VUNITS == kBlock || tid < VUNITS) {
+      Pack<T, EPV> rows[4];
+#pragma unroll
+      for (int x = 0; x < 4; ++x) rows[x] = __builtin_bit_cast(Pack<T, EPV>, vreg[x]);
+#pragma unroll
+      for (int e = 0; e < EPV; ++e) {
+        Pack<T, 4> col;
+#pragma unroll
+        for (int x = 0; x < 4; ++x) col.v[x] = rows[x].v[e];
+        store_pack<T, 4>(&vdst[(v_c * EPV + e) * VPITCH + v_kq * 4], col);
       }
     }
   };
-  fetch(0);
 
   floatx16 o[DMT];
 #pragma unroll
@@ -139,47 +161,60 @@ __global__ __launch_bounds__(kBlock, 2) void attn_fused_kernel(FusedArgs fa) {
   float m_run = -INFINITY, l_run = 0.f;
   const float c_exp = fa.scale * kLog2e;
 
+  // Tile kt is computed out of LDS buffer kt & 1 while tile kt + 1 travels HBM -> registers ->
+  // the other buffer; one barrier per tile.
+  fetch();
+  stage(lds_k[0], lds_v[0]);
+  lds_barrier();
+
   for (int kt = 0; kt < nkt; ++kt) {
     const int k0 = kt * BK;
-    // registers -> LDS: K as is, V transposed (four keys of one channel per 64-bit store)
-#pragma unroll
-    for (int i = 0; i < KLOADS; ++i) {
-      const int v = tid + i * kBlock;
-      *reinterpret_cast<uint4 *>(&lds_k[(v / KVEC_ROW) * KPITCH + (v % KVEC_ROW) * EPV]) = kreg[i];
-    }
-#pragma unroll
-    for (int i = 0; i < VLOADS; ++i) {
-      const int u = tid + i * kBlock;
-      if (VUNITS % kBlock == 0 || u < VUNITS) {
-        const int c = (u % 4) + 4 * (u / (4 * NQUAD));
-        const int kq = (u / 4) % NQUAD;
-        Pack<T, EPV> rows[4];
-#pragma unroll
-        for (int x = 0; x < 4; ++x) rows[x] = __builtin_bit_cast(Pack<T, EPV>, vreg[i][x]);
-#pragma unroll
-        for (int e = 0; e < EPV; ++e) {
-          Pack<T, 4> col;
-#pragma unroll
-          for (int x = 0; x < 4; ++x) col.v[x] = rows[x].v[e];
-          store_pack<T, 4>(&lds_v[(c * EPV + e) * VPITCH + kq * 4], col);
-        }
-      }
-    }
-    lds_barrier();
-    fetch(kt + 1);
+    const T *ksrc = lds_k[kt & 1], *vsrc = lds_v[kt & 1];
+    fetch();
 
-    // ---- S^T = K Q^T for the tile's KB blocks of 32 keys
+    // ---- S^T = K Q^T; the K fragments are read from LDS two steps ahead of the MFMAs
     floatx16 s[KB];
 #pragma unroll
-    for (int kb = 0; kb < KB; ++kb) {
+    for (int kb = 0; kb < KB; ++kb)
 #pragma unroll
       for (int x = 0; x < 16; ++x) s[kb][x] = 0.f;
+    {
+      constexpr int NST = NVS / 2;                 // stages of two steps each
+      uint4 kf[2][2][KB];
+      auto load_stage = [&](int st, uint4 (&dst)[2][KB]) {
 #pragma unroll
-      for (int vs = 0; vs < NVS; ++vs) {
-        const uint4 kf = *reinterpret_cast<const uint4 *>(&lds_k[(kb * 32 + r) * KPITCH + M::k_of(vs, g, NVS)]);
-        M::step(kf, qf[vs], s[kb]);
+        for (int u = 0; u < 2; ++u)
+#pragma unroll
+          for (int kb = 0; kb < KB; ++kb)
+            dst[u][kb] = *reinterpret_cast<const uint4 *>(&ksrc[(kb * 32 + r) * KPITCH + M::k_of(2 * st + u, g, NVS)]);
+      };
+      load_stage(0, kf[0]);
+#pragma unroll
+      for (int st = 0; st < NST; ++st) {
+        if (st + 1 < NST) load_stage(st + 1, kf[(st + 1) & 1]);
+        __builtin_amdgcn_sched_barrier(0);         // keep the reads of the next stage ahead of these MFMAs
+#pragma unroll
+        for (int u = 0; u < 2; ++u)
+#pragma unroll
+          for (int kb = 0; kb < KB; ++kb) M::step(kf[st & 1][u][kb], qf[2 * st + u], s[kb]);
+        __builtin_amdgcn_sched_barrier(0);
       }
     }
+
+    // first V^T fragments are requested before the softmax arithmetic
+    constexpr int NG = KB * 2;                      // groups of 16 keys
+    uint4 va[2][DMT];
+    auto load_group = [&](int gi, uint4 (&dst)[DMT]) {
+      const int kk = gi * 16 + 4 * g;
+#pragma unroll
+      for (int mt = 0; mt < DMT; ++mt) {
+        const T *vrow = &vsrc[(mt * 32 + r) * VPITCH + kk];
+        const uint2 lo = *reinterpret_cast<const uint2 *>(vrow);
+        const uint2 hi = *reinterpret_cast<const uint2 *>(vrow + 8);
+        dst[mt] = make_uint4(lo.x, lo.y, hi.x, hi.y);
+      }
+    };
+    load_group(0, va[0]);
 
     // ---- mask + online softmax; register 4j+i of block kb holds key k0 + 32kb + 8j + 4g + i
     float m_tile = -INFINITY;
@@ -199,49 +234,59 @@ __global__ __launch_bounds__(kBlock, 2) void attn_fused_kernel(FusedArgs fa) {
           m_tile = fmaxf(m_tile, v);
         }
     }
-    m_tile = fmaxf(m_tile, __shfl_xor(m_tile, 32, kWave));   // the other half of this query's keys
+    {  // the other half of this query's keys sits in lane r + 32
+      float lo, hi;
+      halves_of(m_tile, lo, hi);
+      m_tile = fmaxf(lo, hi);
+    }
     const float m_new = fmaxf(m_run, m_tile);
     const float moff = (m_new == -INFINITY) ? 0.f : -m_new * c_exp;
     const float alpha = (m_run == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(fmaf(m_run, c_exp, moff));
     float l_tile = 0.f;
-    uint4 pf[KB][2];                                           // B operands of the second MFMA
+    uint4 pf[NG];                                              // B operands of the second MFMA
 #pragma unroll
     for (int kb = 0; kb < KB; ++kb) {
       Pack<T, EPV> pk[2];
 #pragma unroll
       for (int x = 0; x < 16; ++x) {
-        const float p = (s[kb][x] == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(fmaf(s[kb][x], c_exp, moff));
-        const T pt = E::from_float(p);
-        l_tile += E::to_float(pt);                             // sum what is actually multiplied
-        pk[x >> 3].v[x & 7] = pt;                              // step t = x/8 takes registers j = 2t, 2t+1
+        // exp2(-inf) is 0, so masked keys need no special case
+        const float p = __builtin_amdgcn_exp2f(fmaf(s[kb][x], c_exp, moff));
+        l_tile += p;
+        pk[x >> 3].v[x & 7] = E::from_float(p);                // group t = x/8 takes registers j = 2t, 2t+1
       }
-      pf[kb][0] = __builtin_bit_cast(uint4, pk[0]);
-      pf[kb][1] = __builtin_bit_cast(uint4, pk[1]);
+      pf[2 * kb] = __builtin_bit_cast(uint4, pk[0]);
+      pf[2 * kb + 1] = __builtin_bit_cast(uint4, pk[1]);
     }
-    l_tile += __shfl_xor(l_tile, 32, kWave);
+    {
+      float lo, hi;
+      halves_of(l_tile, lo, hi);
+      l_tile = lo + hi;
+    }
     l_run = l_run * alpha + l_tile;
+    // the running maximum settles after a few tiles; skip the rescale while no lane's maximum moved
+    if (__builtin_amdgcn_ballot_w64(m_new != m_run) != 0) {
+#pragma unroll
+      for (int mt = 0; mt < DMT; ++mt)
+#pragma unroll
+        for (int x = 0; x < 16; ++x) o[mt][x] *= alpha;
+    }
     m_run = m_new;
-#pragma unroll
-    for (int mt = 0; mt < DMT; ++mt)
-#pragma unroll
-      for (int x = 0; x < 16; ++x) o[mt][x] *= alpha;
 
     // ---- O^T += V^T P^T; the A operand reads V^T at the keys the B registers hold:
-    //      elements 0..3 <-> keys 16t + 4g + 0..3, elements 4..7 <-> keys 16t + 8 + 4g + 0..3
+    //      elements 0..3 <-> keys 16gi + 4g + 0..3, elements 4..7 <-> keys 16gi + 8 + 4g + 0..3
 #pragma unroll
-    for (int kb = 0; kb < KB; ++kb)
+    for (int gi = 0; gi < NG; ++gi) {
+      if (gi + 1 < NG) load_group(gi + 1, va[(gi + 1) & 1]);
+      __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-      for (int t = 0; t < 2; ++t) {
-        const int kk = kb * 32 + 16 * t + 4 * g;
-#pragma unroll
-        for (int mt = 0; mt < DMT; ++mt) {
-          const T *vrow = &lds_v[(mt * 32 + r) * VPITCH + kk];
-          const uint2 lo = *reinterpret_cast<const uint2 *>(vrow);
-          const uint2 hi = *reinterpret_cast<const uint2 *>(vrow + 8);
-          M::step(make_uint4(lo.x, lo.y, hi.x, hi.y), pf[kb][t], o[mt]);
-        }
-      }
-    lds_barrier();  // tiles are consumed before the next ones are written
+      for (int mt = 0; mt < DMT; ++mt) M::step(va[gi & 1][mt], pf[gi], o[mt]);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+
+    // the tile fetched during this iteration goes to the other buffer, which everyone left
+    // before the barrier that ended the previous iteration
+    stage(lds_k[(kt + 1) & 1], lds_v[(kt + 1) & 1]);
+    lds_barrier();
   }
 
   // ---- normalise and store: register 4j+i of tile mt holds channel 32mt + 8j + 4g + i of this lane's query
@@ -284,7 +329,7 @@ extern "C" int en_attn_fused(const void *q, const void *k, const void *v, void *
   if (batch < 1 || head_num < 1 || q_seq_len < 1 || k_seq_len < 1 || size_per_head < 1) return EN_ERR_SHAPE;
   if (dtype != EN_F16 && dtype != EN_BF16) return EN_ERR_DTYPE;
   if (size_per_head > 128 || (size_per_head % 8) != 0) return EN_ERR_UNSUPPORTED;
-  if (!(scale >= 0.f)) return EN_ERR_UNSUPPORTED;
+  if (!(scale > 0.f)) return EN_ERR_UNSUPPORTED;  // masked scores are -inf; -inf * 0 would not stay masked
   if ((int64_t)batch * head_num > INT32_MAX / 64) return EN_ERR_SHAPE;
   if (!aligned_to(q, 16) || !aligned_to(k, 16) || !aligned_to(v, 16) || !aligned_to(ctx, 8)) return EN_ERR_ALIGN;
   for (int i = 0; i < 3; ++i) {

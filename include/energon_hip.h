@@ -183,7 +183,7 @@ int en_decode_pv(const void *p, const void *v_cache, void *ctx, const int32_t *k
  * lengths; batch b then starts at row offsets[b] (give stride[0] = 0), so neither
  * transpose_pad before nor transpose_depad after is needed; q_seq_len / k_seq_len
  * are then upper bounds of the lengths.  Null offsets select the padded layout.
- * Rows i >= q_lens[b] of ctx are left untouched.  fp16 / bf16, fp32 accumulation and statistics; D a multiple of 8, D <= 128. */
+ * scale must be positive.  Rows i >= q_lens[b] of ctx are left untouched.  fp16 / bf16, fp32 accumulation and statistics; D a multiple of 8, D <= 128. */
 int en_attn_fused(const void *q, const void *k, const void *v, void *ctx, const int32_t *k_lens,
                   const int32_t *q_lens, int batch, int head_num, int q_seq_len, int k_seq_len, int size_per_head,
                   const int64_t *q_strides, const int64_t *k_strides, const int64_t *v_strides,
