@@ -81,15 +81,17 @@ __global__ __launch_bounds__(kBlock, 2) void attn_fused_kernel(FusedArgs fa) {
   const int nkt = (nk + BK - 1) / BK;
 
   const int tid = threadIdx.x;
-  const int lane = tid & 63, wave = tid >> 6;
+  const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int r = lane & 31, g = lane >> 5;
   const int q = q0 + wave * 32 + r;              // this lane's query row
   const bool q_valid = q < ql;
   // keys this query may see: k < vis
   const int vis = q_valid ? (a.causal ? min(kl, q + (kl - ql) + 1) : kl) : 0;
-  // smallest extent among the wave's 32 queries (wave-uniform): tiles below it need no masking
+  // smallest and largest extent among the wave's 32 queries (wave-uniform): tiles below the
+  // smallest need no masking, tiles from the largest on hold nothing for this wave
   const int q_first = q0 + wave * 32;
   const int vis_min = (q_first + 31 < ql) ? (a.causal ? min(kl, q_first + (kl - ql) + 1) : kl) : 0;
+  const int vis_max = (q_first < ql) ? (a.causal ? min(kl, min(q_first + 31, ql - 1) + (kl - ql) + 1) : kl) : 0;
 
   // batch base: b * batch stride (padded layout) or first-row * row stride (packed layout)
   const int64_t qr = fa.q_row0 ? fa.q_row0[b] : 0, kr = fa.k_row0 ? fa.k_row0[b] : 0;
@@ -160,6 +162,11 @@ __global__ __launch_bounds__(kBlock, 2) void attn_fused_kernel(FusedArgs fa) {
     for (int x = 0; x < 16; ++x) o[mt][x] = 0.f;
   float m_run = -INFINITY, l_run = 0.f;
   const float c_exp = fa.scale * kLog2e;
+  // The running maximum is only moved (and the accumulators rescaled) when some query's new
+  // maximum exceeds it by more than 2^8 after scaling: until then probabilities are formed
+  // against the older, slightly smaller maximum and stay below 2^8, well inside the 16-bit
+  // range, and the final division by the row sum cancels the common factor.
+  const float lazy_gap = 8.0f / c_exp;
 
   // Tile kt is computed out of LDS buffer kt & 1 while tile kt + 1 travels HBM -> registers ->
   // the other buffer; one barrier per tile.
@@ -172,115 +179,117 @@ __global__ __launch_bounds__(kBlock, 2) void attn_fused_kernel(FusedArgs fa) {
     const T *ksrc = lds_k[kt & 1], *vsrc = lds_v[kt & 1];
     fetch();
 
-    // ---- S^T = K Q^T; the K fragments are read from LDS two steps ahead of the MFMAs
-    floatx16 s[KB];
+    if (k0 < vis_max) {  // wave-uniform: later tiles are masked for all of this wave's queries
+      // ---- S^T = K Q^T; the K fragments are read from LDS two steps ahead of the MFMAs
+      floatx16 s[KB];
 #pragma unroll
-    for (int kb = 0; kb < KB; ++kb)
+      for (int kb = 0; kb < KB; ++kb)
 #pragma unroll
-      for (int x = 0; x < 16; ++x) s[kb][x] = 0.f;
-    {
-      constexpr int NST = NVS / 2;                 // stages of two steps each
-      uint4 kf[2][2][KB];
-      auto load_stage = [&](int st, uint4 (&dst)[2][KB]) {
+        for (int x = 0; x < 16; ++x) s[kb][x] = 0.f;
+      {
+        constexpr int NST = NVS / 2;                 // stages of two steps each
+        uint4 kf[2][2][KB];
+        auto load_stage = [&](int st, uint4 (&dst)[2][KB]) {
 #pragma unroll
-        for (int u = 0; u < 2; ++u)
+          for (int u = 0; u < 2; ++u)
 #pragma unroll
-          for (int kb = 0; kb < KB; ++kb)
-            dst[u][kb] = *reinterpret_cast<const uint4 *>(&ksrc[(kb * 32 + r) * KPITCH + M::k_of(2 * st + u, g, NVS)]);
+            for (int kb = 0; kb < KB; ++kb)
+              dst[u][kb] = *reinterpret_cast<const uint4 *>(&ksrc[(kb * 32 + r) * KPITCH + M::k_of(2 * st + u, g, NVS)]);
+        };
+        load_stage(0, kf[0]);
+#pragma unroll
+        for (int st = 0; st < NST; ++st) {
+          if (st + 1 < NST) load_stage(st + 1, kf[(st + 1) & 1]);
+          __builtin_amdgcn_sched_barrier(0);         // keep the reads of the next stage ahead of these MFMAs
+#pragma unroll
+          for (int u = 0; u < 2; ++u)
+#pragma unroll
+            for (int kb = 0; kb < KB; ++kb) M::step(kf[st & 1][u][kb], qf[2 * st + u], s[kb]);
+          __builtin_amdgcn_sched_barrier(0);
+        }
+      }
+
+      // first V^T fragments are requested before the softmax arithmetic
+      constexpr int NG = KB * 2;                      // groups of 16 keys
+      uint4 va[2][DMT];
+      auto load_group = [&](int gi, uint4 (&dst)[DMT]) {
+        const int kk = gi * 16 + 4 * g;
+#pragma unroll
+        for (int mt = 0; mt < DMT; ++mt) {
+          const T *vrow = &vsrc[(mt * 32 + r) * VPITCH + kk];
+          const uint2 lo = *reinterpret_cast<const uint2 *>(vrow);
+          const uint2 hi = *reinterpret_cast<const uint2 *>(vrow + 8);
+          dst[mt] = make_uint4(lo.x, lo.y, hi.x, hi.y);
+        }
       };
-      load_stage(0, kf[0]);
-#pragma unroll
-      for (int st = 0; st < NST; ++st) {
-        if (st + 1 < NST) load_stage(st + 1, kf[(st + 1) & 1]);
-        __builtin_amdgcn_sched_barrier(0);         // keep the reads of the next stage ahead of these MFMAs
-#pragma unroll
-        for (int u = 0; u < 2; ++u)
-#pragma unroll
-          for (int kb = 0; kb < KB; ++kb) M::step(kf[st & 1][u][kb], qf[2 * st + u], s[kb]);
-        __builtin_amdgcn_sched_barrier(0);
-      }
-    }
+      load_group(0, va[0]);
 
-    // first V^T fragments are requested before the softmax arithmetic
-    constexpr int NG = KB * 2;                      // groups of 16 keys
-    uint4 va[2][DMT];
-    auto load_group = [&](int gi, uint4 (&dst)[DMT]) {
-      const int kk = gi * 16 + 4 * g;
+      // ---- mask + online softmax; register 4j+i of block kb holds key k0 + 32kb + 8j + 4g + i
+      float m_tile = -INFINITY;
+      if (k0 + BK <= vis_min) {  // whole tile visible to every query of this wave: no masking work
 #pragma unroll
-      for (int mt = 0; mt < DMT; ++mt) {
-        const T *vrow = &vsrc[(mt * 32 + r) * VPITCH + kk];
-        const uint2 lo = *reinterpret_cast<const uint2 *>(vrow);
-        const uint2 hi = *reinterpret_cast<const uint2 *>(vrow + 8);
-        dst[mt] = make_uint4(lo.x, lo.y, hi.x, hi.y);
+        for (int kb = 0; kb < KB; ++kb)
+#pragma unroll
+          for (int x = 0; x < 16; ++x) m_tile = fmaxf(m_tile, s[kb][x]);
+      } else {
+        const int lim = vis - k0 - 4 * g;      // register (kb, x) is visible iff 32kb + 8(x/4) + x%4 < lim
+#pragma unroll
+        for (int kb = 0; kb < KB; ++kb)
+#pragma unroll
+          for (int x = 0; x < 16; ++x) {
+            const float v = (kb * 32 + 8 * (x >> 2) + (x & 3) < lim) ? s[kb][x] : -INFINITY;
+            s[kb][x] = v;
+            m_tile = fmaxf(m_tile, v);
+          }
       }
-    };
-    load_group(0, va[0]);
-
-    // ---- mask + online softmax; register 4j+i of block kb holds key k0 + 32kb + 8j + 4g + i
-    float m_tile = -INFINITY;
-    if (k0 + BK <= vis_min) {  // whole tile visible to every query of this wave: no masking work
+      {  // the other half of this query's keys sits in lane r + 32
+        float lo, hi;
+        halves_of(m_tile, lo, hi);
+        m_tile = fmaxf(lo, hi);
+      }
+      if (__builtin_amdgcn_ballot_w64(m_tile > m_run + lazy_gap) != 0) {   // -inf + gap stays -inf: the first tile moves it
+        const float m_new = fmaxf(m_run, m_tile);
+        const float alpha = (m_run == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f((m_run - m_new) * c_exp);
+        l_run *= alpha;
 #pragma unroll
-      for (int kb = 0; kb < KB; ++kb)
+        for (int mt = 0; mt < DMT; ++mt)
 #pragma unroll
-        for (int x = 0; x < 16; ++x) m_tile = fmaxf(m_tile, s[kb][x]);
-    } else {
+          for (int x = 0; x < 16; ++x) o[mt][x] *= alpha;
+        m_run = m_new;
+      }
+      const float moff = (m_run == -INFINITY) ? 0.f : -m_run * c_exp;
+      float l_tile = 0.f;
+      uint4 pf[NG];                                              // B operands of the second MFMA
 #pragma unroll
-      for (int kb = 0; kb < KB; ++kb)
+      for (int kb = 0; kb < KB; ++kb) {
+        Pack<T, EPV> pk[2];
 #pragma unroll
         for (int x = 0; x < 16; ++x) {
-          const int key = k0 + kb * 32 + 8 * (x >> 2) + 4 * g + (x & 3);
-          const float v = (key < vis) ? s[kb][x] : -INFINITY;
-          s[kb][x] = v;
-          m_tile = fmaxf(m_tile, v);
+          // exp2(-inf) is 0, so masked keys need no special case
+          const float p = __builtin_amdgcn_exp2f(fmaf(s[kb][x], c_exp, moff));
+          l_tile += p;
+          pk[x >> 3].v[x & 7] = E::from_float(p);                // group t = x/8 takes registers j = 2t, 2t+1
         }
-    }
-    {  // the other half of this query's keys sits in lane r + 32
-      float lo, hi;
-      halves_of(m_tile, lo, hi);
-      m_tile = fmaxf(lo, hi);
-    }
-    const float m_new = fmaxf(m_run, m_tile);
-    const float moff = (m_new == -INFINITY) ? 0.f : -m_new * c_exp;
-    const float alpha = (m_run == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(fmaf(m_run, c_exp, moff));
-    float l_tile = 0.f;
-    uint4 pf[NG];                                              // B operands of the second MFMA
-#pragma unroll
-    for (int kb = 0; kb < KB; ++kb) {
-      Pack<T, EPV> pk[2];
-#pragma unroll
-      for (int x = 0; x < 16; ++x) {
-        // exp2(-inf) is 0, so masked keys need no special case
-        const float p = __builtin_amdgcn_exp2f(fmaf(s[kb][x], c_exp, moff));
-        l_tile += p;
-        pk[x >> 3].v[x & 7] = E::from_float(p);                // group t = x/8 takes registers j = 2t, 2t+1
+        pf[2 * kb] = __builtin_bit_cast(uint4, pk[0]);
+        pf[2 * kb + 1] = __builtin_bit_cast(uint4, pk[1]);
       }
-      pf[2 * kb] = __builtin_bit_cast(uint4, pk[0]);
-      pf[2 * kb + 1] = __builtin_bit_cast(uint4, pk[1]);
-    }
-    {
-      float lo, hi;
-      halves_of(l_tile, lo, hi);
-      l_tile = lo + hi;
-    }
-    l_run = l_run * alpha + l_tile;
-    // the running maximum settles after a few tiles; skip the rescale while no lane's maximum moved
-    if (__builtin_amdgcn_ballot_w64(m_new != m_run) != 0) {
-#pragma unroll
-      for (int mt = 0; mt < DMT; ++mt)
-#pragma unroll
-        for (int x = 0; x < 16; ++x) o[mt][x] *= alpha;
-    }
-    m_run = m_new;
+      {
+        float lo, hi;
+        halves_of(l_tile, lo, hi);
+        l_tile = lo + hi;
+      }
+      l_run += l_tile;
 
-    // ---- O^T += V^T P^T; the A operand reads V^T at the keys the B registers hold:
-    //      elements 0..3 <-> keys 16gi + 4g + 0..3, elements 4..7 <-> keys 16gi + 8 + 4g + 0..3
+      // ---- O^T += V^T P^T; the A operand reads V^T at the keys the B registers hold:
+      //      elements 0..3 <-> keys 16gi + 4g + 0..3, elements 4..7 <-> keys 16gi + 8 + 4g + 0..3
 #pragma unroll
-    for (int gi = 0; gi < NG; ++gi) {
-      if (gi + 1 < NG) load_group(gi + 1, va[(gi + 1) & 1]);
-      __builtin_amdgcn_sched_barrier(0);
+      for (int gi = 0; gi < NG; ++gi) {
+        if (gi + 1 < NG) load_group(gi + 1, va[(gi + 1) & 1]);
+        __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-      for (int mt = 0; mt < DMT; ++mt) M::step(va[gi & 1][mt], pf[gi], o[mt]);
-      __builtin_amdgcn_sched_barrier(0);
+        for (int mt = 0; mt < DMT; ++mt) M::step(va[gi & 1][mt], pf[gi], o[mt]);
+        __builtin_amdgcn_sched_barrier(0);
+      }
     }
 
     // the tile fetched during this iteration goes to the other buffer, which everyone left

@@ -223,6 +223,30 @@ def test_attn_fused_packed(dtype, causal, B, H, S, D, lens):
     assert bool((g[0] == sentinel).all()) and bool((g[T + 1] == sentinel).all())
 
 
+@pytest.mark.parametrize("slope", [0.002, 0.02, 0.3])
+def test_attn_fused_growing_maximum(slope):
+    """Scores that rise with the key index: the running maximum keeps moving, slowly (the kernel
+    may keep an older maximum for a while) or by large steps (it must rescale every tile)."""
+    k = _kernel()
+    B, H, S, D = 2, 2, 512, 64
+    lens = [512, 333]
+    announce("attn fused growing max", slope)
+    g = torch.Generator().manual_seed(5)
+    q = (1.0 + 0.1 * torch.randn(B, H, S, D, generator=g)).half()
+    ramp = (slope * torch.arange(S, dtype=torch.float32)).view(1, 1, S, 1)
+    kk = (ramp * (1.0 + 0.05 * torch.randn(B, H, S, D, generator=g))).half()
+    v = torch.randn(B, H, S, D, generator=g).half()
+    lens_t = torch.tensor(lens, dtype=torch.int32).cuda()
+    for causal in (True, False):
+        ctx = k.attn_fused(q.cuda(), kk.cuda(), v.cuda(), lens_t, scale=D ** -0.5, causal=causal).cpu()
+        scores = eager.attn_qk(q, kk, torch.float64)
+        probs = eager.scale_mask_softmax(B, S, H, scores, lens, scale=D ** -0.5, causal=causal,
+                                         acc_dtype=torch.float64, out_dtype=torch.float64)
+        want = eager.attn_pv(probs, v, torch.float64)
+        for b, n in enumerate(lens):
+            assert max_abs(ctx[b, :, :n], want[b, :, :n]) <= 2e-3 * max(1.0, float(want[b, :, :n].abs().max()))
+
+
 def test_attn_fused_matches_unfused_pipeline_on_c2_shape():
     """Same inputs through the three separate kernels and through the fused one."""
     k = _kernel()
