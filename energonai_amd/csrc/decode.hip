@@ -149,7 +149,71 @@ static int check_decode(const void *x, const void *kv, const void *out, const in
 
 }  // namespace en
 
+namespace en {
+
+// Appends one new K row and one new V row per (batch, head) to the caches at position
+// kv_lens[b]; sequences whose cache is full are left alone.  Bytes are moved as they are.
+struct AppendArgs {
+  const unsigned char *k_new, *v_new;
+  unsigned char *k_cache, *v_cache;
+  const int32_t *kv_lens;
+  int H, Sk;
+  int row_bytes;
+  int64_t n_sb, n_sh;           // strides of the new rows, bytes
+  int64_t c_sb, c_sh, c_ss;     // strides of the caches, bytes
+};
+
+template <typename Vec>
+__global__ __launch_bounds__(kWave) void kv_append_kernel(AppendArgs a) {
+  const int h = blockIdx.x, b = blockIdx.y;
+  const int pos = a.kv_lens[b];
+  if (pos < 0 || pos >= a.Sk) return;
+  const int64_t src = (int64_t)b * a.n_sb + (int64_t)h * a.n_sh;
+  const int64_t dst = (int64_t)b * a.c_sb + (int64_t)h * a.c_sh + (int64_t)pos * a.c_ss;
+  for (int i = threadIdx.x * (int)sizeof(Vec); i < a.row_bytes; i += kWave * (int)sizeof(Vec)) {
+    *reinterpret_cast<Vec *>(a.k_cache + dst + i) = *reinterpret_cast<const Vec *>(a.k_new + src + i);
+    *reinterpret_cast<Vec *>(a.v_cache + dst + i) = *reinterpret_cast<const Vec *>(a.v_new + src + i);
+  }
+}
+
+}  // namespace en
+
 extern "C" {
+
+int en_kv_append(const void *k_new, const void *v_new, void *k_cache, void *v_cache, const int32_t *kv_lens,
+                 int batch, int head_num, int k_seq_len, int size_per_head, int64_t new_stride_b,
+                 int64_t new_stride_h, int64_t cache_stride_b, int64_t cache_stride_h, int64_t cache_stride_s,
+                 int elem_size, en_stream_t stream) {
+  using namespace en;
+  if (!k_new || !v_new || !k_cache || !v_cache || !kv_lens) return EN_ERR_NULL;
+  if (elem_size != 2 && elem_size != 4) return EN_ERR_DTYPE;
+  if (batch < 1 || head_num < 1 || k_seq_len < 1 || size_per_head < 1) return EN_ERR_SHAPE;
+  if (batch > 65535) return EN_ERR_SHAPE;
+  if (new_stride_b < 0 || new_stride_h < 0 || cache_stride_b < 0 || cache_stride_h < 0 || cache_stride_s < 0)
+    return EN_ERR_UNSUPPORTED;
+  AppendArgs a{(const unsigned char *)k_new, (const unsigned char *)v_new, (unsigned char *)k_cache,
+               (unsigned char *)v_cache, kv_lens, head_num, k_seq_len, size_per_head * elem_size,
+               new_stride_b * elem_size, new_stride_h * elem_size, cache_stride_b * elem_size,
+               cache_stride_h * elem_size, cache_stride_s * elem_size};
+  const dim3 grid((unsigned)head_num, (unsigned)batch, 1);
+  hipStream_t s = (hipStream_t)stream;
+  const bool v16 = (a.row_bytes % 16 == 0) && aligned_to(k_new, 16) && aligned_to(v_new, 16) &&
+                   aligned_to(k_cache, 16) && aligned_to(v_cache, 16) && a.n_sb % 16 == 0 && a.n_sh % 16 == 0 &&
+                   a.c_sb % 16 == 0 && a.c_sh % 16 == 0 && a.c_ss % 16 == 0;
+  if (v16) {
+    kv_append_kernel<uint4><<<grid, kWave, 0, s>>>(a);
+  } else if (elem_size == 4) {
+    if (!aligned_to(k_new, 4) || !aligned_to(v_new, 4) || !aligned_to(k_cache, 4) || !aligned_to(v_cache, 4))
+      return EN_ERR_ALIGN;
+    kv_append_kernel<uint32_t><<<grid, kWave, 0, s>>>(a);
+  } else {
+    if (!aligned_to(k_new, 2) || !aligned_to(v_new, 2) || !aligned_to(k_cache, 2) || !aligned_to(v_cache, 2))
+      return EN_ERR_ALIGN;
+    kv_append_kernel<uint16_t><<<grid, kWave, 0, s>>>(a);
+  }
+  EN_RETURN_IF_LAUNCH_FAILED();
+  return EN_OK;
+}
 
 int en_decode_qk(const void *q, const void *k_cache, void *scores, const int32_t *kv_lens, int batch, int head_num,
                  int k_seq_len, int size_per_head, int64_t k_stride_b, int64_t k_stride_h, int64_t k_stride_s,

@@ -31,9 +31,11 @@ struct Ptrs3 {
 
 // transpose_pad: grid.x = head + H * s_tile (heads fastest so that blocks in
 // flight together read neighbouring pieces of the same packed token rows).
+// The packed source may hold more head rows per token than are moved (Hs >= H rows, of
+// which rows h0..h0+H-1 are taken): one third of a fused projection output, say.
 struct PadMap {
   const int32_t *cu;
-  int H, S, R;
+  int H, S, R, Hs, h0;
   __device__ bool active(int, int) const { return true; }
   __device__ void operator()(int tx, int b, int r, int64_t &src, int64_t &dst) const {
     const int h = tx % H;
@@ -41,7 +43,7 @@ struct PadMap {
     const int start = cu[b];
     const int len = cu[b + 1] - start;
     dst = (s < S) ? ((int64_t)b * H + h) * S + s : kSkipRow;
-    src = (s < len) ? ((int64_t)(start + s)) * H + h : kZeroRow;
+    src = (s < len) ? ((int64_t)(start + s)) * Hs + h0 + h : kZeroRow;
   }
 };
 
@@ -71,6 +73,21 @@ struct DepadRowsMap {
     const int len = cu[b + 1] - start;
     src = (int64_t)b * S + s + (left ? S - len : 0);
     dst = (s < len) ? (int64_t)start + s : kSkipRow;
+  }
+};
+
+// repad: inverse of depad; every row of the padded output is written (copy or zeros).
+struct RepadRowsMap {
+  const int32_t *cu;
+  int S, R, left;
+  __device__ bool active(int, int) const { return true; }
+  __device__ void operator()(int tx, int b, int r, int64_t &src, int64_t &dst) const {
+    const int s = tx * R + r;
+    const int start = cu[b];
+    const int len = cu[b + 1] - start;
+    const int i = s - (left ? S - len : 0);     // position inside the sequence
+    dst = (s < S) ? (int64_t)b * S + s : kSkipRow;
+    src = (i >= 0 && i < len) ? (int64_t)start + i : kZeroRow;
   }
 };
 
@@ -326,18 +343,40 @@ int en_depad(const void *src, void *dst, const int32_t *cu_seqlens, int batch, i
   }, (hipStream_t)stream);
 }
 
-int en_transpose_pad(const void *src, void *dst, const int32_t *cu_seqlens, int batch, int max_seq_len, int head_num,
-                     int size_per_head, int elem_size, en_stream_t stream) {
+int en_repad(const void *src, void *dst, const int32_t *cu_seqlens, int batch, int max_seq_len, int64_t hidden,
+             int elem_size, int left_padded, en_stream_t stream) {
+  if (!src || !dst || !cu_seqlens) return EN_ERR_NULL;
+  if (check_elem(elem_size)) return EN_ERR_DTYPE;
+  if (batch < 1 || max_seq_len < 1 || hidden < 1) return EN_ERR_SHAPE;
+  if (!aligned_to(src, elem_size) || !aligned_to(dst, elem_size)) return EN_ERR_ALIGN;
+  Ptrs3 p = {{src, nullptr, nullptr}, {dst, nullptr, nullptr}};
+  return launch_row_gather<RepadRowsMap, 1>(hidden * elem_size, max_seq_len,
+                                            (int64_t)batch * max_seq_len * hidden * elem_size, p, [&](int R, dim3 &grid) {
+    grid = dim3((unsigned)ceil_div(max_seq_len, R), (unsigned)batch, 1);
+    return RepadRowsMap{cu_seqlens, max_seq_len, R, left_padded ? 1 : 0};
+  }, (hipStream_t)stream);
+}
+
+int en_transpose_pad_heads(const void *src, void *dst, const int32_t *cu_seqlens, int batch, int max_seq_len,
+                           int head_num, int size_per_head, int src_head_rows, int src_head_first, int elem_size,
+                           en_stream_t stream) {
   if (!src || !dst || !cu_seqlens) return EN_ERR_NULL;
   if (check_elem(elem_size)) return EN_ERR_DTYPE;
   if (batch < 1 || max_seq_len < 1 || head_num < 1 || size_per_head < 1) return EN_ERR_SHAPE;
+  if (src_head_first < 0 || src_head_rows < src_head_first + head_num) return EN_ERR_SHAPE;
   if (!aligned_to(src, elem_size) || !aligned_to(dst, elem_size)) return EN_ERR_ALIGN;
   Ptrs3 p = {{src, nullptr, nullptr}, {dst, nullptr, nullptr}};
   return launch_row_gather<PadMap, 1>((int64_t)size_per_head * elem_size, max_seq_len,
                                       (int64_t)batch * max_seq_len * head_num * size_per_head * elem_size, p, [&](int R, dim3 &grid) {
     grid = dim3((unsigned)(ceil_div(max_seq_len, R) * head_num), (unsigned)batch, 1);
-    return PadMap{cu_seqlens, head_num, max_seq_len, R};
+    return PadMap{cu_seqlens, head_num, max_seq_len, R, src_head_rows, src_head_first};
   }, (hipStream_t)stream);
+}
+
+int en_transpose_pad(const void *src, void *dst, const int32_t *cu_seqlens, int batch, int max_seq_len, int head_num,
+                     int size_per_head, int elem_size, en_stream_t stream) {
+  return en_transpose_pad_heads(src, dst, cu_seqlens, batch, max_seq_len, head_num, size_per_head, head_num, 0,
+                                elem_size, stream);
 }
 
 int en_transpose_depad(const void *src, void *dst, const int32_t *cu_seqlens, int batch, int max_seq_len,

@@ -6,16 +6,17 @@ gfx950 kernels through the C ABI of libenergon_hip.so.  ``attn_qk`` /
 callers use ``torch.matmul`` for the two contractions.  ``attn_fused`` and
 ``attn_fused_packed`` run the contractions and the softmax in one kernel.
 """
-from .cuda_native import transpose_pad, transpose_depad, depad, scale_mask_softmax
+from .cuda_native import transpose_pad, transpose_depad, depad, repad, scale_mask_softmax
 from .cuda_native import (ft_build_padding_offsets, ft_remove_padding, ft_rebuild_padding,
                           ft_transpose_remove_padding, ft_transpose_rebuild_padding)
 from .cuda_native import linear, find_algo
 from .cuda_native import LayerNorm, layer_norm_forward
-from .attention import attn_qk, attn_pv, attn_fused, attn_fused_packed, decode_qk, decode_pv
+from .attention import (attn_qk, attn_pv, attn_fused, attn_fused_packed, attn_fused_varlen, decode_qk, decode_pv,
+                        kv_cache_fill, kv_cache_append)
 
 __all__ = [
     "transpose_pad", "transpose_depad", "depad", "scale_mask_softmax", "ft_build_padding_offsets",
     "ft_remove_padding", "ft_rebuild_padding", "ft_transpose_remove_padding", "ft_transpose_rebuild_padding",
     "linear", "find_algo", "LayerNorm", "layer_norm_forward", "attn_qk", "attn_pv", "attn_fused",
-    "attn_fused_packed", "decode_qk", "decode_pv",
+    "attn_fused_packed", "attn_fused_varlen", "decode_qk", "decode_pv", "kv_cache_fill", "kv_cache_append", "repad",
 ]

@@ -128,39 +128,93 @@ def attn_fused(q, k, v, seq_len_list, *, scale: Optional[float] = None, causal: 
     return out
 
 
+def _thd(t: torch.Tensor, name: str):
+    _lib.require_gpu(t, name, contiguous=False)
+    if t.dim() != 3 or t.stride(2) != 1:
+        raise RuntimeError(f"{name} must be a [tokens, head, size_per_head] view with contiguous channels")
+    return 0, t.stride(1), t.stride(0)
+
+
+def attn_fused_varlen(q, k, v, batch_size: int, max_seq_len: int, seq_len_list, *, scale: Optional[float] = None,
+                      causal: bool = True, out: Optional[torch.Tensor] = None):
+    """Self-attention on packed tokens: ``q``, ``k``, ``v`` are ``[T,H,D]`` views (any token and head
+    strides) of the projection output, the result is the packed context ``[1,T,H,D]``.  Batch ``b``
+    occupies rows ``cu_seqlens[b] .. cu_seqlens[b+1]``; no padded tensor is built.  fp16 / bf16 only.
+    """
+    qs, ks, vs = _thd(q, "q"), _thd(k, "k"), _thd(v, "v")
+    T, H, D = q.shape
+    if k.shape != q.shape or v.shape != q.shape or k.dtype != q.dtype or v.dtype != q.dtype:
+        raise RuntimeError("attn_fused_varlen: q, k, v disagree in shape or dtype")
+    if q.dtype not in (torch.float16, torch.bfloat16):
+        raise RuntimeError("attn_fused_varlen: Datatype not implemented (float16 and bfloat16 only)")
+    info = seq_info(seq_len_list, batch_size, q.device)
+    if out is None:
+        out = torch.empty((1, T, H, D), dtype=q.dtype, device=q.device)
+    elif out.numel() != T * H * D or out.dtype != q.dtype or not out.is_contiguous():
+        raise RuntimeError("attn_fused_varlen: out must be contiguous [1,T,H,D] of q's dtype")
+    arr = ctypes.c_int64 * 3
+    cu = info.cu_seqlens.data_ptr()
+    scale = float(D) ** -0.5 if scale is None else float(scale)
+    with _lib.device_guard(q):
+        _lib.check(_lib.fn.en_attn_fused(q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(),
+                                         info.lens.data_ptr(), None, batch_size, H, int(max_seq_len),
+                                         int(max_seq_len), D, arr(*qs), arr(*ks), arr(*vs), arr(0, D, H * D), cu, cu,
+                                         scale, int(bool(causal)), _lib.dtype_tag(q, "attn_fused_varlen"),
+                                         _lib.stream_of(q)), "attn_fused_varlen")
+    return out
+
+
 def attn_fused_packed(qkv, batch_size: int, max_seq_len: int, seq_len_list, head_num: int, size_per_head: int, *,
                       scale: Optional[float] = None, causal: bool = True, out: Optional[torch.Tensor] = None):
     """Self-attention straight on the packed projection output: ``qkv`` is ``[1,T,H,3D]`` (or ``[T,H,3D]``,
     the layout ``transpose_pad`` is fed with in examples/bert/bert.py:100-104), the result is the packed
-    context ``[1,T,H,D]`` that ``transpose_depad`` would return (bert.py:123).  No padded tensor is built:
-    batch ``b`` is addressed at row ``cu_seqlens[b]``.  fp16 / bf16 only.
+    context ``[1,T,H,D]`` that ``transpose_depad`` would return (bert.py:123).  fp16 / bf16 only.
     """
     _lib.require_gpu(qkv, "qkv")
     H, D = int(head_num), int(size_per_head)
-    if qkv.dtype not in (torch.float16, torch.bfloat16):
-        raise RuntimeError("attn_fused_packed: Datatype not implemented (float16 and bfloat16 only)")
     if qkv.numel() % (3 * H * D) != 0:
         raise RuntimeError("attn_fused_packed: qkv must be [1,T,H,3D]")
-    T = qkv.numel() // (3 * H * D)
-    info = seq_info(seq_len_list, batch_size, qkv.device)
-    if out is None:
-        out = torch.empty((1, T, H, D), dtype=qkv.dtype, device=qkv.device)
-    elif out.numel() != T * H * D or out.dtype != qkv.dtype or not out.is_contiguous():
-        raise RuntimeError("attn_fused_packed: out must be contiguous [1,T,H,D] of qkv's dtype")
-    arr = ctypes.c_int64 * 3
-    es = qkv.element_size()
-    in_strides = arr(0, 3 * D, 3 * H * D)
-    out_strides = arr(0, D, H * D)
-    base = qkv.data_ptr()
-    cu = info.cu_seqlens.data_ptr()
-    scale = float(D) ** -0.5 if scale is None else float(scale)
-    with _lib.device_guard(qkv):
-        _lib.check(_lib.fn.en_attn_fused(base, base + D * es, base + 2 * D * es, out.data_ptr(), info.lens.data_ptr(),
-                                         None, batch_size, H, int(max_seq_len), int(max_seq_len), D, in_strides,
-                                         in_strides, in_strides, out_strides, cu, cu, scale, int(bool(causal)),
-                                         _lib.dtype_tag(qkv, "attn_fused_packed"), _lib.stream_of(qkv)),
-                   "attn_fused_packed")
-    return out
+    q, k, v = torch.chunk(qkv.view(-1, H, 3 * D), 3, dim=-1)
+    return attn_fused_varlen(q, k, v, batch_size, max_seq_len, seq_len_list, scale=scale, causal=causal, out=out)
+
+
+def kv_cache_fill(src, cache, batch_size: int, seq_len_list, head_first: int = 0):
+    """Writes ``cache[b,h,s,:] = src[cu[b]+s, head_first+h, :]`` for ``s < len[b]`` and zeros for the rest of
+    the ``[B,H,Smax,D]`` cache.  ``src`` is the packed projection output seen as ``[T,Hs,D]`` (contiguous),
+    so K and V caches are filled from their thirds of a fused projection without copying them out first.
+    """
+    _lib.require_gpu(src, "src")
+    _lib.require_gpu(cache, "cache")
+    if src.dim() != 3 or cache.dim() != 4 or cache.shape[0] != batch_size or cache.shape[3] != src.shape[2] \
+            or cache.dtype != src.dtype:
+        raise RuntimeError("kv_cache_fill: src must be [T,Hs,D] and cache [B,H,Smax,D] of one dtype")
+    B, H, Smax, D = cache.shape
+    info = seq_info(seq_len_list, batch_size, src.device)
+    with _lib.device_guard(src):
+        _lib.check(_lib.fn.en_transpose_pad_heads(src.data_ptr(), cache.data_ptr(), info.cu_seqlens.data_ptr(), B, Smax,
+                                                  H, D, src.shape[1], int(head_first), src.element_size(),
+                                                  _lib.stream_of(src)), "kv_cache_fill")
+    return cache
+
+
+def kv_cache_append(k_new, v_new, k_cache, v_cache, kv_len_list):
+    """Writes the new token's rows ``k_new`` / ``v_new`` (``[B,H,D]`` views) into the ``[B,H,Smax,D]`` caches at
+    position ``kv_len[b]``.  The caller advances the lengths afterwards."""
+    for t, n in ((k_new, "k_new"), (v_new, "v_new")):
+        _lib.require_gpu(t, n, contiguous=False)
+        if t.dim() != 3 or t.stride(2) != 1:
+            raise RuntimeError(f"kv_cache_append: {n} must be a [B,H,D] view with contiguous channels")
+    cs = _bhsd(k_cache, "k_cache")
+    if _bhsd(v_cache, "v_cache") != cs or k_new.stride() != v_new.stride() or k_cache.shape != v_cache.shape:
+        raise RuntimeError("kv_cache_append: K and V must share shapes and strides")
+    B, H, Smax, D = k_cache.shape
+    if k_new.shape != (B, H, D) or v_new.shape != (B, H, D) or k_new.dtype != k_cache.dtype:
+        raise RuntimeError("kv_cache_append: new rows must be [B,H,D] of the cache dtype")
+    info = seq_info(kv_len_list, B, k_cache.device)
+    with _lib.device_guard(k_cache):
+        _lib.check(_lib.fn.en_kv_append(k_new.data_ptr(), v_new.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(),
+                                        info.lens.data_ptr(), B, H, Smax, D, k_new.stride(0), k_new.stride(1), *cs,
+                                        k_cache.element_size(), _lib.stream_of(k_cache)), "kv_cache_append")
 
 
 def decode_qk(q, k_cache, kv_len_list, *, alpha: float = 1.0, out: Optional[torch.Tensor] = None):

@@ -102,6 +102,27 @@ def depad(src, batch_size, seq_lens, left_padded=False, sum_seq=None):
     return dst
 
 
+def repad(src, batch_size, max_seq_len, seq_lens, left_padded=False):
+    """[1,T,hid] -> [B,S,hid] with zero padding rows: the inverse of :func:`depad`.
+
+    An addition for the exit of the packed path; the reference callers rebuild
+    right-padded batches with ``ft_rebuild_padding`` (examples/gpt/gpt.py:321-323)
+    while their generation batches are left-padded (examples/opt/batch.py:12-24).
+    """
+    _lib.require_gpu(src, "src", contiguous=False)
+    src = src.contiguous()
+    hid = src.shape[-1]
+    info = seq_info(seq_lens, batch_size, src.device)
+    if src.numel() % hid != 0 or src.dim() < 2:
+        raise RuntimeError("repad: src must be [1, total, hidden]")
+    S = _as_int(max_seq_len)
+    dst = torch.empty((batch_size, S, hid), dtype=src.dtype, device=src.device)
+    with _lib.device_guard(src):
+        _lib.check(_lib.fn.en_repad(src.data_ptr(), dst.data_ptr(), info.cu_seqlens.data_ptr(), batch_size, S, hid,
+                                    _elem_size(src, "repad"), int(bool(left_padded)), _lib.stream_of(src)), "repad")
+    return dst
+
+
 # From FasterTransformer
 
 

@@ -1,0 +1,40 @@
+"""Preallocated per-sequence K/V cache for incremental decode.
+
+The reference keeps the whole projection history and ``torch.cat``s one more
+position onto it on every step, then recomputes attention for every position
+(energonai/model/attention.py:61-71,89-98).  Here K and V live in two
+``[B,H,Smax,D]`` buffers with a device-side length per sequence: prefill writes
+each sequence's rows at positions ``0..len-1`` (whatever side the batch was
+padded on), a decode step appends one row per sequence and reads only the
+valid prefix.
+"""
+from __future__ import annotations
+
+import torch
+
+from ..kernel import kv_cache_append, kv_cache_fill
+from ..seqinfo import SeqInfo
+
+
+class KVCache:
+    def __init__(self, batch_size: int, head_num: int, max_seq_len: int, size_per_head: int, dtype, device):
+        self.k = torch.zeros((batch_size, head_num, max_seq_len, size_per_head), dtype=dtype, device=device)
+        self.v = torch.zeros_like(self.k)
+        self.lens = torch.zeros(batch_size, dtype=torch.int32, device=device)
+        self.batch_size = batch_size
+        self.max_seq_len = max_seq_len
+        # lengths are advanced in place, so the kernels are handed this fixed view instead of
+        # going through the per-tensor offset cache
+        self.info = SeqInfo(self.lens, None, batch_size, None, self.lens)
+
+    def fill(self, k_src: torch.Tensor, v_src: torch.Tensor, info: SeqInfo, k_head_first: int = 0,
+             v_head_first: int = 0) -> None:
+        """Prefill from packed projections seen as ``[T,Hs,D]`` (see ``kv_cache_fill``)."""
+        kv_cache_fill(k_src, self.k, self.batch_size, info, k_head_first)
+        kv_cache_fill(v_src, self.v, self.batch_size, info, v_head_first)
+        self.lens.copy_(info.lens)
+
+    def append(self, k_new: torch.Tensor, v_new: torch.Tensor) -> None:
+        """One new ``[B,H,D]`` row per sequence; lengths advance by one."""
+        kv_cache_append(k_new, v_new, self.k, self.v, self.info)
+        self.lens.add_(1)

@@ -59,11 +59,28 @@ int en_prefix_sum(const void *seq_lens, int lens_are_i64, int batch, int32_t *cu
 int en_depad(const void *src, void *dst, const int32_t *cu_seqlens, int batch, int max_seq_len, int64_t hidden,
              int elem_size, int left_padded, en_stream_t stream);
 
+/* repad: [T,hid] -> [B,S,hid], the inverse of en_depad with zeros in the padding
+ * rows; the exit of the packed path (the reference callers use
+ * ft_rebuild_padding for right-padded batches, examples/gpt/gpt.py:321-323, and
+ * left-pad their generation batches, examples/opt/batch.py:12-24).  Every row
+ * of dst is written. */
+int en_repad(const void *src, void *dst, const int32_t *cu_seqlens, int batch, int max_seq_len, int64_t hidden,
+             int elem_size, int left_padded, en_stream_t stream);
+
 /* transpose_pad_wrapper (csrc/transpose_pad_fusion_wrapper.cpp:33-57, kernel
  * csrc/transpose_pad_fusion_kernel.cu:58-96): [T,H,Dk] -> [B,H,S,Dk]; every
  * byte of dst is written, padding rows as zero. */
 int en_transpose_pad(const void *src, void *dst, const int32_t *cu_seqlens, int batch, int max_seq_len, int head_num,
                      int size_per_head, int elem_size, en_stream_t stream);
+
+/* en_transpose_pad whose packed source holds src_head_rows rows of size_per_head
+ * elements per token, of which rows src_head_first .. src_head_first+head_num-1
+ * are moved: fills a [B,H,S,D] K or V cache from the k / v third of a fused
+ * projection output without first copying that third out (the reference makes
+ * the thirds contiguous with .contiguous(), energonai/model/attention.py:74). */
+int en_transpose_pad_heads(const void *src, void *dst, const int32_t *cu_seqlens, int batch, int max_seq_len,
+                           int head_num, int size_per_head, int src_head_rows, int src_head_first, int elem_size,
+                           en_stream_t stream);
 
 /* transpose_depad_wrapper (wrapper.cpp:59-83, kernel.cu:8-46):
  * [B,H,S,D] -> [T,H,D]; every byte of dst is written when T = cu_seqlens[B]. */
@@ -170,6 +187,18 @@ int en_decode_qk(const void *q, const void *k_cache, void *scores, const int32_t
 int en_decode_pv(const void *p, const void *v_cache, void *ctx, const int32_t *kv_lens, int batch, int head_num,
                  int k_seq_len, int size_per_head, int64_t v_stride_b, int64_t v_stride_h, int64_t v_stride_s,
                  int dtype, en_stream_t stream);
+
+/* Appends the new token's K and V rows to [B,H,Smax,D] caches at position
+ * kv_lens[b] (the caller then adds one to kv_lens); replaces the reference's
+ * torch.cat of the whole projection history on every step
+ * (energonai/model/attention.py:66-71,89-98).  k_new / v_new are addressed as
+ * base + b*new_stride_b + h*new_stride_h + d, the caches as
+ * base + b*stride_b + h*stride_h + s*stride_s + d (elements of elem_size bytes).
+ * A sequence with kv_lens[b] >= k_seq_len is left alone. */
+int en_kv_append(const void *k_new, const void *v_new, void *k_cache, void *v_cache, const int32_t *kv_lens,
+                 int batch, int head_num, int k_seq_len, int size_per_head, int64_t new_stride_b,
+                 int64_t new_stride_h, int64_t cache_stride_b, int64_t cache_stride_h, int64_t cache_stride_s,
+                 int elem_size, en_stream_t stream);
 
 /* Fused attention (an addition: the reference callers run matmul, softmax, matmul,
  * examples/bert/bert.py:108-119): ctx[b,h,i,:] = sum_j softmax_j(scale * <q_i, k_j>) v[b,h,j,:]

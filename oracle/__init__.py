@@ -10,6 +10,8 @@ Contents
 eager.py      torch-eager restatement of every op on the path, written from the
               reference's Python wrappers, CUDA index formulas and its own test
               oracle (each function cites the reference file:line it follows).
+models.py     the same for the reference's attention / MLP / block modules on padded
+              batches (the callers either side of the path).
 brute.py      pure-Python triple loops that replay the reference CUDA kernels'
               blockIdx/threadIdx arithmetic on tiny inputs; they pin eager.py.
 kernels_ref.c plain-C replay of the same kernels (grid loops on the CPU) for

@@ -76,6 +76,28 @@ def depad(src: torch.Tensor, batch_size: int, seq_lens, left_padded: bool = Fals
     return torch.cat(parts, dim=1)
 
 
+def repad(src: torch.Tensor, batch_size: int, max_seq_len: int, seq_lens, left_padded: bool = False) -> torch.Tensor:
+    """[1,T,hid] -> [B,S,hid]: the inverse of :func:`depad`, padding rows zero.
+
+    For right-padded batches this is what ft_rebuild_padding produces from the
+    packed rows (csrc/transpose_pad_fusion_kernel.cu:176-199, caller
+    examples/gpt/gpt.py:321-323); ``left_padded`` puts sequence b at rows S-len:S.
+    """
+    lens = _as_len_list(seq_lens)
+    hid = src.shape[-1]
+    rows = src.reshape(-1, hid)
+    out = torch.zeros((batch_size, max_seq_len, hid), dtype=src.dtype)
+    start = 0
+    for i in range(batch_size):
+        n = lens[i]
+        if left_padded:
+            out[i, max_seq_len - n:max_seq_len] = rows[start:start + n]
+        else:
+            out[i, 0:n] = rows[start:start + n]
+        start += n
+    return out
+
+
 def transpose_pad(src: torch.Tensor, batch_size: int, max_seq_len: int, seq_lens,
                   head_num: int, size_per_head: int) -> torch.Tensor:
     """[1,T,H,Dk] -> zero-padded [B,H,S,Dk].

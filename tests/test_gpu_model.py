@@ -1,0 +1,149 @@
+"""Model glue (attention / MLP / block modules, K/V cache, repad) against the padded eager oracle."""
+import pytest
+import torch
+import torch.nn.functional as F
+
+from gpu_util import announce, max_abs
+from oracle import eager, models
+
+pytestmark = pytest.mark.gpu
+
+
+def _mods():
+    import energonai_amd.kernel as K
+    import energonai_amd.model as M
+    return K, M
+
+
+def _fp32_params(module):
+    return {k: v.detach().float().cpu() for k, v in module.state_dict().items()}
+
+
+def _padded_batch(B, S, hid, lens, left, dtype, seed):
+    g = torch.Generator().manual_seed(seed)
+    x = torch.randn(B, S, hid, generator=g).to(dtype)
+    valid = torch.zeros(B, S)
+    for b, n in enumerate(lens):
+        if left:
+            valid[b, S - n:] = 1
+        else:
+            valid[b, :n] = 1
+    return x * valid.unsqueeze(-1).to(dtype), valid
+
+
+def _init(module, seed):
+    g = torch.Generator().manual_seed(seed)
+    with torch.no_grad():
+        for name, prm in module.named_parameters():
+            if name.endswith("weight") and prm.dim() == 1:
+                prm.copy_(1.0 + 0.05 * torch.randn(prm.shape, generator=g))
+            elif prm.dim() == 1:
+                prm.copy_(0.05 * torch.randn(prm.shape, generator=g))
+            else:
+                prm.copy_(torch.randn(prm.shape, generator=g) / prm.shape[1] ** 0.5)
+
+
+def _valid_rows(t, lens, left):
+    S = t.shape[1]
+    return torch.cat([t[b, S - n:] if left else t[b, :n] for b, n in enumerate(lens)])
+
+
+@pytest.mark.parametrize("left", [True, False])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.float32])
+def test_repad_is_inverse_of_depad(dtype, left):
+    K, _ = _mods()
+    B, S, hid = 5, 37, 96
+    lens = [37, 1, 0, 20, 36]
+    announce("repad", dtype, left)
+    x, _ = _padded_batch(B, S, hid, lens, left, dtype, 11)
+    lens_t = torch.tensor(lens, dtype=torch.int64).cuda()
+    packed = K.depad(x.cuda(), B, lens_t, left_padded=left)
+    back = K.repad(packed, B, S, lens_t, left_padded=left).cpu()
+    assert torch.equal(back, x)
+    assert torch.equal(back, eager.repad(packed.cpu(), B, S, lens, left_padded=left))
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.float32])
+def test_kv_cache_fill_and_append_bit_exact(dtype):
+    K, M = _mods()
+    B, H, D, Smax = 3, 4, 64, 50
+    lens = [7, 30, 1]
+    T = sum(lens)
+    announce("kv cache", dtype)
+    g = torch.Generator().manual_seed(12)
+    kvq = torch.randn(T, 3 * H, D, generator=g).to(dtype)
+    info_lens = torch.tensor(lens, dtype=torch.int32).cuda()
+    cache = M.KVCache(B, H, Smax, D, dtype, "cuda")
+    from energonai_amd.seqinfo import seq_info
+    info = seq_info(info_lens, B, torch.device("cuda"))
+    cache.fill(kvq.cuda(), kvq.cuda(), info, 0, H)
+    want_k = torch.zeros(B, H, Smax, D, dtype=dtype)
+    want_v = torch.zeros_like(want_k)
+    start = 0
+    for b, n in enumerate(lens):
+        want_k[b, :, :n] = kvq[start:start + n, :H].permute(1, 0, 2)
+        want_v[b, :, :n] = kvq[start:start + n, H:2 * H].permute(1, 0, 2)
+        start += n
+    assert torch.equal(cache.k.cpu(), want_k) and torch.equal(cache.v.cpu(), want_v)
+    assert cache.lens.cpu().tolist() == lens
+    for step in range(3):
+        new = torch.randn(B, 3 * H, D, generator=g).to(dtype)
+        new_g = new.cuda()
+        cache.append(new_g[:, :H], new_g[:, H:2 * H])
+        for b, n in enumerate(lens):
+            want_k[b, :, n + step] = new[b, :H]
+            want_v[b, :, n + step] = new[b, H:2 * H]
+        assert torch.equal(cache.k.cpu(), want_k) and torch.equal(cache.v.cpu(), want_v)
+        assert cache.lens.cpu().tolist() == [n + step + 1 for n in lens]
+
+
+@pytest.mark.parametrize("fused_qkv", [True, False])
+@pytest.mark.parametrize("is_decoder", [True, False])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16, torch.float32])
+def test_attention_module_prefill(dtype, is_decoder, fused_qkv):
+    """MultiHeadAttention1D.forward on a padded batch equals the reference forward on valid positions."""
+    _, M = _mods()
+    B, S, hid, heads = 4, 160, 256, 4
+    lens = [160, 33, 97, 128]
+    left = is_decoder
+    announce("mha prefill", dtype, is_decoder, fused_qkv)
+    attn = M.MultiHeadAttention1D(hid, heads, dtype=dtype, max_seq_len=192, fused_qkv=fused_qkv,
+                                  is_decoder=is_decoder, disable_past_cache=True).cuda()
+    _init(attn, 21)
+    x, valid = _padded_batch(B, S, hid, lens, left, dtype, 22)
+    mask = models.additive_mask(valid)
+    got = attn(x.cuda(), attention_mask=mask.to(dtype).cuda()).float().cpu()
+    want = models.mha_forward(x, _fp32_params(attn), heads, is_decoder, mask, fused_qkv)
+    tol = {torch.float16: 4e-3, torch.bfloat16: 3e-2, torch.float32: 2e-4}[dtype]
+    assert max_abs(_valid_rows(got, lens, left), _valid_rows(want, lens, left)) <= tol
+    pad = torch.cat([got[b, :S - n] if left else got[b, n:] for b, n in enumerate(lens)])
+    assert bool((pad == 0).all())          # padding rows come back as zeros
+
+
+@pytest.mark.parametrize("post", [True, False])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.float32])
+def test_block_prefill_and_incremental_decode(dtype, post):
+    """Block1D: prefill with first_cache=True, then three decode steps; the newest position of each
+    step equals the reference block recomputed on the whole extended (left-padded) batch."""
+    _, M = _mods()
+    B, S, hid, heads = 3, 70, 128, 2
+    lens = [70, 9, 41]
+    announce("block decode", dtype, post)
+    blk = M.Block1D(hid, heads, 4.0, dtype=dtype, apply_post_layernorm=post, max_seq_len=96).cuda()
+    _init(blk, 31)
+    p = _fp32_params(blk)
+    x, valid = _padded_batch(B, S, hid, lens, True, dtype, 32)
+    tol = {torch.float16: 1.5e-2, torch.float32: 5e-4}[dtype]
+    mask = models.additive_mask(valid)
+    got = blk(x.cuda(), attention_mask=mask.to(dtype).cuda(), first_cache=True).float().cpu()
+    want = models.block_forward(x, p, heads, 1e-5, post, True, mask)
+    assert max_abs(_valid_rows(got, lens, True), _valid_rows(want, lens, True)) <= tol
+    g = torch.Generator().manual_seed(33)
+    for step in range(3):
+        x = torch.cat((x, torch.randn(B, 1, hid, generator=g).to(dtype)), 1)
+        valid = torch.cat((valid, torch.ones(B, 1)), 1)
+        mask = models.additive_mask(valid)
+        got = blk(x.cuda(), attention_mask=mask.to(dtype).cuda(), first_cache=False).float().cpu()
+        want = models.block_forward(x, p, heads, 1e-5, post, True, mask)
+        assert got.shape == want.shape
+        assert max_abs(got[:, -1], want[:, -1]) <= tol, step
