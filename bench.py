@@ -132,6 +132,74 @@ def add_eager_aux(torch, w, d, device):
 
 
 # ---------------------------------------------------------------------------
+# whole transformer block (projections and MLP included): Block1D of this package on packed
+# tokens against the reference block's forward (energonai/model/endecoder.py:48-70,
+# attention.py:56-136 without the past cache) written with stock torch ops on the padded batch
+# ---------------------------------------------------------------------------
+def eager_block_forward(torch, blk, x, mask, heads, causal_tri, neg):
+    import torch.nn.functional as F
+    B, S, hid = x.shape
+    D = hid // heads
+    n1, n2, at, mlp = blk.norm1, blk.norm2, blk.attn, blk.mlp
+    h = F.layer_norm(x, (hid,), n1.weight, n1.bias, n1.eps)
+    k, v, q = torch.chunk(at.query_key_value(h), 3, dim=-1)
+    sp = lambda t: t.reshape(B, S, heads, D).permute(0, 2, 1, 3)
+    q, k, v = sp(q) * (D ** -0.5), sp(k), sp(v)
+    sc = torch.where(causal_tri, torch.matmul(q, k.transpose(-1, -2)), neg) + mask
+    pr = torch.softmax(sc, -1, dtype=torch.float).to(x.dtype)
+    ctx = torch.matmul(pr, v).transpose(1, 2).reshape(B, S, hid)
+    s1 = x + at.dense(ctx)
+    h2 = F.layer_norm(s1, (hid,), n2.weight, n2.bias, n2.eps)
+    return s1 + mlp.dense_2(mlp.activation(mlp.dense_1(h2)))
+
+
+def run_block(torch, w, steps, warmup):
+    """Prefill of one pre-LN decoder block at the workload's shape (left-padded batch in, padded batch out)."""
+    from energonai_amd import workloads
+    from energonai_amd.model import Block1D
+    from energonai_amd.seqinfo import seq_info
+    dev = torch.device("cuda")
+    B, S, hid, H = w.batch, w.seq, w.heads * w.head_dim, w.heads
+    lens = workloads.make_lens(w)
+    ll = [int(v) for v in lens]
+    g = torch.Generator().manual_seed(3000 + w.index)
+    blk = Block1D(hid, H, 4.0, dtype=w.dtype, max_seq_len=S, disable_past_cache=True).to(dev)
+    with torch.no_grad():
+        for name, prm in blk.named_parameters():
+            if prm.dim() == 2:
+                prm.copy_((0.02 * torch.randn(prm.shape, generator=g)).to(w.dtype))
+    x = torch.randn(B, S, hid, generator=g).to(w.dtype)
+    valid = torch.zeros(B, S)
+    for b, n in enumerate(ll):
+        valid[b, S - n:] = 1
+    x = (x * valid.unsqueeze(-1).to(w.dtype)).to(dev)
+    mask = ((1.0 - valid) * -10000.0).to(w.dtype).view(B, 1, 1, S).to(dev)
+    tri = torch.tril(torch.ones(S, S, dtype=torch.bool, device=dev)).view(1, 1, S, S)
+    neg = torch.tensor(-1e4, dtype=w.dtype, device=dev)
+    info = seq_info(lens.to(dev), B, dev)
+    tokens = info.total
+    with torch.no_grad():
+        ours = lambda: blk(x, seq_lens=info)
+        ref = lambda: eager_block_forward(torch, blk, x, mask, H, tri, neg)
+        a, b_ = ours(), ref()
+        rows = valid.bool().to(dev)
+        err = (a[rows].float() - b_[rows].float()).abs().max().item()
+        for _ in range(warmup):
+            ours()
+        torch.cuda.synchronize()
+        ms = _event_time_ms(ours, steps, torch)
+        for _ in range(max(2, warmup // 2)):
+            ref()
+        torch.cuda.synchronize()
+        ms_ref = _median_step_ms(ref, max(5, steps // 2), torch)
+    del blk
+    torch.cuda.empty_cache()
+    return {"shape": f"{w.name}: hidden {hid}, {H} heads, batch {B}, bucket {S}, {tokens} valid tokens, left-padded",
+            "ms_per_block": ms, "tokens_per_s": tokens / (ms * 1e-3), "eager_padded_ms_per_block": ms_ref,
+            "speedup_vs_eager_padded": ms_ref / ms, "max_abs_diff_vs_eager_on_valid_rows": err}
+
+
+# ---------------------------------------------------------------------------
 # one workload on the GPU
 # ---------------------------------------------------------------------------
 def run_workload(torch, w, steps, warmup, want_eager=True, want_kernels=True):
@@ -439,6 +507,13 @@ def main(argv=None) -> int:
             except Exception as exc:
                 others[ow.name] = {"error": str(exc)[:300]}
         out["workloads"] = others
+        blocks = {}
+        for name in ("c2", "c3"):
+            try:
+                blocks[name] = run_block(torch, workloads.BY_NAME[name], max(5, ns.steps // 2), max(2, ns.warmup // 2))
+            except Exception as exc:
+                blocks[name] = {"error": str(exc)[:300]}
+        out["model_block_prefill"] = blocks
     if not ns.no_cpu:
         out["cpu_baseline"] = cpu_baseline(torch, w)
     else:
