@@ -154,7 +154,7 @@ def eager_block_forward(torch, blk, x, mask, heads, causal_tri, neg):
 
 
 def run_block(torch, w, steps, warmup):
-    """Prefill of one pre-LN decoder block at the workload's shape (left-padded batch in, padded batch out)."""
+    """Prefill of one pre-LN OPT decoder block (ReLU MLP) at the workload's shape (left-padded batch in, padded batch out)."""
     from energonai_amd import workloads
     from energonai_amd.model import Block1D
     from energonai_amd.seqinfo import seq_info
@@ -163,7 +163,8 @@ def run_block(torch, w, steps, warmup):
     lens = workloads.make_lens(w)
     ll = [int(v) for v in lens]
     g = torch.Generator().manual_seed(3000 + w.index)
-    blk = Block1D(hid, H, 4.0, dtype=w.dtype, max_seq_len=S, disable_past_cache=True).to(dev)
+    import torch.nn.functional as F
+    blk = Block1D(hid, H, 4.0, activation=F.relu, dtype=w.dtype, max_seq_len=S, disable_past_cache=True).to(dev)   # OPT: ReLU
     with torch.no_grad():
         for name, prm in blk.named_parameters():
             if prm.dim() == 2:

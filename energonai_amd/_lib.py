@@ -48,7 +48,35 @@ SIGNATURES = {
     "en_copy_bytes": (c_int, [c_void_p, c_void_p, c_int64, c_void_p]),
 }
 
+LINEAR_LIB_NAME = "libenergon_linear.so"
+LINEAR_LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), LINEAR_LIB_NAME)
+LINEAR_SIGNATURES = {
+    "en_linear": (c_int, [c_void_p] * 4 + [c_int64] * 3 + [c_int] * 3 + [c_void_p, c_int64, c_void_p]),
+    "en_linear_algo_count": (c_int, [c_int64] * 3 + [c_int] * 3 + [c_int64]),
+    "en_linear_status_string": (ctypes.c_char_p, [c_int]),
+}
+
 _lib = None
+_linear_lib = None
+
+
+def load_linear() -> ctypes.CDLL:
+    """Loads the hipBLASLt front end once; raises RuntimeError if it is not built."""
+    global _linear_lib
+    if _linear_lib is None:
+        if not os.path.exists(LINEAR_LIB_PATH):
+            raise RuntimeError(f"energonai_linear_func requires cuda extensions: {LINEAR_LIB_NAME} is not built "
+                               f"(run `python -m energonai_amd.build`)")
+        try:
+            lib = ctypes.CDLL(LINEAR_LIB_PATH)
+        except OSError as exc:
+            raise RuntimeError(f"energonai_linear_func requires cuda extensions: cannot load {LINEAR_LIB_PATH}: {exc}") from exc
+        for name, (restype, argtypes) in LINEAR_SIGNATURES.items():
+            fn = getattr(lib, name)
+            fn.restype = restype
+            fn.argtypes = argtypes
+        _linear_lib = lib
+    return _linear_lib
 
 
 def load() -> ctypes.CDLL:

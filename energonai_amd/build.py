@@ -1,4 +1,5 @@
-"""Builds libenergon_hip.so (gfx950) from energonai_amd/csrc/*.hip with hipcc.
+"""Builds libenergon_hip.so (gfx950) from energonai_amd/csrc/*.hip with hipcc, and
+libenergon_linear.so (host code over hipBLASLt) from csrc/linear_blaslt.cpp.
 
     python -m energonai_amd.build            # compile every source, link the library
     python -m energonai_amd.build --force    # recompile even if objects look fresh
@@ -22,6 +23,9 @@ CSRC = os.path.join(PKG_DIR, "csrc")
 INCLUDE = os.path.join(ROOT, "include")
 OBJ_DIR = os.path.join(PKG_DIR, "build")
 LIB_PATH = os.path.join(PKG_DIR, "libenergon_hip.so")
+# host-only hipBLASLt front end for the projection GEMMs; the only piece that links more than the HIP runtime
+LINEAR_SRC = os.path.join(CSRC, "linear_blaslt.cpp")
+LINEAR_LIB_PATH = os.path.join(PKG_DIR, "libenergon_linear.so")
 
 ARCH = "gfx950"
 # packed fp32 VALU ops are switched off for device code on purpose (they have
@@ -79,7 +83,20 @@ def build(force: bool = True, verbose: bool = False, jobs: int = 4) -> str:
     if proc.returncode != 0:
         raise RuntimeError("link failed:\n" + proc.stdout)
     os.replace(tmp, LIB_PATH)
+    build_linear()
     return LIB_PATH
+
+
+def build_linear() -> str:
+    rocm_lib = os.path.join(os.path.dirname(os.path.dirname(os.path.realpath(_hipcc()))), "lib")
+    tmp = LINEAR_LIB_PATH + ".tmp"
+    cmd = [_hipcc(), "-O2", "-std=c++17", "-fPIC", "-shared", f"-I{INCLUDE}", LINEAR_SRC, "-o", tmp,
+           f"-L{rocm_lib}", "-L/opt/rocm/lib", "-lhipblaslt", "-lamdhip64"]
+    proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    if proc.returncode != 0:
+        raise RuntimeError("building libenergon_linear.so failed:\n" + proc.stdout)
+    os.replace(tmp, LINEAR_LIB_PATH)
+    return LINEAR_LIB_PATH
 
 
 def main(argv=None) -> int:

@@ -43,6 +43,23 @@ def test_library_exports_every_declared_symbol():
     assert b"NULL" in lib.en_status_string(-1)
 
 
+def test_linear_library_exports_every_declared_symbol():
+    from energonai_amd import _lib
+    lib = _lib.load_linear()
+    header = os.path.join(ROOT, "include", "energon_linear.h")
+    text = re.sub(r"/\*.*?\*/", "", open(header).read(), flags=re.S)
+    declared = sorted(set(re.findall(r"\b(en_linear[a-z0-9_]*)\s*\(", text)))
+    assert sorted(_lib.LINEAR_SIGNATURES) == declared
+    for name, (_, argtypes) in _lib.LINEAR_SIGNATURES.items():
+        assert hasattr(lib, name)
+        m = re.search(r"\b%s\s*\((.*?)\)\s*;" % re.escape(name), text, flags=re.S)
+        assert len(argtypes) == len(m.group(1).split(",")), name
+    assert lib.en_linear_status_string(0) == b"ok"
+    # argument errors are found before any hipBLASLt or GPU call
+    assert lib.en_linear(None, None, None, None, 1, 1, 1, 0, 1, -1, None, 0, None) == -1
+    assert lib.en_linear(16, 32, None, 48, 0, 1, 1, 0, 1, -1, None, 0, None) == -1
+
+
 def test_entry_points_validate_before_launch():
     """NULL pointers and bad extents are refused on the host: no GPU is touched."""
     from energonai_amd import _lib

@@ -147,3 +147,24 @@ def test_block_prefill_and_incremental_decode(dtype, post):
         want = models.block_forward(x, p, heads, 1e-5, post, True, mask)
         assert got.shape == want.shape
         assert max_abs(got[:, -1], want[:, -1]) <= tol, step
+
+
+@pytest.mark.parametrize("act_name", ["relu", "gelu_tanh", "gelu"])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.float32])
+def test_mlp_with_gemm_epilogues(dtype, act_name):
+    """MLP1D: ReLU and tanh-GELU ride in the first GEMM's epilogue, erf-GELU stays a separate op; all
+    three equal the reference MLP forward."""
+    import functools
+    _, M = _mods()
+    hid, rows = 256, 77
+    announce("mlp", dtype, act_name)
+    act = {"relu": F.relu, "gelu_tanh": functools.partial(F.gelu, approximate="tanh"), "gelu": F.gelu}[act_name]
+    mlp = M.MLP1D(hid, 4.0, act, dtype=dtype, disable_past_cache=True).cuda()
+    assert (mlp._epilogue is None) == (act_name == "gelu")
+    _init(mlp, 51)
+    g = torch.Generator().manual_seed(52)
+    x = torch.randn(1, rows, hid, generator=g).to(dtype)
+    got = mlp(x.cuda()).float().cpu()
+    want = models.mlp_forward(x, _fp32_params(mlp), act)
+    tol = {torch.float16: 6e-3, torch.float32: 2e-4}[dtype]
+    assert max_abs(got, want) <= tol * max(1.0, float(want.abs().max()))
