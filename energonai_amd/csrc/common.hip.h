@@ -33,11 +33,9 @@ inline int dtype_size(int dt) { return dt == EN_F32 ? 4 : ((dt == EN_F16 || dt =
 typedef _Float16 half_t;
 
 __device__ __forceinline__ float bf16_bits_to_float(uint16_t v) { return __uint_as_float(((uint32_t)v) << 16); }
+// Round to nearest even in hardware (v_cvt_pk_bf16_f32 on gfx950; NaN stays NaN).
 __device__ __forceinline__ uint16_t float_to_bf16_bits(float f) {
-  uint32_t u = __float_as_uint(f);
-  if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x0040u);  // quiet NaN
-  u += 0x7fffu + ((u >> 16) & 1u);                                             // round to nearest even
-  return (uint16_t)(u >> 16);
+  return __builtin_bit_cast(uint16_t, static_cast<__bf16>(f));
 }
 
 template <int DT> struct Elem;
