@@ -10,5 +10,6 @@ from .kv_cache import KVCache
 from .attention import MultiHeadAttention1D
 from .mlp import MLP1D
 from .endecoder import Block1D
+from .stack import PackedStack
 
-__all__ = ["KVCache", "MultiHeadAttention1D", "MLP1D", "Block1D"]
+__all__ = ["KVCache", "MultiHeadAttention1D", "MLP1D", "Block1D", "PackedStack"]

@@ -18,7 +18,7 @@ from ..kernel import (attn_fused_varlen, attn_pv, attn_qk, decode_pv, decode_qk,
                       transpose_depad)
 from ..kernel.attention import kv_cache_fill
 from ..seqinfo import SeqInfo, seq_info
-from .kv_cache import KVCache
+from .kv_cache import KVCache, OutputHistory
 
 
 def lens_from_mask(attention_mask: torch.Tensor) -> torch.Tensor:
@@ -53,7 +53,7 @@ class MultiHeadAttention1D(nn.Module):
             self.value_ = nn.Linear(hidden_size, hidden_size, bias=bias, dtype=dtype)
         self.dense = nn.Linear(hidden_size, hidden_size, bias=True, dtype=dtype)
         self.kv_cache: Optional[KVCache] = None
-        self._out = None     # [B, S_so_far, hid]: what the reference keeps in past_cache['dense']
+        self._history = OutputHistory()     # what the reference keeps in past_cache['dense']
 
     # ---- projections: packed rows in, [rows, H, D] views of q, k, v out --------------------
     def _project(self, x: torch.Tensor):
@@ -117,9 +117,7 @@ class MultiHeadAttention1D(nn.Module):
     def forward(self, hidden_states, attention_mask=None, first_cache=False, seq_lens=None):
         B, S, hid = hidden_states.shape
         if not self.disable_past_cache and not first_cache:
-            new = self.forward_last(hidden_states[:, -1:, :])
-            self._out = torch.cat((self._out, new), 1)
-            return self._out
+            return self._history.push(self.forward_last(hidden_states[:, -1:, :]))
         if seq_lens is None:
             seq_lens = lens_from_mask(attention_mask) if attention_mask is not None else \
                 torch.full((B,), S, dtype=torch.int32, device=hidden_states.device)
@@ -128,7 +126,7 @@ class MultiHeadAttention1D(nn.Module):
         y = self.forward_packed(x, info, B, S, fill_cache=not self.disable_past_cache)
         out = repad(y, B, S, info, left_padded=self.left_padded)
         if not self.disable_past_cache:
-            self._out = out
+            return self._history.start(out, self.max_seq_len)
         return out
 
 

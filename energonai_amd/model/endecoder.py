@@ -13,6 +13,7 @@ from torch import nn
 from ..kernel import LayerNorm, depad, layer_norm_forward, repad
 from ..seqinfo import SeqInfo, seq_info
 from .attention import MultiHeadAttention1D, lens_from_mask
+from .kv_cache import OutputHistory
 from .mlp import MLP1D
 
 
@@ -31,7 +32,8 @@ class Block1D(nn.Module):
         self.norm2 = LayerNorm(hidden_size, eps=layernorm_epsilon, dtype=dtype)
         self.mlp = MLP1D(hidden_size=hidden_size, mlp_ratio=mlp_ratio, activation=activation, dtype=dtype, bias=bias,
                          disable_past_cache=disable_past_cache)
-        self._out = None
+        self.max_seq_len = max_seq_len
+        self._history = OutputHistory()
 
     def _rows(self, x: torch.Tensor, attend) -> torch.Tensor:
         """endecoder.py:48-70 on any ``[.., rows, hid]`` tensor; ``attend`` maps normalised rows
@@ -56,9 +58,7 @@ class Block1D(nn.Module):
     def forward(self, hidden_states, attention_mask=None, first_cache=False, seq_lens=None):
         B, S, hid = hidden_states.shape
         if not self.disable_past_cache and not first_cache:
-            new = self._rows(hidden_states[:, -1:, :].contiguous(), self.attn.forward_last)
-            self._out = torch.cat((self._out, new), 1)
-            return self._out
+            return self._history.push(self._rows(hidden_states[:, -1:, :].contiguous(), self.attn.forward_last))
         if seq_lens is None:
             seq_lens = lens_from_mask(attention_mask) if attention_mask is not None else \
                 torch.full((B,), S, dtype=torch.int32, device=hidden_states.device)
@@ -68,5 +68,5 @@ class Block1D(nn.Module):
         y = self.forward_packed(x, info, B, S, fill_cache=not self.disable_past_cache)
         out = repad(y, B, S, info, left_padded=left)
         if not self.disable_past_cache:
-            self._out = out
+            return self._history.start(out, self.max_seq_len)
         return out

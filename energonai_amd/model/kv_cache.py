@@ -38,3 +38,33 @@ class KVCache:
         """One new ``[B,H,D]`` row per sequence; lengths advance by one."""
         kv_cache_append(k_new, v_new, self.k, self.v, self.info)
         self.lens.add_(1)
+
+
+class OutputHistory:
+    """The padded ``[B, S_so_far, hid]`` output a cached module hands back on every call
+    (``past_cache['dense']`` and friends in the reference, energonai/model/attention.py:126-135),
+    kept in one preallocated buffer: a decode step writes one position and returns a view,
+    where the reference concatenates the whole history again."""
+
+    def __init__(self) -> None:
+        self.buf = None
+        self.cur = 0
+
+    def start(self, out: torch.Tensor, max_seq_len: int) -> torch.Tensor:
+        B, S, hid = out.shape
+        self.buf = torch.empty((B, max(int(max_seq_len), S), hid), dtype=out.dtype, device=out.device)
+        self.buf[:, :S].copy_(out)
+        self.cur = S
+        return self.buf[:, :S]
+
+    def push(self, new: torch.Tensor) -> torch.Tensor:
+        if self.buf is None:
+            raise RuntimeError("decode step before a first_cache=True call")
+        if self.cur == self.buf.shape[1]:      # past the planned length: grow geometrically
+            grown = torch.empty((self.buf.shape[0], 2 * self.cur, self.buf.shape[2]), dtype=self.buf.dtype,
+                                device=self.buf.device)
+            grown[:, :self.cur].copy_(self.buf)
+            self.buf = grown
+        self.buf[:, self.cur:self.cur + 1].copy_(new)
+        self.cur += 1
+        return self.buf[:, :self.cur]

@@ -168,3 +168,40 @@ def test_mlp_with_gemm_epilogues(dtype, act_name):
     want = models.mlp_forward(x, _fp32_params(mlp), act)
     tol = {torch.float16: 6e-3, torch.float32: 2e-4}[dtype]
     assert max_abs(got, want) <= tol * max(1.0, float(want.abs().max()))
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.float32])
+def test_packed_stack_prefill_and_decode(dtype):
+    """Three blocks with the padding dropped once for all of them, then two decode steps, against the
+    reference blocks chained on the padded batch."""
+    _, M = _mods()
+    B, S, hid, heads, L = 3, 48, 128, 2, 3
+    lens = [48, 5, 30]
+    announce("stack", dtype)
+    blocks = [M.Block1D(hid, heads, 4.0, activation=F.relu, dtype=dtype, max_seq_len=64) for _ in range(L)]
+    stack = M.PackedStack(blocks).cuda()
+    for i, blk in enumerate(stack.blocks):
+        _init(blk, 60 + i)
+    ps = [_fp32_params(blk) for blk in stack.blocks]
+    x, valid = _padded_batch(B, S, hid, lens, True, dtype, 70)
+    tol = {torch.float16: 4e-2, torch.float32: 2e-3}[dtype]
+
+    def reference(x, valid):
+        h = x.float()
+        for p in ps:
+            h = models.block_forward(h, p, heads, 1e-5, False, True, models.additive_mask(valid), F.relu)
+        return h
+
+    mask = models.additive_mask(valid)
+    got = stack(x.cuda(), attention_mask=mask.to(dtype).cuda(), first_cache=True).float().cpu()
+    want = reference(x, valid)
+    scale = max(1.0, float(_valid_rows(want, lens, True).abs().max()))
+    assert max_abs(_valid_rows(got, lens, True), _valid_rows(want, lens, True)) <= tol * scale
+    g = torch.Generator().manual_seed(71)
+    for step in range(2):
+        x = torch.cat((x, torch.randn(B, 1, hid, generator=g).to(dtype)), 1)
+        valid = torch.cat((valid, torch.ones(B, 1)), 1)
+        got = stack(x.cuda(), attention_mask=models.additive_mask(valid).to(dtype).cuda(), first_cache=False)
+        want = reference(x, valid)
+        assert got.shape == want.shape
+        assert max_abs(got[:, -1].float().cpu(), want[:, -1]) <= tol * scale, step
