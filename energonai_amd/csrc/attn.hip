@@ -463,7 +463,8 @@ int en_attn_pv(const void *p, const void *v, void *ctx, const int32_t *k_lens, c
   if (!strides_vec_ok(v_stride_b, v_stride_h, v_stride_s, epv) ||
       !strides_vec_ok(c_stride_b, c_stride_h, c_stride_s, 4))
     return EN_ERR_ALIGN;
-  if (v_stride_s < 0 || (int64_t)k_seq_len * v_stride_s * es >= (1ll << 31)) return EN_ERR_UNSUPPORTED;
+  // 32-bit byte offsets into V, advanced a tile at a time up to two tiles past the end
+  if (v_stride_s < 0 || ((int64_t)k_seq_len + 256) * v_stride_s * es >= (1ll << 31)) return EN_ERR_UNSUPPORTED;
   AttnArgs a{};
   a.a_ptr = p; a.b_ptr = v; a.out = ctx; a.k_lens = k_lens; a.q_lens = q_lens;
   a.B = batch; a.H = head_num; a.Sq = q_seq_len; a.Sk = k_seq_len; a.D = size_per_head;

@@ -345,8 +345,9 @@ extern "C" int en_attn_fused(const void *q, const void *k, const void *v, void *
     if ((q_strides[i] % 8) || (k_strides[i] % 8) || (v_strides[i] % 8) || (c_strides[i] % 4)) return EN_ERR_ALIGN;
     if (q_strides[i] < 0 || k_strides[i] < 0 || v_strides[i] < 0 || c_strides[i] < 0) return EN_ERR_UNSUPPORTED;
   }
-  if ((int64_t)q_seq_len * q_strides[2] * 2 >= (1ll << 31) || (int64_t)k_seq_len * k_strides[2] * 2 >= (1ll << 31) ||
-      (int64_t)k_seq_len * v_strides[2] * 2 >= (1ll << 31))
+  // 32-bit byte offsets, advanced a tile at a time up to two tiles past the end
+  if ((int64_t)q_seq_len * q_strides[2] * 2 >= (1ll << 31) || ((int64_t)k_seq_len + 256) * k_strides[2] * 2 >= (1ll << 31) ||
+      ((int64_t)k_seq_len + 256) * v_strides[2] * 2 >= (1ll << 31))
     return EN_ERR_UNSUPPORTED;
   FusedArgs fa{};
   AttnArgs &a = fa.base;
