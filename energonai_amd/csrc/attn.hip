@@ -180,6 +180,162 @@ __global__ __launch_bounds__(kBlock) void attn_qk_kernel(AttnArgs a) {
 }
 
 // ===========================================================================
+// scores = alpha * Q K^T, 16-bit operands with 16-byte aligned score rows.
+//
+// Wave w of the workgroup owns queries 32w..32w+31 of a 128-query tile and computes
+// S^T = K Q^T for 64 keys at a time: Q fragments stay in registers, K tiles are shared
+// through LDS, double-buffered and fetched one tile ahead, which leaves ONE barrier per
+// tile.  The 32x64 result of a wave is turned into row-major order through a strip of LDS
+// that belongs to that wave alone (no workgroup barrier: a wave's LDS operations complete
+// in order) and leaves as whole 128-byte row segments.  The loads of the next K tile and
+// the stores of this tile are issued in the same iteration, before the only wait on the
+// loads, so the stores are never waited for.
+// ===========================================================================
+template <int DT, int DP, bool STREAM>
+__global__ __launch_bounds__(kBlock, 3) void attn_qk_strip_kernel(AttnArgs a) {
+  static_assert(DT != EN_F32, "16-bit storage only");
+  typedef Elem<DT> E;
+  typedef typename E::T T;
+  typedef Mma<DT> M;
+  constexpr int EPV = 8;
+  constexpr int BK = 64;                         // keys per tile
+  constexpr int KB = BK / 32;                    // 32-key MFMA blocks per tile
+  constexpr int NVS = DP / 16;                   // MFMA steps over the head dim
+  constexpr int KPITCH = DP + EPV;               // LDS pitch of a K row
+  constexpr int CPITCH = BK + EPV;               // LDS pitch of a score row in a wave's strip
+  constexpr int KVEC_ROW = DP / EPV;
+  constexpr int KLOADS = BK * KVEC_ROW / kBlock;
+  constexpr int CVEC_ROW = BK / EPV;             // 128-bit vectors per score row of a tile
+  constexpr int CSTORES = 32 * CVEC_ROW / kWave; // vectors each lane stores per tile
+  static_assert(BK * KVEC_ROW % kBlock == 0, "K tile must divide over the block");
+  __shared__ __attribute__((aligned(16))) T lds_k[2][BK * KPITCH];
+  __shared__ __attribute__((aligned(16))) T lds_c[kBlock / kWave][32 * CPITCH];
+
+  int unit, qi;
+  if (!map_block(a, unit, qi)) return;
+  const int b = unit / a.H, h = unit % a.H;
+  int kl, ql;
+  seq_extents(a, b, kl, ql);
+  const int q0 = qi * kQTile;
+  if (q0 >= ql) return;
+  const int nk = tile_key_extent(a, min(q0 + kQTile, ql) - 1, kl, ql);
+  if (nk <= 0) return;
+  const int nkt = (nk + BK - 1) / BK;
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int r = lane & 31, g = lane >> 5;
+  const int qw = q0 + wave * 32;                 // first query of this wave
+  const int q = qw + r;                          // query whose scores this lane accumulates
+
+  const T *qbase = reinterpret_cast<const T *>(a.a_ptr) + (int64_t)b * a.q_sb + (int64_t)h * a.q_sh;
+  const T *kbase = reinterpret_cast<const T *>(a.b_ptr) + (int64_t)b * a.k_sb + (int64_t)h * a.k_sh;
+  T *sbase = reinterpret_cast<T *>(a.out) + ((int64_t)unit * a.Sq) * a.Sk;
+
+  // Q fragments (B operand): this lane's query row, 8 channels per step; rows >= ql read as zero
+  uint4 qf[NVS];
+  {
+    const rsrc_t q_rsrc = make_rsrc(qbase, (uint32_t)(((int64_t)(ql - 1) * a.q_ss + a.D) * E::kSize));
+#pragma unroll
+    for (int vs = 0; vs < NVS; ++vs) {
+      const int d = M::k_of(vs, g, NVS);
+      const uint32_t off = (uint32_t)(((int64_t)q * a.q_ss + d) * E::kSize);
+      qf[vs] = buffer_load16(q_rsrc, (q < ql && d < a.D) ? off : kOutOfRange);
+    }
+  }
+
+  // K rows past the last valid key read as zeros through the bounds check (no traffic, no branches);
+  // lanes whose channel chunk lies past the head size sit at an offset that stays out of range
+  const rsrc_t k_rsrc = make_rsrc(kbase, (uint32_t)(((int64_t)(kl - 1) * a.k_ss + a.D) * E::kSize));
+  const rsrc_t s_rsrc = make_rsrc(sbase, (uint32_t)((int64_t)ql * a.Sk * E::kSize));   // rows >= ql are dropped
+  const uint32_t k_row_bytes = (uint32_t)(a.k_ss * E::kSize);
+  const int k_row = tid / KVEC_ROW, k_c = tid % KVEC_ROW;
+  uint32_t k_off = (k_c * EPV < a.D) ? k_row * k_row_bytes + k_c * EPV * E::kSize : kOutOfRange;
+  uint4 kreg[KLOADS];
+  auto fetch_k = [&]() {
+#pragma unroll
+    for (int i = 0; i < KLOADS; ++i) kreg[i] = buffer_load16(k_rsrc, k_off + i * (kBlock / KVEC_ROW) * k_row_bytes);
+    k_off += BK * k_row_bytes;
+  };
+  auto stage_k = [&](T *kdst) {
+#pragma unroll
+    for (int i = 0; i < KLOADS; ++i)
+      *reinterpret_cast<uint4 *>(&kdst[(k_row + i * (kBlock / KVEC_ROW)) * KPITCH + k_c * EPV]) = kreg[i];
+  };
+
+  // where this lane's vectors of the strip go: row sr + 8i of the wave's 32 rows, 8 keys at column sc
+  T *strip = lds_c[wave];
+  const int sr = lane / CVEC_ROW, sc = (lane % CVEC_ROW) * EPV;
+  int k_end[CSTORES];          // only vectors holding a key the row may see are written
+  uint32_t s_off[CSTORES];
+#pragma unroll
+  for (int i = 0; i < CSTORES; ++i) {
+    const int row = qw + sr + i * (kWave / CVEC_ROW);
+    k_end[i] = min(a.causal ? min(kl, row + (kl - ql) + 1) : kl, a.Sk);
+    s_off[i] = (uint32_t)(((int64_t)row * a.Sk + sc) * E::kSize);
+  }
+
+  fetch_k();
+  stage_k(lds_k[0]);
+  lds_barrier();
+  for (int kt = 0; kt < nkt; ++kt) {
+    const int k0 = kt * BK;
+    const T *ksrc = lds_k[kt & 1];
+    fetch_k();                                   // next tile (past the end: out of range, zeros)
+
+    floatx16 s[KB];
+#pragma unroll
+    for (int kb = 0; kb < KB; ++kb)
+#pragma unroll
+      for (int x = 0; x < 16; ++x) s[kb][x] = 0.f;
+    {
+      constexpr int NST = NVS / 2;               // K fragments are read two steps ahead of the MFMAs
+      uint4 kf[2][2][KB];
+      auto load_stage = [&](int st, uint4 (&dst)[2][KB]) {
+#pragma unroll
+        for (int u = 0; u < 2; ++u)
+#pragma unroll
+          for (int kb = 0; kb < KB; ++kb)
+            dst[u][kb] = *reinterpret_cast<const uint4 *>(&ksrc[(kb * 32 + r) * KPITCH + M::k_of(2 * st + u, g, NVS)]);
+      };
+      load_stage(0, kf[0]);
+#pragma unroll
+      for (int st = 0; st < NST; ++st) {
+        if (st + 1 < NST) load_stage(st + 1, kf[(st + 1) & 1]);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int u = 0; u < 2; ++u)
+#pragma unroll
+          for (int kb = 0; kb < KB; ++kb) M::step(kf[st & 1][u][kb], qf[2 * st + u], s[kb]);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    }
+
+    // register 4j+i of block kb holds key 32kb + 8j + 4g + i of query r: into the wave's strip, row-major
+#pragma unroll
+    for (int kb = 0; kb < KB; ++kb)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        Pack<T, 4> pk;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) pk.v[i] = E::from_float(s[kb][4 * j + i] * a.alpha);
+        store_pack<T, 4>(&strip[r * CPITCH + kb * 32 + 8 * j + 4 * g], pk);
+      }
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // the strip is this wave's own: no barrier needed
+#pragma unroll
+    for (int i = 0; i < CSTORES; ++i) {
+      const uint4 v = *reinterpret_cast<const uint4 *>(&strip[(sr + i * (kWave / CVEC_ROW)) * CPITCH + sc]);
+      const uint32_t off = s_off[i] + (uint32_t)(k0 * E::kSize);
+      buffer_store16<STREAM ? 2 : 0>(s_rsrc, (k0 + sc < k_end[i]) ? off : kOutOfRange, v);
+    }
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // strip read out before the next tile overwrites it
+
+    stage_k(lds_k[(kt + 1) & 1]);                // waits for the loads of this iteration only
+    lds_barrier();
+  }
+}
+
+// ===========================================================================
 // ctx = P V
 // ===========================================================================
 template <int DT, int DP, bool VEC, bool STREAM>
@@ -366,6 +522,19 @@ static int launch_qk(AttnArgs &a, hipStream_t s) {
   const unsigned grid = (unsigned)(ceil_div(a.units, kXcds) * kXcds * a.ntq);
   // a score tensor too large to stay in the memory-side cache is written with the non-temporal policy
   const bool stream = (int64_t)a.units * a.Sq * a.Sk * Elem<DT>::kSize >= kStreamScoreBytes;
+  if constexpr (DT != EN_F32) {
+    if (a.vec_out) {   // 16-bit, aligned rows
+      if (a.D <= 64) {
+        if (stream) attn_qk_strip_kernel<DT, 64, true><<<grid, kBlock, 0, s>>>(a);
+        else attn_qk_strip_kernel<DT, 64, false><<<grid, kBlock, 0, s>>>(a);
+      } else {
+        if (stream) attn_qk_strip_kernel<DT, 128, true><<<grid, kBlock, 0, s>>>(a);
+        else attn_qk_strip_kernel<DT, 128, false><<<grid, kBlock, 0, s>>>(a);
+      }
+      EN_RETURN_IF_LAUNCH_FAILED();
+      return EN_OK;
+    }
+  }
   if (a.vec_out) {
     if (a.D <= 64) {
       if (stream) attn_qk_kernel<DT, 64, true, true><<<grid, kBlock, 0, s>>>(a);
@@ -433,7 +602,8 @@ int en_attn_qk(const void *q, const void *k, void *scores, const int32_t *k_lens
   if (!strides_vec_ok(q_stride_b, q_stride_h, q_stride_s, epv) ||
       !strides_vec_ok(k_stride_b, k_stride_h, k_stride_s, epv))
     return EN_ERR_ALIGN;
-  if (k_stride_s < 0 || (int64_t)k_seq_len * k_stride_s * es >= (1ll << 31)) return EN_ERR_UNSUPPORTED;
+  // 32-bit byte offsets into K, advanced a tile at a time up to two tiles past the end
+  if (k_stride_s < 0 || ((int64_t)k_seq_len + 256) * k_stride_s * es >= (1ll << 31)) return EN_ERR_UNSUPPORTED;
   AttnArgs a{};
   a.a_ptr = q; a.b_ptr = k; a.out = scores; a.k_lens = k_lens; a.q_lens = q_lens;
   a.B = batch; a.H = head_num; a.Sq = q_seq_len; a.Sk = k_seq_len; a.D = size_per_head;
