@@ -510,6 +510,179 @@ __global__ __launch_bounds__(kBlock) void attn_pv_kernel(AttnArgs a) {
   }
 }
 
+// ===========================================================================
+// ctx = P V, 16-bit operands with 16-byte aligned probability rows.
+//
+// Same strip form as QK^T above: wave w owns queries 32w..32w+31 and every channel,
+// O^T += V^T P^T per 64-key tile.  V tiles are shared through LDS (transposed, double-
+// buffered, fetched one tile ahead: one barrier per tile).  Each wave reads its own 32
+// probability rows with row-contiguous 128-bit loads, one tile ahead, and passes them
+// through a strip of LDS of its own to get the MFMA operand order; no barrier is involved.
+// ===========================================================================
+template <int DT, int DP, bool STREAM>
+__global__ __launch_bounds__(kBlock, 3) void attn_pv_strip_kernel(AttnArgs a) {
+  static_assert(DT != EN_F32, "16-bit storage only");
+  typedef Elem<DT> E;
+  typedef typename E::T T;
+  typedef Mma<DT> M;
+  constexpr int EPV = 8;
+  constexpr int BK = 64;                         // keys per tile
+  constexpr int NVS = BK / 16;                   // MFMA steps over a key tile
+  constexpr int DMT = DP / 32;                   // 32-channel MFMA tiles of the output
+  constexpr int VPITCH = BK + 4;                 // V^T rows: 34 dwords, conflict-free 64-bit accesses
+  constexpr int PPITCH = BK + EPV;               // probability rows in a wave's strip
+  constexpr int NQUAD = BK / 4, NCHUNK = DP / EPV;
+  constexpr int VUNITS = NQUAD * NCHUNK;         // (four keys, eight channels) units of a V tile
+  constexpr int PVEC_ROW = BK / EPV;
+  constexpr int PLOADS = 32 * PVEC_ROW / kWave;  // vectors each lane fetches per tile
+  static_assert(VUNITS <= kBlock, "one V unit per lane");
+  __shared__ __attribute__((aligned(16))) T lds_v[2][DP * VPITCH];
+  __shared__ __attribute__((aligned(16))) T lds_p[kBlock / kWave][32 * PPITCH];
+
+  int unit, qi;
+  if (!map_block(a, unit, qi)) return;
+  const int b = unit / a.H, h = unit % a.H;
+  int kl, ql;
+  seq_extents(a, b, kl, ql);
+  const int q0 = qi * kQTile;
+  const int tid = threadIdx.x;
+  T *cbase = reinterpret_cast<T *>(a.out) + (int64_t)b * a.q_sb + (int64_t)h * a.q_sh;
+
+  if (q0 >= ql) {
+    if (a.zero_padding) {  // whole tile is padding
+      const int rows = min(kQTile, a.Sq - q0);
+      for (int i = tid; i < rows * a.D; i += kBlock) {
+        const int row = i / a.D, d = i - row * a.D;
+        cbase[(int64_t)(q0 + row) * a.q_ss + d] = E::from_float(0.f);
+      }
+    }
+    return;
+  }
+  const int nk = tile_key_extent(a, min(q0 + kQTile, ql) - 1, kl, ql);
+  const int nkt = (nk + BK - 1) / BK;
+
+  const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int r = lane & 31, g = lane >> 5;
+  const int qw = q0 + wave * 32;                 // first query of this wave
+  const int q = qw + r;                          // query whose context this lane accumulates
+
+  const T *pbase = reinterpret_cast<const T *>(a.a_ptr) + ((int64_t)unit * a.Sq) * a.Sk;
+  const T *vbase = reinterpret_cast<const T *>(a.b_ptr) + (int64_t)b * a.k_sb + (int64_t)h * a.k_sh;
+  // rows of padded queries lie past the end of the resource and read as zero; so do V rows >= kl
+  const rsrc_t p_rsrc = make_rsrc(pbase, (uint32_t)((int64_t)ql * a.Sk * E::kSize));
+  const uint32_t v_bytes = kl > 0 ? (uint32_t)(((int64_t)(kl - 1) * a.k_ss + a.D) * E::kSize) : 0u;
+  const rsrc_t v_rsrc = make_rsrc(vbase, v_bytes);
+  const uint32_t v_row_bytes = (uint32_t)(a.k_ss * E::kSize);
+  const int v_c = (tid % 4) + 4 * (tid / (4 * NQUAD)), v_kq = (tid / 4) % NQUAD;
+  uint32_t v_off = (tid < VUNITS && v_c * EPV < a.D) ? v_kq * 4 * v_row_bytes + v_c * EPV * E::kSize : kOutOfRange;
+  uint4 vreg[4];
+  auto fetch_v = [&]() {
+#pragma unroll
+    for (int x = 0; x < 4; ++x) vreg[x] = buffer_load16(v_rsrc, v_off + x * v_row_bytes);
+    v_off += BK * v_row_bytes;
+  };
+  auto stage_v = [&](T *vdst) {
+    if (VUNITS == kBlock || tid < VUNITS) {
+      Pack<T, EPV> rows[4];
+#pragma unroll
+      for (int x = 0; x < 4; ++x) rows[x] = __builtin_bit_cast(Pack<T, EPV>, vreg[x]);
+#pragma unroll
+      for (int e = 0; e < EPV; ++e) {
+        Pack<T, 4> col;
+#pragma unroll
+        for (int x = 0; x < 4; ++x) col.v[x] = rows[x].v[e];
+        store_pack<T, 4>(&vdst[(v_c * EPV + e) * VPITCH + v_kq * 4], col);
+      }
+    }
+  };
+
+  // this lane's share of the wave's probability strip: row pr + 8i, eight keys at column pc
+  T *strip = lds_p[wave];
+  const int pr = lane / PVEC_ROW, pc = (lane % PVEC_ROW) * EPV;
+  uint32_t p_off[PLOADS];
+#pragma unroll
+  for (int i = 0; i < PLOADS; ++i)
+    p_off[i] = (uint32_t)(((int64_t)(qw + pr + i * (kWave / PVEC_ROW)) * a.Sk + pc) * E::kSize);
+  uint4 preg[PLOADS];
+  // keys at or past nk were never written by the softmax: they must not be read
+  auto fetch_p = [&](int kt) {
+    const int k0 = kt * BK;
+#pragma unroll
+    for (int i = 0; i < PLOADS; ++i)
+      preg[i] = buffer_load16<STREAM ? 2 : 0>(p_rsrc, (k0 + pc < nk) ? p_off[i] + (uint32_t)(k0 * E::kSize) : kOutOfRange);
+  };
+  auto stage_p = [&]() {
+#pragma unroll
+    for (int i = 0; i < PLOADS; ++i)
+      *reinterpret_cast<uint4 *>(&strip[(pr + i * (kWave / PVEC_ROW)) * PPITCH + pc]) = preg[i];
+  };
+
+  floatx16 o[DMT];
+#pragma unroll
+  for (int mt = 0; mt < DMT; ++mt)
+#pragma unroll
+    for (int x = 0; x < 16; ++x) o[mt][x] = 0.f;
+
+  fetch_v();
+  fetch_p(0);
+  stage_v(lds_v[0]);
+  stage_p();
+  lds_barrier();
+  for (int kt = 0; kt < nkt; ++kt) {
+    const T *vsrc = lds_v[kt & 1];
+    fetch_v();                                   // next tiles (past the end: out of range, no traffic)
+    fetch_p(kt + 1);
+
+    // B operands: keys 16vs + 8g .. +7 of this lane's query, out of the wave's own strip
+    uint4 pf[NVS];
+#pragma unroll
+    for (int vs = 0; vs < NVS; ++vs) pf[vs] = *reinterpret_cast<const uint4 *>(&strip[r * PPITCH + vs * 16 + 8 * g]);
+    // A operands: V^T at the same keys, read one step ahead of the MFMAs
+    uint4 va[2][DMT];
+    auto load_step = [&](int vs, uint4 (&dst)[DMT]) {
+#pragma unroll
+      for (int mt = 0; mt < DMT; ++mt) {
+        const T *vrow = &vsrc[(mt * 32 + r) * VPITCH + vs * 16 + 8 * g];
+        const uint2 lo = *reinterpret_cast<const uint2 *>(vrow);
+        const uint2 hi = *reinterpret_cast<const uint2 *>(vrow + 4);
+        dst[mt] = make_uint4(lo.x, lo.y, hi.x, hi.y);
+      }
+    };
+    load_step(0, va[0]);
+#pragma unroll
+    for (int vs = 0; vs < NVS; ++vs) {
+      if (vs + 1 < NVS) load_step(vs + 1, va[(vs + 1) & 1]);
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int mt = 0; mt < DMT; ++mt) M::step(va[vs & 1][mt], pf[vs], o[mt]);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // this wave has read its strip: it may be overwritten
+    stage_v(lds_v[(kt + 1) & 1]);
+    stage_p();
+    lds_barrier();
+  }
+
+  // register 4j+i of tile mt holds channel 32mt + 8j + 4g + i of this lane's query
+  if (q >= a.Sq) return;
+  const bool valid = q < ql;
+  if (!valid && !a.zero_padding) return;
+  T *crow = cbase + (int64_t)q * a.q_ss;
+#pragma unroll
+  for (int mt = 0; mt < DMT; ++mt)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int d = mt * 32 + 8 * j + 4 * g;
+      if (d < a.D) {
+        Pack<T, 4> pk;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) pk.v[i] = E::from_float(valid ? o[mt][4 * j + i] : 0.f);
+        store_pack<T, 4>(crow + d, pk);
+      }
+    }
+}
+
 // ---------------------------------------------------------------------------
 // host side
 // ---------------------------------------------------------------------------
@@ -556,6 +729,19 @@ static int launch_pv(AttnArgs &a, hipStream_t s) {
   const unsigned grid = (unsigned)(ceil_div(a.units, kXcds) * kXcds * a.ntq);
   // probabilities of a tensor too large to stay cached are read with the non-temporal policy
   const bool stream = (int64_t)a.units * a.Sq * a.Sk * Elem<DT>::kSize >= kStreamScoreBytes;
+  if constexpr (DT != EN_F32) {
+    if (a.vec_out) {   // 16-bit, aligned rows
+      if (a.D <= 64) {
+        if (stream) attn_pv_strip_kernel<DT, 64, true><<<grid, kBlock, 0, s>>>(a);
+        else attn_pv_strip_kernel<DT, 64, false><<<grid, kBlock, 0, s>>>(a);
+      } else {
+        if (stream) attn_pv_strip_kernel<DT, 128, true><<<grid, kBlock, 0, s>>>(a);
+        else attn_pv_strip_kernel<DT, 128, false><<<grid, kBlock, 0, s>>>(a);
+      }
+      EN_RETURN_IF_LAUNCH_FAILED();
+      return EN_OK;
+    }
+  }
   if (a.vec_out) {
     if (a.D <= 64) {
       if (stream) attn_pv_kernel<DT, 64, true, true><<<grid, kBlock, 0, s>>>(a);
