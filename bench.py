@@ -39,9 +39,9 @@ MFMA_PEAK_TFLOPS = {"f16": 2500.0, "bf16": 2500.0, "f32": 157.3}
 MEASURED_TRAFFIC_C2 = {
     "depad": 26.3e6,
     "transpose_pad": 114.9e6,
-    "attn_qk": 63.1e6,
+    "attn_qk": 59.5e6,
     "scale_mask_softmax_tiled": 82.2e6,
-    "attn_pv": 71.2e6,
+    "attn_pv": 71.3e6,
     "transpose_depad": 26.3e6,
     "layernorm_residual": 39.4e6,
     "attn_fused": 52.6e6,
