@@ -18,6 +18,7 @@ import torch
 
 from .kernel import (attn_fused, attn_fused_packed, attn_pv, attn_qk, decode_pv, decode_qk, depad, layer_norm_forward, scale_mask_softmax,
                      transpose_depad, transpose_pad)
+from . import _lib
 from .seqinfo import SeqInfo, seq_info
 
 
@@ -44,6 +45,9 @@ def padding_removal_layer(hidden_padded: torch.Tensor, qkv_packed: torch.Tensor,
     info = seq_info(seq_lens, B, hidden_padded.device)
     T = info.total if sum_seq is None else int(sum_seq)
     scale = float(D) ** -0.5 if scale is None else scale
+    if not keep:
+        return _layer_one_call(hidden_padded, qkv_packed, info, B, S, H, D, hid, T, gamma, beta, eps, scale, causal,
+                               left_padded, dense_out, fused_attention)
 
     x = depad(hidden_padded, B, info, left_padded=left_padded, sum_seq=T)
     if fused_attention == "packed":
@@ -67,6 +71,44 @@ def padding_removal_layer(hidden_padded: torch.Tensor, qkv_packed: torch.Tensor,
     y = layer_norm_forward(attn_out, gamma, beta, (hid,), eps, residual=x)
     if keep:
         return dict(x=x, qkv=qkv, probs=probs, ctx=ctx, ctx_packed=ctx_packed, y=y)
+    return y
+
+
+_FORMS = {False: 0, True: 1, "packed": 2}
+
+
+def _layer_one_call(hidden_padded, qkv_packed, info, B, S, H, D, hid, T, gamma, beta, eps, scale, causal, left_padded,
+                    dense_out, fused_attention):
+    """The same seven launches through ``en_padding_removal_layer``: one foreign call per step."""
+    dev, dt = hidden_padded.device, hidden_padded.dtype
+    form = _FORMS[fused_attention]
+    _lib.require_gpu(hidden_padded, "hidden_padded")
+    _lib.require_gpu(qkv_packed, "qkv_packed")
+    if qkv_packed.numel() != T * H * 3 * D or qkv_packed.dtype != dt:
+        raise RuntimeError("padding_removal_layer: qkv_packed must be [1,T,H,3D] of the activation dtype")
+    if gamma.dtype != dt or beta.dtype != dt or gamma.numel() != hid or beta.numel() != hid:
+        raise RuntimeError("padding_removal_layer: gamma and beta must be [hidden] of the activation dtype")
+    if dense_out is not None:
+        _lib.require_gpu(dense_out, "dense_out")
+        if dense_out.numel() != T * hid or dense_out.dtype != dt:
+            raise RuntimeError("padding_removal_layer: dense_out must be [1,T,hidden] of the activation dtype")
+    elif hid != H * D:
+        raise RuntimeError("padding_removal_layer: without dense_out the LayerNorm width must equal heads * size_per_head")
+    if form and dt == torch.float32:
+        raise RuntimeError("padding_removal_layer: fused attention is for float16 and bfloat16")
+    x = torch.empty((1, T, hid), dtype=dt, device=dev)
+    y = torch.empty((1, T, hid), dtype=dt, device=dev)
+    ctx_packed = torch.empty((1, T, H, D), dtype=dt, device=dev)
+    qkv = torch.empty((B, H, S, 3 * D), dtype=dt, device=dev) if form != 2 else None
+    ctx = torch.empty((B, H, S, D), dtype=dt, device=dev) if form != 2 else None
+    scores = torch.empty((B, H, S, S), dtype=dt, device=dev) if form == 0 else None
+    with _lib.device_guard(hidden_padded):
+        _lib.check(_lib.fn.en_padding_removal_layer(
+            hidden_padded.data_ptr(), qkv_packed.data_ptr(), _lib.ptr(dense_out), gamma.data_ptr(), beta.data_ptr(),
+            x.data_ptr(), _lib.ptr(qkv), _lib.ptr(scores), _lib.ptr(ctx), ctx_packed.data_ptr(), y.data_ptr(),
+            info.cu_seqlens.data_ptr(), info.lens.data_ptr(), B, S, H, D, hid, T, float(scale), float(eps),
+            int(bool(causal)), int(bool(left_padded)), form, _lib.dtype_tag(hidden_padded, "padding_removal_layer"),
+            _lib.stream_of(hidden_padded)), "padding_removal_layer")
     return y
 
 

@@ -221,6 +221,24 @@ int en_attn_fused(const void *q, const void *k, const void *v, void *ctx, const 
 
 /* ---- measurement helper ------------------------------------------------- */
 
+/* The whole step in one call: depad, transpose_pad, QK^T, scale_mask_softmax, PV,
+ * transpose_depad, residual + LayerNorm launched back to back on `stream`, each through
+ * its own entry point above (the sequence of examples/bert/bert.py:54-62,91-134 with the
+ * projections left to the caller).  One foreign call instead of seven for callers whose
+ * per-call overhead matters (Python: about 60 us for the seven).  The caller owns every
+ * buffer: x_packed [T,hid] (residual stream), qkv_padded [B,H,S,3D], scores [B,H,S,S],
+ * ctx [B,H,S,D], ctx_packed [T,H*D], y [T,hid].  dense_out [T,hid], if not NULL, is what
+ * the LayerNorm adds to x_packed instead of ctx_packed (the output projection lies between
+ * the two in a real layer).  attention_form: 0 = the three separate ops, 1 = en_attn_fused
+ * on the padded buffer (scores unused), 2 = en_attn_fused on the packed projections
+ * (qkv_padded, scores and ctx unused).  gamma/beta in the activation dtype. */
+int en_padding_removal_layer(const void *hidden_padded, const void *qkv_packed, const void *dense_out,
+                             const void *gamma, const void *beta, void *x_packed, void *qkv_padded, void *scores,
+                             void *ctx, void *ctx_packed, void *y, const int32_t *cu_seqlens,
+                             const int32_t *seq_lens, int batch, int max_seq_len, int head_num, int size_per_head,
+                             int64_t hidden, int64_t total_tokens, float scale, float eps, int causal,
+                             int left_padded, int attention_form, int dtype, en_stream_t stream);
+
 /* Plain device-to-device copy of nbytes (multiple of 16, 16-byte aligned) with
  * the same 128-bit access pattern the packing kernels use.  Used as the
  * bandwidth yardstick and to calibrate hardware byte counters. */

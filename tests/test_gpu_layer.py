@@ -184,3 +184,22 @@ def test_layer_c2_fused_attention(mode):
                                 acc_dtype=torch.float32)
     assert max_abs(got["ctx_packed"].cpu(), want["ctx_packed"]) <= 2e-3
     assert max_abs(got["y"].cpu(), want["y"]) <= 6e-3
+
+
+@pytest.mark.parametrize("name,form", [("c1", False), ("c2", False), ("c2", True), ("c2", "packed")])
+def test_layer_single_call_equals_the_op_by_op_sequence(name, form):
+    """padding_removal_layer without keep= goes through the one-call entry point of the library; it must give
+    bit for bit what the same ops give when called one by one."""
+    layer, wl = _mods()
+    w = wl.BY_NAME[name]
+    announce("layer one call", name, form)
+    inp = wl.make_inputs(w)
+    args = (inp["hidden_padded"].cuda(), inp["qkv_packed"].cuda(), inp["lens"].cuda(), w.heads, w.head_dim,
+            inp["gamma"].cuda(), inp["beta"].cuda(), 1e-5, w.scale, w.causal, w.left_padded)
+    dense = inp.get("dense_out")
+    dense = None if dense is None else dense.cuda()
+    steps = layer.padding_removal_layer(*args, dense_out=dense, keep=True, fused_attention=form)
+    once = layer.padding_removal_layer(*args, dense_out=dense, fused_attention=form)
+    assert torch.equal(once, steps["y"])
+    twice = layer.padding_removal_layer(*args, dense_out=dense, fused_attention=form, sum_seq=int(inp["lens"].sum()))
+    assert torch.equal(twice, once)
