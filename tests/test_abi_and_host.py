@@ -74,6 +74,25 @@ def test_entry_points_validate_before_launch():
     assert lib.en_layernorm_fwd(16, None, None, None, 32, None, 48, 64, 1, 8, 1e-5, 1, 0, None) == -3  # (f16 -> f32)
     assert lib.en_attn_qk(16, 32, 48, 64, None, 1, 1, 8, 8, 200, 0, 0, 200, 0, 0, 200, 1.0, 1, 1, None) == -5  # D > 128
     assert lib.en_copy_bytes(16, 32, 24, None) == -2                     # not a multiple of 16
+    # entry points added beside the reference's own surface
+    i64x3 = (ctypes.c_int64 * 3)(0, 64, 768)
+    assert lib.en_repad(None, 32, 48, 1, 1, 1, 2, 0, None) == -1
+    assert lib.en_repad(16, 32, 48, 1, 0, 1, 2, 0, None) == -2           # max_seq_len 0
+    assert lib.en_transpose_pad_heads(16, 32, 48, 1, 1, 4, 8, 6, 4, 2, None) == -2   # heads 4..7 of a 6-row source
+    assert lib.en_kv_append(16, 32, 48, 64, None, 1, 1, 1, 8, 8, 8, 8, 8, 8, 2, None) == -1
+    assert lib.en_kv_append(16, 32, 48, 64, 80, 1, 1, 1, 8, 8, 8, 8, 8, 8, 3, None) == -3   # element size 3
+    assert lib.en_attn_fused(16, 32, 48, 64, 80, None, 1, 1, 8, 8, 64, i64x3, i64x3, i64x3, i64x3, None, None, 1.0, 1, 0,
+                             None) == -3                                 # fp32 is not a fused-attention dtype
+    assert lib.en_attn_fused(16, 32, 48, 64, 80, None, 1, 1, 8, 8, 64, i64x3, i64x3, i64x3, i64x3, None, None, 0.0, 1, 1,
+                             None) == -5                                 # scale must be positive
+    assert lib.en_attn_fused(16, 32, 48, 64, 80, None, 1, 1, 8, 8, 200, i64x3, i64x3, i64x3, i64x3, None, None, 1.0, 1, 1,
+                             None) == -5                                 # head size above 128
+    assert lib.en_padding_removal_layer(16, 32, None, 48, 64, 80, 96, 112, 128, 144, 160, 176, 192, 1, 8, 2, 8, 16, 4,
+                                        1.0, 1e-5, 1, 0, 3, 1, None) == -5   # unknown attention form
+    assert lib.en_padding_removal_layer(16, 32, None, 48, 64, 80, 96, 112, 128, 144, 160, 176, 192, 1, 8, 2, 8, 32, 4,
+                                        1.0, 1e-5, 1, 0, 0, 1, None) == -2   # LayerNorm width 32 != 2 heads x 8, no dense_out
+    assert lib.en_padding_removal_layer(16, 32, None, 48, 64, 80, None, 112, 128, 144, 160, 176, 192, 1, 8, 2, 8, 16, 4,
+                                        1.0, 1e-5, 1, 0, 0, 1, None) == -1   # unfused form without the padded buffer
 
 
 def test_python_api_keeps_reference_names_and_signatures():
