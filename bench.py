@@ -200,6 +200,84 @@ def run_block(torch, w, steps, warmup):
             "speedup_vs_eager_padded": ms_ref / ms, "max_abs_diff_vs_eager_on_valid_rows": err}
 
 
+def run_block_decode(torch, w, steps, warmup):
+    """Incremental decode of one pre-LN OPT block at the decode workload's shape: prefill a left-padded batch
+    with first_cache=True, then time single-token steps.  Baseline: the same block with stock torch ops and a
+    padded [B,H,Smax,D] K/V cache (scatter of the new row, masked single-query attention over the whole cache)."""
+    import torch.nn.functional as F
+    from energonai_amd import workloads
+    from energonai_amd.model import Block1D
+    dev = torch.device("cuda")
+    B, hid, H, D = w.batch, w.heads * w.head_dim, w.heads, w.head_dim
+    lens = workloads.make_lens(w)
+    S = int(lens.max())
+    smax = w.seq + 64
+    g = torch.Generator().manual_seed(4000 + w.index)
+    blk = Block1D(hid, H, 4.0, activation=F.relu, dtype=w.dtype, max_seq_len=smax).to(dev)
+    with torch.no_grad():
+        for name, prm in blk.named_parameters():
+            if prm.dim() == 2:
+                prm.copy_((0.02 * torch.randn(prm.shape, generator=g)).to(w.dtype))
+        total = warmup + steps + 2
+        buf = torch.zeros(B, S + total, hid, dtype=w.dtype, device=dev)      # the padded batch, one column per step
+        valid = (torch.arange(S).view(1, S) >= (S - lens.view(B, 1))).to(dev)
+        buf[:, :S] = torch.randn(B, S, hid, device=dev, dtype=w.dtype) * valid.unsqueeze(-1)
+        buf[:, S:] = torch.randn(B, total, hid, device=dev, dtype=w.dtype)
+        lens_dev = lens.to(dev)
+        blk(buf[:, :S], seq_lens=lens_dev, first_cache=True)
+        torch.cuda.synchronize()
+        pos = [S]
+
+        def ours():
+            pos[0] += 1
+            return blk(buf[:, :pos[0]], first_cache=False)
+        for _ in range(warmup):
+            ours()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            ours()
+        torch.cuda.synchronize()
+        ms = (time.perf_counter() - t0) * 1e3 / steps
+
+        # baseline: padded cache [B,H,smax,D], positions as in the left-padded batch
+        at, mlp, n1, n2 = blk.attn, blk.mlp, blk.norm1, blk.norm2
+        kc = torch.randn(B, H, smax, D, device=dev, dtype=w.dtype)
+        vc = torch.randn(B, H, smax, D, device=dev, dtype=w.dtype)
+        cur = [S]
+        key_pos = torch.arange(smax, device=dev).view(1, 1, 1, smax)
+        first = (S - lens_dev).view(B, 1, 1, 1)
+
+        def ref():
+            x = buf[:, cur[0]:cur[0] + 1]
+            h = F.layer_norm(x, (hid,), n1.weight, n1.bias, n1.eps)
+            k, v, q = torch.chunk(at.query_key_value(h), 3, dim=-1)
+            kc[:, :, cur[0]] = k.view(B, H, D)
+            vc[:, :, cur[0]] = v.view(B, H, D)
+            cur[0] += 1
+            mask = ((key_pos >= first) & (key_pos < cur[0])).to(w.dtype)
+            sc = torch.matmul(q.view(B, H, 1, D) * (D ** -0.5), kc.transpose(-1, -2)) + (1.0 - mask) * -10000.0
+            pr = torch.softmax(sc, -1, dtype=torch.float).to(w.dtype)
+            ctx = torch.matmul(pr, vc).transpose(1, 2).reshape(B, 1, hid)
+            s1 = x + at.dense(ctx)
+            h2 = F.layer_norm(s1, (hid,), n2.weight, n2.bias, n2.eps)
+            return s1 + mlp.dense_2(F.relu(mlp.dense_1(h2)))
+        for _ in range(max(2, warmup // 2)):
+            ref()
+        torch.cuda.synchronize()
+        n_ref = max(5, steps // 2)
+        t0 = time.perf_counter()
+        for _ in range(n_ref):
+            ref()
+        torch.cuda.synchronize()
+        ms_ref = (time.perf_counter() - t0) * 1e3 / n_ref
+    del blk, buf, kc, vc
+    torch.cuda.empty_cache()
+    return {"shape": f"{w.name}: hidden {hid}, {H} heads, batch {B}, cached lengths {int(lens.min())}..{S}, one new token each",
+            "ms_per_step": ms, "tokens_per_s": B / (ms * 1e-3), "eager_padded_cache_ms_per_step": ms_ref,
+            "speedup_vs_eager_padded_cache": ms_ref / ms}
+
+
 # ---------------------------------------------------------------------------
 # one workload on the GPU
 # ---------------------------------------------------------------------------
@@ -515,6 +593,10 @@ def main(argv=None) -> int:
             except Exception as exc:
                 blocks[name] = {"error": str(exc)[:300]}
         out["model_block_prefill"] = blocks
+        try:
+            out["model_block_decode"] = run_block_decode(torch, workloads.BY_NAME["c5"], max(5, ns.steps // 2), 3)
+        except Exception as exc:
+            out["model_block_decode"] = {"error": str(exc)[:300]}
     if not ns.no_cpu:
         out["cpu_baseline"] = cpu_baseline(torch, w)
     else:
