@@ -1,13 +1,15 @@
 // The two attention contractions on the padded [B,H,S,*] layout, restricted to
 // the region softmax actually uses (valid query rows, visible keys):
 //
-//   scores = alpha * Q K^T      (attn_qk_kernel)
-//   ctx    = P V                (attn_pv_kernel)
+//   scores = alpha * Q K^T      (attn_qk_strip_kernel; attn_qk_kernel for fp32 / unaligned rows)
+//   ctx    = P V                (attn_pv_strip_kernel; attn_pv_kernel for fp32 / unaligned rows)
 //
-// Both run on the 32x32 MFMA of gfx950 (32x32x16 for fp16/bf16, 32x32x2 for
-// fp32) with fp32 accumulation.  A workgroup is four waves in a 2x2 arrangement
-// over a 128-query tile; the operand that is streamed (K tiles for QK^T, P and
-// V tiles for PV) is staged through LDS with coalesced 128-bit loads and the
+// All run on the 32x32 MFMA of gfx950 (32x32x16 for fp16/bf16, 32x32x2 for
+// fp32) with fp32 accumulation over a 128-query tile per workgroup of four
+// waves.  The strip kernels give each wave 32 queries and share only the K (or
+// V^T) tile through LDS, one barrier per tile; the general kernels arrange the
+// waves 2x2 over the tile and stage both operands and the result through LDS.
+// In both, the streamed operand arrives by coalesced 128-bit loads and the
 // next tile is prefetched into registers while the current one is multiplied.
 //
 // The MFMA result layout has lanes running along the N operand and registers

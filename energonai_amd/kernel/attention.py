@@ -40,7 +40,7 @@ def attn_qk(q, k, seq_len_list, *, alpha: float = 1.0, causal: bool = True, q_le
             out: Optional[torch.Tensor] = None):
     """scores[b,h,i,j] = alpha * <q[b,h,i,:], k[b,h,j,:]> as a new ``[B,H,Sq,Sk]`` tensor.
 
-    Only rows of valid queries and (rounded up to the 128-key tile) the keys
+    Only rows of valid queries and (rounded up to a 16-byte vector) the keys
     they can see are written; the rest of ``scores`` is uninitialised, exactly
     the region ``scale_mask_softmax`` never reads.
     """
