@@ -346,6 +346,20 @@ def run_workload(torch, w, steps, warmup, want_eager=True, want_kernels=True):
         torch.cuda.synchronize()
         res["packed_fused_attention_ms_per_step"] = (time.perf_counter() - t0) * 1e3 / steps
 
+        def step_folded():
+            return layer.padding_removal_layer(d["hidden_padded"], d["qkv_packed"], info, w.heads, w.head_dim,
+                                               d["gamma"], d["beta"], workloads.EPS, w.scale, w.causal,
+                                               w.left_padded, dense_out=d["dense_out"], sum_seq=tokens,
+                                               fused_attention="packed", fold_depad=True)
+        for _ in range(max(2, warmup // 2)):
+            step_folded()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            step_folded()
+        torch.cuda.synchronize()
+        res["packed_fused_folded_depad_ms_per_step"] = (time.perf_counter() - t0) * 1e3 / steps
+
     # the same step replayed from a HIP graph (launch overhead removed); reported, never the headline
     try:
         g = torch.cuda.CUDAGraph()
@@ -572,6 +586,7 @@ def main(argv=None) -> int:
         "graph_ms_per_step": head.get("graph_ms_per_step"),
         "fused_attention_ms_per_step": head.get("fused_attention_ms_per_step"),
         "packed_fused_attention_ms_per_step": head.get("packed_fused_attention_ms_per_step"),
+        "packed_fused_folded_depad_ms_per_step": head.get("packed_fused_folded_depad_ms_per_step"),
         "eager_gpu_ms_per_step": head.get("eager_gpu_ms_per_step"),
         "speedup_vs_eager_gpu": head.get("speedup_vs_eager_gpu"),
         "kernels": kt,

@@ -12,10 +12,12 @@ extern "C" int en_padding_removal_layer(const void *hidden_padded, const void *q
                                         const int32_t *cu_seqlens, const int32_t *seq_lens, int batch,
                                         int max_seq_len, int head_num, int size_per_head, int64_t hidden,
                                         int64_t total_tokens, float scale, float eps, int causal, int left_padded,
-                                        int attention_form, int dtype, en_stream_t stream) {
+                                        int attention_form, const int32_t *fold_depad_offsets, int dtype,
+                                        en_stream_t stream) {
   using namespace en;
-  if (!hidden_padded || !qkv_packed || !gamma || !beta || !x_packed || !ctx_packed || !y || !cu_seqlens || !seq_lens)
+  if (!hidden_padded || !qkv_packed || !gamma || !beta || !ctx_packed || !y || !cu_seqlens || !seq_lens)
     return EN_ERR_NULL;
+  if (!x_packed && !fold_depad_offsets) return EN_ERR_NULL;
   if (attention_form < 0 || attention_form > 2) return EN_ERR_UNSUPPORTED;
   if (attention_form != 2 && (!qkv_padded || !ctx)) return EN_ERR_NULL;
   if (attention_form == 0 && !scores) return EN_ERR_NULL;
@@ -25,8 +27,11 @@ extern "C" int en_padding_removal_layer(const void *hidden_padded, const void *q
   if (!dense_out && hidden != (int64_t)head_num * size_per_head) return EN_ERR_SHAPE;
   if (total_tokens == 0) return EN_OK;
   const int B = batch, S = max_seq_len, H = head_num, D = size_per_head;
-  int rc = en_depad(hidden_padded, x_packed, cu_seqlens, B, S, hidden, es, left_padded, stream);
-  if (rc) return rc;
+  int rc = EN_OK;
+  if (!fold_depad_offsets) {
+    rc = en_depad(hidden_padded, x_packed, cu_seqlens, B, S, hidden, es, left_padded, stream);
+    if (rc) return rc;
+  }
   const unsigned char *qkv_bytes = static_cast<const unsigned char *>(qkv_padded);
   if (attention_form == 2) {
     // fused attention on the packed projections: no padded tensor at all
@@ -63,6 +68,8 @@ extern "C" int en_padding_removal_layer(const void *hidden_padded, const void *q
     rc = en_transpose_depad(ctx, ctx_packed, cu_seqlens, B, S, H, D, es, stream);
     if (rc) return rc;
   }
-  return en_layernorm_fwd(y, nullptr, nullptr, nullptr, dense_out ? dense_out : ctx_packed, x_packed, gamma, beta,
-                          total_tokens, hidden, eps, dtype, dtype, stream);
+  // with the offsets the residual rows come straight out of the padded activations: no depad copy at all
+  return en_layernorm_fwd(y, nullptr, nullptr, nullptr, dense_out ? dense_out : ctx_packed,
+                          fold_depad_offsets ? hidden_padded : x_packed, fold_depad_offsets, gamma, beta, total_tokens,
+                          hidden, eps, dtype, dtype, stream);
 }

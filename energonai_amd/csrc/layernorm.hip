@@ -20,6 +20,7 @@ struct LnArgs {
   void *sum_out;
   const void *in;
   const void *residual;
+  const int32_t *res_off;   // residual row of output row t is t + res_off[t] (null: t)
   const void *gamma;
   const void *beta;
   int64_t n1;
@@ -47,7 +48,7 @@ __global__ __launch_bounds__(TPR < kBlock ? kBlock : TPR) void layernorm_rows_ke
 
   const int nvec = a.n2 / EPV;
   const TI *in = reinterpret_cast<const TI *>(a.in) + row * a.n2;
-  const TI *res = a.residual ? reinterpret_cast<const TI *>(a.residual) + row * a.n2 : nullptr;
+  const TI *res = a.residual ? reinterpret_cast<const TI *>(a.residual) + (row + (a.res_off ? a.res_off[row] : 0)) * a.n2 : nullptr;
   TI *sum_out = a.sum_out ? reinterpret_cast<TI *>(a.sum_out) + row * a.n2 : nullptr;
 
   float x[VPL][EPV];
@@ -129,7 +130,7 @@ __global__ __launch_bounds__(kBlock) void layernorm_generic_kernel(LnArgs a) {
   __shared__ float s_b[kBlock / kWave];
   const int64_t row = blockIdx.x;
   const TI *in = reinterpret_cast<const TI *>(a.in) + row * a.n2;
-  const TI *res = a.residual ? reinterpret_cast<const TI *>(a.residual) + row * a.n2 : nullptr;
+  const TI *res = a.residual ? reinterpret_cast<const TI *>(a.residual) + (row + (a.res_off ? a.res_off[row] : 0)) * a.n2 : nullptr;
   TI *sum_out = a.sum_out ? reinterpret_cast<TI *>(a.sum_out) + row * a.n2 : nullptr;
   float s = 0.f;
   for (int i = threadIdx.x; i < a.n2; i += kBlock) {
@@ -206,8 +207,9 @@ static int dispatch(const LnArgs &a, hipStream_t s) {
 }  // namespace en
 
 extern "C" int en_layernorm_fwd(void *out, float *mean, float *invvar, void *sum_out, const void *in,
-                                const void *residual, const void *gamma, const void *beta, int64_t n1, int64_t n2,
-                                float eps, int in_dtype, int out_dtype, en_stream_t stream) {
+                                const void *residual, const int32_t *residual_row_offsets, const void *gamma,
+                                const void *beta, int64_t n1, int64_t n2, float eps, int in_dtype, int out_dtype,
+                                en_stream_t stream) {
   using namespace en;
   if (!out || !in || !gamma || !beta) return EN_ERR_NULL;
   if (n1 < 0 || n2 < 1 || n2 > (int64_t)INT32_MAX) return EN_ERR_SHAPE;
@@ -217,7 +219,8 @@ extern "C" int en_layernorm_fwd(void *out, float *mean, float *invvar, void *sum
   if (!aligned_to(in, esi) || !aligned_to(out, eso) || !aligned_to(gamma, eso) || !aligned_to(beta, eso) ||
       (residual && !aligned_to(residual, esi)) || (sum_out && !aligned_to(sum_out, esi)))
     return EN_ERR_ALIGN;
-  LnArgs a{out, mean, invvar, sum_out, in, residual, gamma, beta, n1, (int)n2, eps};
+  if (residual_row_offsets && !residual) return EN_ERR_NULL;
+  LnArgs a{out, mean, invvar, sum_out, in, residual, residual_row_offsets, gamma, beta, n1, (int)n2, eps};
   hipStream_t s = (hipStream_t)stream;
   if (in_dtype == EN_F32 && out_dtype == EN_F32) return dispatch<EN_F32, EN_F32>(a, s);
   if (in_dtype == EN_F32 && out_dtype == EN_F16) return dispatch<EN_F32, EN_F16>(a, s);

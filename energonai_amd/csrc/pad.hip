@@ -290,7 +290,7 @@ static int launch_row_gather(int64_t row_bytes, int64_t tile_dim_rows, int64_t o
 // ---------------------------------------------------------------------------
 __global__ __launch_bounds__(kBlock) void ft_build_offsets_kernel(const int32_t *__restrict__ lens, int batch,
                                                                   int max_seq_len, int32_t *__restrict__ valid,
-                                                                  int32_t *__restrict__ tmp_off) {
+                                                                  int32_t *__restrict__ tmp_off, int left_padded) {
   __shared__ int32_t s_tok[kBlock / kWave];
   __shared__ int32_t s_pad[kBlock / kWave];
   const int b = blockIdx.x;
@@ -315,11 +315,12 @@ __global__ __launch_bounds__(kBlock) void ft_build_offsets_kernel(const int32_t 
   tok = s_tok[0] + s_tok[1] + s_tok[2] + s_tok[3];
   pad = s_pad[0] + s_pad[1] + s_pad[2] + s_pad[3];
   if (b == 0) {
-    if (tid == 0) valid[0] = tok;
+    if (tid == 0 && valid) valid[0] = tok;
     tok = 0;
     pad = 0;
   }
   const int32_t n = lens[b];
+  if (left_padded) pad += max_seq_len - n;   // a left-padded sequence starts behind its own padding as well
   for (int j = tid; j < n; j += kBlock) tmp_off[tok + j] = pad;
 }
 
@@ -401,7 +402,17 @@ int en_ft_build_offsets(const int32_t *seq_lens, int batch, int max_seq_len, int
   if (!seq_lens || !valid_word_num || !tmp_mask_offset) return EN_ERR_NULL;
   if (batch < 1 || max_seq_len < 1) return EN_ERR_SHAPE;
   ft_build_offsets_kernel<<<batch, kBlock, 0, (hipStream_t)stream>>>(seq_lens, batch, max_seq_len, valid_word_num,
-                                                                      tmp_mask_offset);
+                                                                      tmp_mask_offset, 0);
+  EN_RETURN_IF_LAUNCH_FAILED();
+  return EN_OK;
+}
+
+int en_padding_offsets(const int32_t *seq_lens, int batch, int max_seq_len, int left_padded, int32_t *row_offsets,
+                       en_stream_t stream) {
+  if (!seq_lens || !row_offsets) return EN_ERR_NULL;
+  if (batch < 1 || max_seq_len < 1) return EN_ERR_SHAPE;
+  ft_build_offsets_kernel<<<batch, kBlock, 0, (hipStream_t)stream>>>(seq_lens, batch, max_seq_len, nullptr, row_offsets,
+                                                                      left_padded ? 1 : 0);
   EN_RETURN_IF_LAUNCH_FAILED();
   return EN_OK;
 }

@@ -46,11 +46,14 @@ def _check_shapes(input, normalized_shape, weight, bias):
 
 
 def layer_norm_forward(input, weight, bias, normalized_shape, eps=1e-5, residual=None, return_stats=False,
-                       return_sum=False):
+                       return_sum=False, residual_row_offsets=None):
     """forward_affine of the reference extension (csrc/layer_norm_cuda.cpp:82-103) plus a fused residual.
 
     Returns ``output`` (dtype of ``weight``), or a tuple
     ``(output[, mean, invvar][, sum])`` when the optional results are asked for.
+    With ``residual_row_offsets`` (int32 ``[n1]`` on the device, ``SeqInfo.row_offsets``) the residual of row
+    ``t`` is row ``t + offsets[t]`` of ``residual``, i.e. it is read straight from the padded ``[B,S,hid]``
+    activations and no depad copy is needed.
     """
     if isinstance(normalized_shape, numbers.Integral):
         normalized_shape = (normalized_shape,)
@@ -68,8 +71,12 @@ def layer_norm_forward(input, weight, bias, normalized_shape, eps=1e-5, residual
     res_ = None
     if residual is not None:
         _lib.require_gpu(residual, "residual", contiguous=False)
-        if residual.shape != input_.shape or residual.dtype != input_.dtype:
+        if residual.dtype != input_.dtype or (residual_row_offsets is None and residual.shape != input_.shape):
             raise RuntimeError("residual must match input in shape and dtype")
+        if residual_row_offsets is not None and (residual.shape[-1] != input_.shape[-1] or
+                                                 residual_row_offsets.numel() < n1 or
+                                                 residual_row_offsets.dtype != torch.int32):
+            raise RuntimeError("residual_row_offsets must be int32 [rows] and residual [.., hidden]")
         res_ = residual.contiguous()
     output = torch.empty_like(input_, dtype=weight_.dtype)
     mean = invvar = sum_out = None
@@ -81,7 +88,7 @@ def layer_norm_forward(input, weight, bias, normalized_shape, eps=1e-5, residual
     with _lib.device_guard(input_):
         _lib.check(_lib.fn.en_layernorm_fwd(
             output.data_ptr(), _lib.ptr(mean), _lib.ptr(invvar), _lib.ptr(sum_out), input_.data_ptr(),
-            _lib.ptr(res_), weight_.data_ptr(), bias_.data_ptr(), n1, n2, float(eps),
+            _lib.ptr(res_), _lib.ptr(residual_row_offsets), weight_.data_ptr(), bias_.data_ptr(), n1, n2, float(eps),
             _lib.dtype_tag(input_, "layer_norm"), _lib.dtype_tag(weight_, "layer_norm"),
             _lib.stream_of(input_)), "layer_norm")
     extra = ()

@@ -30,7 +30,7 @@ def padding_removal_layer(hidden_padded: torch.Tensor, qkv_packed: torch.Tensor,
                           size_per_head: int, gamma: torch.Tensor, beta: torch.Tensor, eps: float = 1e-5,
                           scale: Optional[float] = None, causal: bool = True, left_padded: bool = False,
                           dense_out: Optional[torch.Tensor] = None, sum_seq: Optional[int] = None,
-                          keep: bool = False, fused_attention=False):
+                          keep: bool = False, fused_attention=False, fold_depad: bool = False):
     """Runs the seven ops on ``hidden_padded`` [B,S,hid] and ``qkv_packed`` [1,T,H,3D].
 
     Returns the normalised ``[1,T,hid]`` output, or a dict of every
@@ -39,6 +39,8 @@ def padding_removal_layer(hidden_padded: torch.Tensor, qkv_packed: torch.Tensor,
     dtypes only); the score tensor is then never written.
     ``fused_attention="packed"`` also drops transpose_pad and transpose_depad:
     the fused kernel reads the packed projections and writes the packed context.
+    ``fold_depad=True`` drops the depad launch as well: the LayerNorm takes its
+    residual rows straight from ``hidden_padded`` (not with ``keep``).
     """
     B, S, hid = hidden_padded.shape
     H, D = head_num, size_per_head
@@ -47,7 +49,9 @@ def padding_removal_layer(hidden_padded: torch.Tensor, qkv_packed: torch.Tensor,
     scale = float(D) ** -0.5 if scale is None else scale
     if not keep:
         return _layer_one_call(hidden_padded, qkv_packed, info, B, S, H, D, hid, T, gamma, beta, eps, scale, causal,
-                               left_padded, dense_out, fused_attention)
+                               left_padded, dense_out, fused_attention, fold_depad)
+    if fold_depad:
+        raise RuntimeError("padding_removal_layer: fold_depad has no intermediates to keep")
 
     x = depad(hidden_padded, B, info, left_padded=left_padded, sum_seq=T)
     if fused_attention == "packed":
@@ -78,7 +82,7 @@ _FORMS = {False: 0, True: 1, "packed": 2}
 
 
 def _layer_one_call(hidden_padded, qkv_packed, info, B, S, H, D, hid, T, gamma, beta, eps, scale, causal, left_padded,
-                    dense_out, fused_attention):
+                    dense_out, fused_attention, fold_depad=False):
     """The same seven launches through ``en_padding_removal_layer``: one foreign call per step."""
     dev, dt = hidden_padded.device, hidden_padded.dtype
     form = _FORMS[fused_attention]
@@ -96,7 +100,8 @@ def _layer_one_call(hidden_padded, qkv_packed, info, B, S, H, D, hid, T, gamma, 
         raise RuntimeError("padding_removal_layer: without dense_out the LayerNorm width must equal heads * size_per_head")
     if form and dt == torch.float32:
         raise RuntimeError("padding_removal_layer: fused attention is for float16 and bfloat16")
-    x = torch.empty((1, T, hid), dtype=dt, device=dev)
+    x = None if fold_depad else torch.empty((1, T, hid), dtype=dt, device=dev)
+    offs = info.row_offsets(S, left_padded) if fold_depad else None
     y = torch.empty((1, T, hid), dtype=dt, device=dev)
     ctx_packed = torch.empty((1, T, H, D), dtype=dt, device=dev)
     qkv = torch.empty((B, H, S, 3 * D), dtype=dt, device=dev) if form != 2 else None
@@ -105,9 +110,10 @@ def _layer_one_call(hidden_padded, qkv_packed, info, B, S, H, D, hid, T, gamma, 
     with _lib.device_guard(hidden_padded):
         _lib.check(_lib.fn.en_padding_removal_layer(
             hidden_padded.data_ptr(), qkv_packed.data_ptr(), _lib.ptr(dense_out), gamma.data_ptr(), beta.data_ptr(),
-            x.data_ptr(), _lib.ptr(qkv), _lib.ptr(scores), _lib.ptr(ctx), ctx_packed.data_ptr(), y.data_ptr(),
+            _lib.ptr(x), _lib.ptr(qkv), _lib.ptr(scores), _lib.ptr(ctx), ctx_packed.data_ptr(), y.data_ptr(),
             info.cu_seqlens.data_ptr(), info.lens.data_ptr(), B, S, H, D, hid, T, float(scale), float(eps),
-            int(bool(causal)), int(bool(left_padded)), form, _lib.dtype_tag(hidden_padded, "padding_removal_layer"),
+            int(bool(causal)), int(bool(left_padded)), form, _lib.ptr(offs),
+            _lib.dtype_tag(hidden_padded, "padding_removal_layer"),
             _lib.stream_of(hidden_padded)), "padding_removal_layer")
     return y
 

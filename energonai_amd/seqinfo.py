@@ -22,7 +22,7 @@ _CACHE_SIZE = 16
 class SeqInfo:
     """Device-resident int32 lengths and exclusive prefix for one batch."""
 
-    __slots__ = ("lens", "cu_seqlens", "batch_size", "_total", "_source")
+    __slots__ = ("lens", "cu_seqlens", "batch_size", "_total", "_source", "_row_offsets")
 
     def __init__(self, lens: torch.Tensor, cu_seqlens: torch.Tensor, batch_size: int, total: Optional[int], source):
         self.lens = lens                # int32 [B] on the device
@@ -30,6 +30,7 @@ class SeqInfo:
         self.batch_size = batch_size
         self._total = total
         self._source = source           # keeps the caller's tensor alive while cached
+        self._row_offsets = {}          # (max_seq_len, left_padded) -> int32 [T]
 
     @property
     def device(self) -> torch.device:
@@ -43,6 +44,21 @@ class SeqInfo:
         if self._total is None:
             self._total = int(self.cu_seqlens[self.batch_size].item())
         return self._total
+
+
+    def row_offsets(self, max_seq_len: int, left_padded: bool) -> torch.Tensor:
+        """``off[t]`` = row of token ``t`` in the padded ``[B*S]`` numbering minus ``t``; computed once per
+        batch and bucket by one small kernel (the reference's ft offsets, csrc/transpose_pad_fusion_kernel.cu:
+        112-131, made aware of left padding)."""
+        key = (int(max_seq_len), bool(left_padded))
+        off = self._row_offsets.get(key)
+        if off is None:
+            off = torch.empty(max(self.total, 1), dtype=torch.int32, device=self.lens.device)
+            with _lib.device_guard(self.lens):
+                _lib.check(_lib.fn.en_padding_offsets(self.lens.data_ptr(), self.batch_size, key[0], int(key[1]),
+                                                      off.data_ptr(), _lib.stream_of(self.lens)), "padding_offsets")
+            self._row_offsets[key] = off
+        return off
 
 
 _cache: "OrderedDict[tuple, SeqInfo]" = OrderedDict()

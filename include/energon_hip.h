@@ -93,6 +93,13 @@ int en_transpose_depad(const void *src, void *dst, const int32_t *cu_seqlens, in
 int en_ft_build_offsets(const int32_t *seq_lens, int batch, int max_seq_len, int32_t *valid_word_num,
                         int32_t *tmp_mask_offset, en_stream_t stream);
 
+/* row_offsets[t] = (row of token t in the padded [B*S] numbering) - t, for right- or
+ * left-padded batches: the left-pad-aware form of the offsets above (the reference
+ * assumes right padding, kernel.cu:118-130, while its generation batches are padded on
+ * the left, examples/opt/batch.py:12-24).  row_offsets has sum(seq_lens) entries. */
+int en_padding_offsets(const int32_t *seq_lens, int batch, int max_seq_len, int left_padded, int32_t *row_offsets,
+                       en_stream_t stream);
+
 /* ft_remove_padding_wrapper (wrapper.cpp:113-139, kernel.cu:142-166):
  * tgt[t,:] = src[t + tmp_mask_offset[t],:]; also copies the offsets into
  * mask_offset. */
@@ -145,10 +152,13 @@ int en_scale_mask_softmax(void *src, const int32_t *k_lens, const int32_t *q_len
  * statistics, one rounding to out_dtype.  gamma/beta have out_dtype.
  * mean/invvar (fp32 [n1]) and sum_out (x rounded to in_dtype, [n1,n2]) are
  * optional (NULL to skip).  Supported (in,out): (f32,f32) (f32,f16) (f32,bf16)
- * (f16,f16) (bf16,bf16), the pairs of csrc/type_shim.h:26-73. */
+ * (f16,f16) (bf16,bf16), the pairs of csrc/type_shim.h:26-73.
+ * residual_row_offsets (device, n1 entries, or NULL): the residual of output row t is row
+ * t + residual_row_offsets[t] of `residual`, which lets the kernel take it straight from the
+ * padded [B,S,n2] activations (offsets from en_padding_offsets) instead of a depad copy. */
 int en_layernorm_fwd(void *out, float *mean, float *invvar, void *sum_out, const void *in, const void *residual,
-                     const void *gamma, const void *beta, int64_t n1, int64_t n2, float eps, int in_dtype,
-                     int out_dtype, en_stream_t stream);
+                     const int32_t *residual_row_offsets, const void *gamma, const void *beta, int64_t n1, int64_t n2,
+                     float eps, int in_dtype, int out_dtype, en_stream_t stream);
 
 /* ---- attention contractions (torch.matmul in the reference callers) ----- */
 
@@ -231,13 +241,16 @@ int en_attn_fused(const void *q, const void *k, const void *v, void *ctx, const 
  * the LayerNorm adds to x_packed instead of ctx_packed (the output projection lies between
  * the two in a real layer).  attention_form: 0 = the three separate ops, 1 = en_attn_fused
  * on the padded buffer (scores unused), 2 = en_attn_fused on the packed projections
- * (qkv_padded, scores and ctx unused).  gamma/beta in the activation dtype. */
+ * (qkv_padded, scores and ctx unused).  fold_depad_offsets (en_padding_offsets of this
+ * batch, or NULL): if given, depad is not run and x_packed may be NULL; the LayerNorm takes
+ * its residual rows straight from hidden_padded.  gamma/beta in the activation dtype. */
 int en_padding_removal_layer(const void *hidden_padded, const void *qkv_packed, const void *dense_out,
                              const void *gamma, const void *beta, void *x_packed, void *qkv_padded, void *scores,
                              void *ctx, void *ctx_packed, void *y, const int32_t *cu_seqlens,
                              const int32_t *seq_lens, int batch, int max_seq_len, int head_num, int size_per_head,
                              int64_t hidden, int64_t total_tokens, float scale, float eps, int causal,
-                             int left_padded, int attention_form, int dtype, en_stream_t stream);
+                             int left_padded, int attention_form, const int32_t *fold_depad_offsets, int dtype,
+                             en_stream_t stream);
 
 /* Plain device-to-device copy of nbytes (multiple of 16, 16-byte aligned) with
  * the same 128-bit access pattern the packing kernels use.  Used as the

@@ -71,7 +71,9 @@ def test_entry_points_validate_before_launch():
     assert lib.en_transpose_pad(16, 32, 48, 0, 1, 1, 1, 2, None) == -2   # batch 0
     assert lib.en_scale_mask_softmax(16, 32, None, 1, 1, 1, 1, 1.0, 1, 0, 7, None) == -3   # dtype tag 7
     assert lib.en_scale_mask_softmax(16, 32, None, 1, 1, 1, 1, 1.0, 1, 96, 1, None) == -2  # tile not a power of two
-    assert lib.en_layernorm_fwd(16, None, None, None, 32, None, 48, 64, 1, 8, 1e-5, 1, 0, None) == -3  # (f16 -> f32)
+    assert lib.en_layernorm_fwd(16, None, None, None, 32, None, None, 48, 64, 1, 8, 1e-5, 1, 0, None) == -3  # (f16 -> f32)
+    assert lib.en_layernorm_fwd(16, None, None, None, 32, None, 80, 48, 64, 1, 8, 1e-5, 1, 1, None) == -1   # offsets, no residual
+    assert lib.en_padding_offsets(16, 0, 8, 0, 32, None) == -2           # batch 0
     assert lib.en_attn_qk(16, 32, 48, 64, None, 1, 1, 8, 8, 200, 0, 0, 200, 0, 0, 200, 1.0, 1, 1, None) == -5  # D > 128
     assert lib.en_copy_bytes(16, 32, 24, None) == -2                     # not a multiple of 16
     # entry points added beside the reference's own surface
@@ -88,11 +90,11 @@ def test_entry_points_validate_before_launch():
     assert lib.en_attn_fused(16, 32, 48, 64, 80, None, 1, 1, 8, 8, 200, i64x3, i64x3, i64x3, i64x3, None, None, 1.0, 1, 1,
                              None) == -5                                 # head size above 128
     assert lib.en_padding_removal_layer(16, 32, None, 48, 64, 80, 96, 112, 128, 144, 160, 176, 192, 1, 8, 2, 8, 16, 4,
-                                        1.0, 1e-5, 1, 0, 3, 1, None) == -5   # unknown attention form
+                                        1.0, 1e-5, 1, 0, 3, None, 1, None) == -5   # unknown attention form
     assert lib.en_padding_removal_layer(16, 32, None, 48, 64, 80, 96, 112, 128, 144, 160, 176, 192, 1, 8, 2, 8, 32, 4,
-                                        1.0, 1e-5, 1, 0, 0, 1, None) == -2   # LayerNorm width 32 != 2 heads x 8, no dense_out
+                                        1.0, 1e-5, 1, 0, 0, None, 1, None) == -2   # LayerNorm width 32 != 2 heads x 8, no dense_out
     assert lib.en_padding_removal_layer(16, 32, None, 48, 64, 80, None, 112, 128, 144, 160, 176, 192, 1, 8, 2, 8, 16, 4,
-                                        1.0, 1e-5, 1, 0, 0, 1, None) == -1   # unfused form without the padded buffer
+                                        1.0, 1e-5, 1, 0, 0, None, 1, None) == -1   # unfused form without the padded buffer
 
 
 def test_python_api_keeps_reference_names_and_signatures():

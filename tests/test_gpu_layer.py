@@ -203,3 +203,36 @@ def test_layer_single_call_equals_the_op_by_op_sequence(name, form):
     assert torch.equal(once, steps["y"])
     twice = layer.padding_removal_layer(*args, dense_out=dense, fused_attention=form, sum_seq=int(inp["lens"].sum()))
     assert torch.equal(twice, once)
+
+
+@pytest.mark.parametrize("name,form", [("c1", False), ("c2", False), ("c2", "packed")])
+def test_layer_with_depad_folded_into_layernorm(name, form):
+    """fold_depad: no depad launch, the LayerNorm reads its residual rows from the padded activations through
+    per-token row offsets (right-padded c1, left-padded c2).  Same bits as the step with the depad copy."""
+    layer, wl = _mods()
+    w = wl.BY_NAME[name]
+    announce("layer fold depad", name, form)
+    inp = wl.make_inputs(w)
+    args = (inp["hidden_padded"].cuda(), inp["qkv_packed"].cuda(), inp["lens"].cuda(), w.heads, w.head_dim,
+            inp["gamma"].cuda(), inp["beta"].cuda(), 1e-5, w.scale, w.causal, w.left_padded)
+    dense = inp.get("dense_out")
+    dense = None if dense is None else dense.cuda()
+    plain = layer.padding_removal_layer(*args, dense_out=dense, fused_attention=form)
+    folded = layer.padding_removal_layer(*args, dense_out=dense, fused_attention=form, fold_depad=True)
+    assert torch.equal(folded, plain)
+
+
+@pytest.mark.parametrize("left", [True, False])
+def test_padding_offsets_against_closed_form(left):
+    from energonai_amd.seqinfo import seq_info
+    lens = [5, 0, 9, 1, 9]
+    B, S = len(lens), 9
+    announce("padding offsets", left)
+    info = seq_info(torch.tensor(lens, dtype=torch.int32).cuda(), B, torch.device("cuda"))
+    got = info.row_offsets(S, left).cpu().tolist()
+    want = []
+    for b, n in enumerate(lens):
+        for i in range(n):
+            row = b * S + (S - n if left else 0) + i
+            want.append(row - len(want))
+    assert got[:len(want)] == want
