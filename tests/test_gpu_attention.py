@@ -263,3 +263,49 @@ def test_attn_fused_matches_unfused_pipeline_on_c2_shape():
     ctx_b = k.attn_fused(q, kk, v, lens_t, causal=True)
     for b, n in enumerate(lens):
         assert max_abs(ctx_a[b, :, :n].cpu(), ctx_b[b, :, :n].cpu()) <= 3e-3
+
+
+@pytest.mark.parametrize("seed", list(range(12)))
+def test_attention_random_shapes(seed):
+    """Seeded random shapes (head sizes 32..128, buckets that are not multiples of the tiles, empty and
+    full sequences) through QK^T -> softmax -> PV and through the fused kernel, against the float64 oracle."""
+    k = _kernel()
+    g = torch.Generator().manual_seed(9000 + seed)
+    ri = lambda lo, hi: int(torch.randint(lo, hi + 1, (1,), generator=g))
+    B, H = ri(1, 5), ri(1, 4)
+    D = [32, 64, 80, 96, 128][ri(0, 4)]
+    S = 8 * ri(2, 60)
+    lens = [ri(0, S) for _ in range(B)]
+    lens[ri(0, B - 1)] = S
+    causal = bool(ri(0, 1))
+    dtype = [torch.float16, torch.bfloat16][ri(0, 1)]
+    announce("attn random", seed, B, H, S, D, lens, causal, dtype)
+    T = sum(lens)
+    qkv_packed = packed_randn(T, H * 3 * D, dtype, 500 + seed).reshape(T, H, 3 * D)
+    qkv = pad_bhsd(qkv_packed, lens, S, H, 3 * D)
+    q, kk, v = torch.chunk(qkv, 3, dim=-1)
+    lens_t = torch.tensor(lens, dtype=torch.int32).cuda()
+    qg, kg, vg = torch.chunk(qkv.cuda(), 3, dim=-1)
+    scale = D ** -0.5
+    scores = eager.attn_qk(q, kk, torch.float64)
+    probs = eager.scale_mask_softmax(B, S, H, scores, lens, scale=scale, causal=causal, acc_dtype=torch.float64,
+                                     out_dtype=torch.float64)
+    for b, n in enumerate(lens):
+        probs[b, :, n:] = 0
+    want = eager.attn_pv(probs, v, torch.float64)
+    s_gpu = k.attn_qk(qg, kg, lens_t, causal=causal)
+    p_gpu = k.scale_mask_softmax(B, S, H, s_gpu, lens_t, scale=scale, causal=causal, tail_rows=128)
+    ctx_a = k.attn_pv(p_gpu, vg, lens_t, causal=causal).cpu()
+    ctx_b = k.attn_fused(qg, kg, vg, lens_t, scale=scale, causal=causal).cpu()
+    ctx_c = k.attn_fused_packed(qkv_packed.reshape(1, T, H, 3 * D).cuda(), B, S, lens_t, H, D, scale=scale,
+                                causal=causal).cpu().reshape(T, H, D)
+    tol = {torch.float16: 3e-3, torch.bfloat16: 2e-2}[dtype]
+    t0 = 0
+    for b, n in enumerate(lens):
+        if n:
+            ref = want[b, :, :n]
+            bound = tol * max(1.0, float(ref.abs().max()))
+            assert max_abs(ctx_a[b, :, :n], ref) <= bound
+            assert max_abs(ctx_b[b, :, :n], ref) <= bound
+            assert max_abs(ctx_c[t0:t0 + n].permute(1, 0, 2), ref) <= bound
+        t0 += n
