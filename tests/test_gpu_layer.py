@@ -222,6 +222,53 @@ def test_layer_with_depad_folded_into_layernorm(name, form):
     assert torch.equal(folded, plain)
 
 
+@pytest.mark.parametrize("name,form", [("c1", False), ("c2", False), ("c2", "packed")])
+def test_layer_recorded_into_a_hip_graph_replays_the_eager_result(name, form):
+    """The step allocates through torch only and never synchronises, so a caller may record it into a HIP graph.
+    Each of three replays, with eager launches and synchronisations between them, must give the eager bits, and
+    new input written into the recorded buffers must be picked up."""
+    layer, wl = _mods()
+    from energonai_amd.seqinfo import seq_info
+    w = wl.BY_NAME[name]
+    announce("layer graph replay", name, form)
+    inp = wl.make_inputs(w)
+    dev = torch.device("cuda", 0)
+    hidden, qkv = inp["hidden_padded"].cuda(), inp["qkv_packed"].cuda()
+    gamma, beta = inp["gamma"].cuda(), inp["beta"].cuda()
+    dense = inp.get("dense_out")
+    dense = None if dense is None else dense.cuda()
+    info = seq_info(inp["lens"], w.batch, dev)       # lengths reach the device before the recording starts
+
+    def step():
+        return layer.padding_removal_layer(hidden, qkv, info, w.heads, w.head_dim, gamma, beta, 1e-5, w.scale,
+                                           w.causal, w.left_padded, dense_out=dense, sum_seq=inp["total"],
+                                           fused_attention=form)
+    eager_y = step().clone()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        step()
+    torch.cuda.current_stream().wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        y = step()
+    torch.cuda.synchronize()
+    for i in range(3):
+        y.fill_(7)
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(y, eager_y), f"replay {i}"
+        assert torch.equal(step(), eager_y)          # eager work between the replays
+        torch.cuda.synchronize()
+    hidden.mul_(0.5)
+    qkv.mul_(-1)
+    eager_y2 = step().clone()
+    graph.replay()
+    torch.cuda.synchronize()
+    assert torch.equal(y, eager_y2)
+    assert not torch.equal(eager_y2, eager_y)
+
+
 @pytest.mark.parametrize("left", [True, False])
 def test_padding_offsets_against_closed_form(left):
     from energonai_amd.seqinfo import seq_info
