@@ -309,3 +309,42 @@ def test_attention_random_shapes(seed):
             assert max_abs(ctx_b[b, :, :n], ref) <= bound
             assert max_abs(ctx_c[t0:t0 + n].permute(1, 0, 2), ref) <= bound
         t0 += n
+
+
+@pytest.mark.parametrize("causal", [True, False])
+def test_attention_long_bucket(causal):
+    """A 4096-token bucket (32 query tiles, 64 key tiles, 8 KiB score rows): the three routes against the fp32
+    oracle on one full-length and one short sequence."""
+    k = _kernel()
+    B, H, S, D = 2, 2, 4096, 128
+    lens = [4096, 777]
+    announce("attn long bucket", causal)
+    T = sum(lens)
+    qkv_packed = packed_randn(T, H * 3 * D, torch.float16, 4242).reshape(T, H, 3 * D)
+    qkv = pad_bhsd(qkv_packed, lens, S, H, 3 * D)
+    q, kk, v = torch.chunk(qkv, 3, dim=-1)
+    scale = D ** -0.5
+    scores = eager.attn_qk(q, kk, torch.float32)
+    probs = eager.scale_mask_softmax(B, S, H, scores, lens, scale=scale, causal=causal, acc_dtype=torch.float32,
+                                     out_dtype=torch.float32)
+    for b, n in enumerate(lens):
+        probs[b, :, n:] = 0
+    want = eager.attn_pv(probs, v, torch.float32)
+    lens_t = torch.tensor(lens, dtype=torch.int32).cuda()
+    qg, kg, vg = torch.chunk(qkv.cuda(), 3, dim=-1)
+    s_gpu = k.attn_qk(qg, kg, lens_t, causal=causal)
+    p_gpu = k.scale_mask_softmax(B, S, H, s_gpu, lens_t, scale=scale, causal=causal, tail_rows=128)
+    for b, n in enumerate(lens):      # rows of probabilities sum to one over the keys of the sequence
+        rows = p_gpu[b, :, :n, :n].float().sum(-1)
+        assert float((rows - 1).abs().max()) <= 4e-3
+    ctx_a = k.attn_pv(p_gpu, vg, lens_t, causal=causal).cpu()
+    ctx_b = k.attn_fused(qg, kg, vg, lens_t, scale=scale, causal=causal).cpu()
+    ctx_c = k.attn_fused_packed(qkv_packed.reshape(1, T, H, 3 * D).cuda(), B, S, lens_t, H, D, scale=scale,
+                                causal=causal).cpu().reshape(T, H, D)
+    t0 = 0
+    for b, n in enumerate(lens):
+        ref = want[b, :, :n]
+        assert max_abs(ctx_a[b, :, :n], ref) <= 2e-3
+        assert max_abs(ctx_b[b, :, :n], ref) <= 2e-3
+        assert max_abs(ctx_c[t0:t0 + n].permute(1, 0, 2), ref) <= 2e-3
+        t0 += n
