@@ -43,7 +43,8 @@ extern "C" int en_padding_removal_layer(const void *hidden_padded, const void *q
                        stream);
     if (rc) return rc;
   } else {
-    rc = en_transpose_pad(qkv_packed, qkv_padded, cu_seqlens, B, S, H, 3 * D, es, stream);
+    // the attention entry points never read a row at or past a sequence's length: no zero fill of the padding
+    rc = en_transpose_pad_heads(qkv_packed, qkv_padded, cu_seqlens, B, S, H, 3 * D, H, 0, 0, es, stream);
     if (rc) return rc;
     // q, k, v are the thirds of the last dimension of the padded [B,H,S,3D] buffer
     const int64_t sb = (int64_t)H * S * 3 * D, sh = (int64_t)S * 3 * D, ss = 3 * D;

@@ -37,14 +37,15 @@ struct Ptrs3 {
 // which rows h0..h0+H-1 are taken): one third of a fused projection output, say.
 struct PadMap {
   const int32_t *cu;
-  int H, S, R, Hs, h0;
-  __device__ bool active(int, int) const { return true; }
+  int H, S, R, Hs, h0, zero;
+  // without the zero fill, tiles that lie wholly in the padding of their sequence have nothing to write
+  __device__ bool active(int tx, int b) const { return zero || (tx / H) * R < cu[b + 1] - cu[b]; }
   __device__ void operator()(int tx, int b, int r, int64_t &src, int64_t &dst) const {
     const int h = tx % H;
     const int s = (tx / H) * R + r;
     const int start = cu[b];
     const int len = cu[b + 1] - start;
-    dst = (s < S) ? ((int64_t)b * H + h) * S + s : kSkipRow;
+    dst = (s < S && (zero || s < len)) ? ((int64_t)b * H + h) * S + s : kSkipRow;
     src = (s < len) ? ((int64_t)(start + s)) * Hs + h0 + h : kZeroRow;
   }
 };
@@ -361,8 +362,8 @@ int en_repad(const void *src, void *dst, const int32_t *cu_seqlens, int batch, i
 }
 
 int en_transpose_pad_heads(const void *src, void *dst, const int32_t *cu_seqlens, int batch, int max_seq_len,
-                           int head_num, int size_per_head, int src_head_rows, int src_head_first, int elem_size,
-                           en_stream_t stream) {
+                           int head_num, int size_per_head, int src_head_rows, int src_head_first,
+                           int zero_padding, int elem_size, en_stream_t stream) {
   if (!src || !dst || !cu_seqlens) return EN_ERR_NULL;
   if (check_elem(elem_size)) return EN_ERR_DTYPE;
   if (batch < 1 || max_seq_len < 1 || head_num < 1 || size_per_head < 1) return EN_ERR_SHAPE;
@@ -372,13 +373,13 @@ int en_transpose_pad_heads(const void *src, void *dst, const int32_t *cu_seqlens
   return launch_row_gather<PadMap, 1>((int64_t)size_per_head * elem_size, max_seq_len,
                                       (int64_t)batch * max_seq_len * head_num * size_per_head * elem_size, p, [&](int R, dim3 &grid) {
     grid = dim3((unsigned)(ceil_div(max_seq_len, R) * head_num), (unsigned)batch, 1);
-    return PadMap{cu_seqlens, head_num, max_seq_len, R, src_head_rows, src_head_first};
+    return PadMap{cu_seqlens, head_num, max_seq_len, R, src_head_rows, src_head_first, zero_padding ? 1 : 0};
   }, (hipStream_t)stream);
 }
 
 int en_transpose_pad(const void *src, void *dst, const int32_t *cu_seqlens, int batch, int max_seq_len, int head_num,
                      int size_per_head, int elem_size, en_stream_t stream) {
-  return en_transpose_pad_heads(src, dst, cu_seqlens, batch, max_seq_len, head_num, size_per_head, head_num, 0,
+  return en_transpose_pad_heads(src, dst, cu_seqlens, batch, max_seq_len, head_num, size_per_head, head_num, 0, 1,
                                 elem_size, stream);
 }
 

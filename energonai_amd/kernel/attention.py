@@ -178,10 +178,12 @@ def attn_fused_packed(qkv, batch_size: int, max_seq_len: int, seq_len_list, head
     return attn_fused_varlen(q, k, v, batch_size, max_seq_len, seq_len_list, scale=scale, causal=causal, out=out)
 
 
-def kv_cache_fill(src, cache, batch_size: int, seq_len_list, head_first: int = 0):
+def kv_cache_fill(src, cache, batch_size: int, seq_len_list, head_first: int = 0, zero_padding: bool = True):
     """Writes ``cache[b,h,s,:] = src[cu[b]+s, head_first+h, :]`` for ``s < len[b]`` and zeros for the rest of
     the ``[B,H,Smax,D]`` cache.  ``src`` is the packed projection output seen as ``[T,Hs,D]`` (contiguous),
     so K and V caches are filled from their thirds of a fused projection without copying them out first.
+    ``zero_padding=False`` leaves the rows past each length as they are (the attention and decode kernels
+    never read them), which saves writing them.
     """
     _lib.require_gpu(src, "src")
     _lib.require_gpu(cache, "cache")
@@ -192,8 +194,8 @@ def kv_cache_fill(src, cache, batch_size: int, seq_len_list, head_first: int = 0
     info = seq_info(seq_len_list, batch_size, src.device)
     with _lib.device_guard(src):
         _lib.check(_lib.fn.en_transpose_pad_heads(src.data_ptr(), cache.data_ptr(), info.cu_seqlens.data_ptr(), B, Smax,
-                                                  H, D, src.shape[1], int(head_first), src.element_size(),
-                                                  _lib.stream_of(src)), "kv_cache_fill")
+                                                  H, D, src.shape[1], int(head_first), int(bool(zero_padding)),
+                                                  src.element_size(), _lib.stream_of(src)), "kv_cache_fill")
     return cache
 
 

@@ -47,8 +47,13 @@ def _int32_gpu(t: torch.Tensor, name: str) -> torch.Tensor:
     return t
 
 
-def transpose_pad(src, batch_size, max_seq_len, seq_len_list, head_num, size_per_head):
-    """[1,T,H,Dk] -> zero-padded [B,H,S,Dk]  (transpose_pad.py:12-18)."""
+def transpose_pad(src, batch_size, max_seq_len, seq_len_list, head_num, size_per_head, zero_padding=True):
+    """[1,T,H,Dk] -> zero-padded [B,H,S,Dk]  (transpose_pad.py:12-18).
+
+    ``zero_padding=False`` (not in the reference) writes the valid rows only and leaves the padding rows of the
+    new tensor uninitialised: for callers whose consumers are bounded by the sequence lengths, as the attention
+    kernels of this package are.
+    """
     src = src.contiguous()
     _lib.require_gpu(src, "src")
     info = seq_info(seq_len_list, batch_size, src.device)
@@ -56,10 +61,15 @@ def transpose_pad(src, batch_size, max_seq_len, seq_len_list, head_num, size_per
         raise RuntimeError("transpose_pad: src size is not a multiple of head_num * size_per_head")
     dst = torch.empty((batch_size, head_num, max_seq_len, size_per_head), dtype=src.dtype, device=src.device)
     with _lib.device_guard(src):
-        _lib.check(_lib.fn.en_transpose_pad(src.data_ptr(), dst.data_ptr(), info.cu_seqlens.data_ptr(),
-                                                batch_size, max_seq_len, head_num, size_per_head,
-                                                _elem_size(src, "transpose_pad"), _lib.stream_of(src)),
-                   "transpose_pad")
+        if zero_padding:
+            rc = _lib.fn.en_transpose_pad(src.data_ptr(), dst.data_ptr(), info.cu_seqlens.data_ptr(), batch_size,
+                                          max_seq_len, head_num, size_per_head, _elem_size(src, "transpose_pad"),
+                                          _lib.stream_of(src))
+        else:
+            rc = _lib.fn.en_transpose_pad_heads(src.data_ptr(), dst.data_ptr(), info.cu_seqlens.data_ptr(), batch_size,
+                                                max_seq_len, head_num, size_per_head, head_num, 0, 0,
+                                                _elem_size(src, "transpose_pad"), _lib.stream_of(src))
+        _lib.check(rc, "transpose_pad")
     return dst
 
 

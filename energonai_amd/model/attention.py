@@ -83,7 +83,7 @@ class MultiHeadAttention1D(nn.Module):
             pads = []
             for t in (q, k, v):
                 buf = torch.empty((batch_size, H, max_seq_len, D), dtype=x.dtype, device=x.device)
-                pads.append(kv_cache_fill(t.contiguous(), buf, batch_size, info))
+                pads.append(kv_cache_fill(t.contiguous(), buf, batch_size, info, zero_padding=False))
             scores = attn_qk(pads[0], pads[1], info, causal=self.is_decoder)
             probs = scale_mask_softmax(batch_size, max_seq_len, H, scores, info, scale=self.scaling,
                                        causal=self.is_decoder, tail_rows=128)

@@ -30,8 +30,9 @@ class KVCache:
     def fill(self, k_src: torch.Tensor, v_src: torch.Tensor, info: SeqInfo, k_head_first: int = 0,
              v_head_first: int = 0) -> None:
         """Prefill from packed projections seen as ``[T,Hs,D]`` (see ``kv_cache_fill``)."""
-        kv_cache_fill(k_src, self.k, self.batch_size, info, k_head_first)
-        kv_cache_fill(v_src, self.v, self.batch_size, info, v_head_first)
+        # the buffers were zeroed when they were allocated and no reader goes past the lengths
+        kv_cache_fill(k_src, self.k, self.batch_size, info, k_head_first, zero_padding=False)
+        kv_cache_fill(v_src, self.v, self.batch_size, info, v_head_first, zero_padding=False)
         self.lens.copy_(info.lens)
 
     def append(self, k_new: torch.Tensor, v_new: torch.Tensor) -> None:

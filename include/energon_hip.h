@@ -77,10 +77,13 @@ int en_transpose_pad(const void *src, void *dst, const int32_t *cu_seqlens, int 
  * elements per token, of which rows src_head_first .. src_head_first+head_num-1
  * are moved: fills a [B,H,S,D] K or V cache from the k / v third of a fused
  * projection output without first copying that third out (the reference makes
- * the thirds contiguous with .contiguous(), energonai/model/attention.py:74). */
+ * the thirds contiguous with .contiguous(), energonai/model/attention.py:74).
+ * zero_padding = 0 leaves rows s >= len[b] of dst untouched: for a destination
+ * whose readers are bounded by the sequence lengths (the attention and decode
+ * entry points here are), which saves the writes of the padding. */
 int en_transpose_pad_heads(const void *src, void *dst, const int32_t *cu_seqlens, int batch, int max_seq_len,
-                           int head_num, int size_per_head, int src_head_rows, int src_head_first, int elem_size,
-                           en_stream_t stream);
+                           int head_num, int size_per_head, int src_head_rows, int src_head_first,
+                           int zero_padding, int elem_size, en_stream_t stream);
 
 /* transpose_depad_wrapper (wrapper.cpp:59-83, kernel.cu:8-46):
  * [B,H,S,D] -> [T,H,D]; every byte of dst is written when T = cu_seqlens[B]. */

@@ -80,7 +80,7 @@ def test_entry_points_validate_before_launch():
     i64x3 = (ctypes.c_int64 * 3)(0, 64, 768)
     assert lib.en_repad(None, 32, 48, 1, 1, 1, 2, 0, None) == -1
     assert lib.en_repad(16, 32, 48, 1, 0, 1, 2, 0, None) == -2           # max_seq_len 0
-    assert lib.en_transpose_pad_heads(16, 32, 48, 1, 1, 4, 8, 6, 4, 2, None) == -2   # heads 4..7 of a 6-row source
+    assert lib.en_transpose_pad_heads(16, 32, 48, 1, 1, 4, 8, 6, 4, 1, 2, None) == -2   # heads 4..7 of a 6-row source
     assert lib.en_kv_append(16, 32, 48, 64, None, 1, 1, 1, 8, 8, 8, 8, 8, 8, 2, None) == -1
     assert lib.en_kv_append(16, 32, 48, 64, 80, 1, 1, 1, 8, 8, 8, 8, 8, 8, 3, None) == -3   # element size 3
     assert lib.en_attn_fused(16, 32, 48, 64, 80, None, 1, 1, 8, 8, 64, i64x3, i64x3, i64x3, i64x3, None, None, 1.0, 1, 0,

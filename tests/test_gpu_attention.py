@@ -334,8 +334,9 @@ def test_attention_long_bucket(causal):
     qg, kg, vg = torch.chunk(qkv.cuda(), 3, dim=-1)
     s_gpu = k.attn_qk(qg, kg, lens_t, causal=causal)
     p_gpu = k.scale_mask_softmax(B, S, H, s_gpu, lens_t, scale=scale, causal=causal, tail_rows=128)
-    for b, n in enumerate(lens):      # rows of probabilities sum to one over the keys of the sequence
-        rows = p_gpu[b, :, :n, :n].float().sum(-1)
+    for b, n in enumerate(lens):      # rows of probabilities sum to one over the keys the row may see
+        blk = p_gpu[b, :, :n, :n].float()      # what lies past a row's query tile is never written: mask it
+        rows = (torch.tril(blk) if causal else blk).sum(-1)
         assert float((rows - 1).abs().max()) <= 4e-3
     ctx_a = k.attn_pv(p_gpu, vg, lens_t, causal=causal).cpu()
     ctx_b = k.attn_fused(qg, kg, vg, lens_t, scale=scale, causal=causal).cpu()

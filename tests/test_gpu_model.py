@@ -97,6 +97,31 @@ def test_kv_cache_fill_and_append_bit_exact(dtype):
         assert cache.lens.cpu().tolist() == [n + step + 1 for n in lens]
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.float32])
+def test_kv_cache_fill_without_zero_fill_leaves_padding_untouched(dtype):
+    """zero_padding=False: rows below each length are written, every other row keeps the bits it had
+    (tiles that lie wholly in the padding are skipped, tiles that straddle a length are written in part)."""
+    K, _ = _mods()
+    B, H, D, Smax = 4, 3, 64, 700
+    lens = [700, 0, 129, 64]
+    T = sum(lens)
+    announce("kv fill no zero", dtype)
+    g = torch.Generator().manual_seed(31)
+    src = torch.randn(T, 2 * H, D, generator=g).to(dtype)
+    sentinel = torch.full((B, H, Smax, D), 123.0, dtype=dtype)
+    lens_t = torch.tensor(lens, dtype=torch.int32).cuda()
+    got = K.kv_cache_fill(src.cuda(), sentinel.clone().cuda(), B, lens_t, head_first=H, zero_padding=False).cpu()
+    full = K.kv_cache_fill(src.cuda(), sentinel.clone().cuda(), B, lens_t, head_first=H).cpu()
+    want = sentinel.clone()
+    start = 0
+    for b, n in enumerate(lens):
+        want[b, :, :n] = src[start:start + n, H:].permute(1, 0, 2)
+        start += n
+    assert torch.equal(got, want)
+    for b, n in enumerate(lens):
+        assert torch.equal(full[b, :, :n], want[b, :, :n]) and not full[b, :, n:].any()
+
+
 @pytest.mark.parametrize("fused_qkv", [True, False])
 @pytest.mark.parametrize("is_decoder", [True, False])
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16, torch.float32])

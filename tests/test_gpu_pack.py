@@ -45,6 +45,10 @@ def test_transpose_pad_depad(dtype, B, S, H, D, lens):
         got = k.transpose_pad(src.cuda(), B, S, lens_t.to(lens_dtype).cuda(), H, D)
         assert got.shape == (B, H, S, D) and got.dtype == dtype
         assert torch.equal(got.cpu(), ref_pad), f"transpose_pad mismatch (lens {lens_dtype})"
+    # valid rows only: same bits on every row below a length (the padding rows are left unwritten)
+    got = k.transpose_pad(src.cuda(), B, S, lens_t.cuda(), H, D, zero_padding=False).cpu()
+    for b, n in enumerate(lens_l):
+        assert torch.equal(got[b, :, :n], ref_pad[b, :, :n])
     # inverse
     ref_depad = eager.transpose_depad(ref_pad, B, T, S, lens_l, H, D)
     assert torch.equal(ref_depad, src)
