@@ -441,7 +441,7 @@ def kernel_table(torch, K, layer, workloads, w, d, info, steps):
                                                                  causal=w.causal)
         fns["scale_mask_softmax_tiled"] = lambda: K.scale_mask_softmax(B, S, H, scores, info, scale=w.scale,
                                                                        causal=w.causal,
-                                                                       tail_rows=layer.PV_QUERY_TILE)
+                                                                       tail_rows=layer.SOFTMAX_TAIL_ROWS)
         fns["attn_pv"] = lambda: K.attn_pv(scores, v, info, causal=w.causal, out=ctx)
         if w.dtype != torch.float32:
             alg["attn_fused"] = 4 * T * H * D * torch.empty(0, dtype=w.dtype).element_size()   # q, k, v in; ctx out

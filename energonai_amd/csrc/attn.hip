@@ -404,6 +404,13 @@ __global__ __launch_bounds__(kBlock) void attn_pv_kernel(AttnArgs a) {
   const rsrc_t v_rsrc = make_rsrc(vbase, (uint32_t)(((int64_t)(max(kl, 1) - 1) * a.k_ss + a.D) * E::kSize));
   uint4 preg[PLOADS];
   uint4 vreg[VLOADS][4];
+  // a probability row is read only as far as its own query sees: what lies past that need not have been written
+  int p_vis[PLOADS];
+#pragma unroll
+  for (int i = 0; i < PLOADS; ++i) {
+    const int q = q0 + (tid + i * kBlock) / PVEC_ROW;
+    p_vis[i] = q < ql ? tile_key_extent(a, q, kl, ql) : 0;
+  }
   auto fetch = [&](int kt) {
     const int k0 = kt * BK;
 #pragma unroll
@@ -413,13 +420,13 @@ __global__ __launch_bounds__(kBlock) void attn_pv_kernel(AttnArgs a) {
       const int q = q0 + row, k = k0 + c * EPV;
       if constexpr (VEC) {
         const uint32_t off = (uint32_t)(((int64_t)q * a.Sk + k) * E::kSize);
-        preg[i] = buffer_load16<STREAM ? 2 : 0>(p_rsrc, (kt < nkt && k < nk) ? off : kOutOfRange);
-      } else if (kt < nkt && q < ql && k < nk) {
+        preg[i] = buffer_load16<STREAM ? 2 : 0>(p_rsrc, (kt < nkt && k < p_vis[i]) ? off : kOutOfRange);
+      } else if (kt < nkt && k < p_vis[i]) {
         const T *gp = pbase + (int64_t)q * a.Sk + k;
         {
           Pack<T, EPV> pk;
 #pragma unroll
-          for (int e = 0; e < EPV; ++e) pk.v[e] = (k + e < nk) ? gp[e] : E::from_float(0.f);
+          for (int e = 0; e < EPV; ++e) pk.v[e] = (k + e < p_vis[i]) ? gp[e] : E::from_float(0.f);
           preg[i] = __builtin_bit_cast(uint4, pk);
         }
       } else {
@@ -602,16 +609,19 @@ __global__ __launch_bounds__(kBlock, 3) void attn_pv_strip_kernel(AttnArgs a) {
   T *strip = lds_p[wave];
   const int pr = lane / PVEC_ROW, pc = (lane % PVEC_ROW) * EPV;
   uint32_t p_off[PLOADS];
+  int p_vis[PLOADS];           // a row is read only as far as its own query sees: the rest need not have been written
 #pragma unroll
-  for (int i = 0; i < PLOADS; ++i)
-    p_off[i] = (uint32_t)(((int64_t)(qw + pr + i * (kWave / PVEC_ROW)) * a.Sk + pc) * E::kSize);
+  for (int i = 0; i < PLOADS; ++i) {
+    const int row = qw + pr + i * (kWave / PVEC_ROW);
+    p_off[i] = (uint32_t)(((int64_t)row * a.Sk + pc) * E::kSize);
+    p_vis[i] = row < ql ? tile_key_extent(a, row, kl, ql) : 0;
+  }
   uint4 preg[PLOADS];
-  // keys at or past nk were never written by the softmax: they must not be read
   auto fetch_p = [&](int kt) {
     const int k0 = kt * BK;
 #pragma unroll
     for (int i = 0; i < PLOADS; ++i)
-      preg[i] = buffer_load16<STREAM ? 2 : 0>(p_rsrc, (k0 + pc < nk) ? p_off[i] + (uint32_t)(k0 * E::kSize) : kOutOfRange);
+      preg[i] = buffer_load16<STREAM ? 2 : 0>(p_rsrc, (k0 + pc < p_vis[i]) ? p_off[i] + (uint32_t)(k0 * E::kSize) : kOutOfRange);
   };
   auto stage_p = [&]() {
 #pragma unroll

@@ -60,8 +60,8 @@ extern "C" int en_padding_removal_layer(const void *hidden_padded, const void *q
       rc = en_attn_qk(q, k, scores, seq_lens, nullptr, B, H, S, S, D, sb, sh, ss, sb, sh, ss, 1.0f, causal, dtype,
                       stream);
       if (rc) return rc;
-      // the PV kernel reads a probability row only up to the extent of its 128-row query tile
-      rc = en_scale_mask_softmax(scores, seq_lens, nullptr, B, H, S, S, scale, causal, 128, dtype, stream);
+      // the PV kernel reads a probability row only as far as its own query sees: no tail is written
+      rc = en_scale_mask_softmax(scores, seq_lens, nullptr, B, H, S, S, scale, causal, 1, dtype, stream);
       if (rc) return rc;
       rc = en_attn_pv(scores, v, ctx, seq_lens, nullptr, B, H, S, S, D, sb, sh, ss, cb, ch, cs, causal, 0, dtype, stream);
       if (rc) return rc;

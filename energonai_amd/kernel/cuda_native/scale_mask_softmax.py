@@ -12,9 +12,11 @@ Keyword extensions (defaults preserve the reference behaviour):
 ``k_seq_len``  key extent when src is rectangular [B,H,batch_seq_len,k_seq_len]
 ``q_len_list`` valid query rows per sequence when they differ from the key
                lengths (decode: one query against a longer cache)
-``tail_rows``  0 zeroes the whole masked tail of each row (reference); 128 zeroes
-               only what ``attn_pv`` reads (the extent of the row's 128-row query
-               tile) and leaves the rest of the row untouched
+``tail_rows``  0 zeroes the whole masked tail of each row (reference); a power of
+               two n zeroes only up to what the last row of the row's n-row tile
+               sees and leaves the rest untouched.  1 writes just the visible
+               prefix (to the end of its last 16-byte vector), which is all that
+               ``attn_pv`` reads of a row
 
 There is no limit on the sequence length (the reference cannot launch above
 1024) and offsets are 64-bit.

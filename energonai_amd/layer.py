@@ -22,8 +22,8 @@ from . import _lib
 from .seqinfo import SeqInfo, seq_info
 
 
-# attn_pv reads a row of probabilities only up to the visible extent of its 128-row query tile
-PV_QUERY_TILE = 128
+# attn_pv reads a row of probabilities only as far as the row's own query sees, so the softmax writes no tail
+SOFTMAX_TAIL_ROWS = 1
 
 
 def padding_removal_layer(hidden_padded: torch.Tensor, qkv_packed: torch.Tensor, seq_lens, head_num: int,
@@ -68,7 +68,7 @@ def padding_removal_layer(hidden_padded: torch.Tensor, qkv_packed: torch.Tensor,
         ctx = attn_fused(q, k, v, info, scale=scale, causal=causal)
     else:
         scores = attn_qk(q, k, info, causal=causal)
-        probs = scale_mask_softmax(B, S, H, scores, info, scale=scale, causal=causal, tail_rows=PV_QUERY_TILE)
+        probs = scale_mask_softmax(B, S, H, scores, info, scale=scale, causal=causal, tail_rows=SOFTMAX_TAIL_ROWS)
         ctx = attn_pv(probs, v, info, causal=causal)
     ctx_packed = transpose_depad(ctx, B, T, S, info, H, D)
     attn_out = ctx_packed.view(1, T, H * D) if dense_out is None else dense_out

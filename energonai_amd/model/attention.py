@@ -86,7 +86,7 @@ class MultiHeadAttention1D(nn.Module):
                 pads.append(kv_cache_fill(t.contiguous(), buf, batch_size, info, zero_padding=False))
             scores = attn_qk(pads[0], pads[1], info, causal=self.is_decoder)
             probs = scale_mask_softmax(batch_size, max_seq_len, H, scores, info, scale=self.scaling,
-                                       causal=self.is_decoder, tail_rows=128)
+                                       causal=self.is_decoder, tail_rows=1)
             ctx = transpose_depad(attn_pv(probs, pads[2], info, causal=self.is_decoder), batch_size, T, max_seq_len,
                                   info, H, D)
         if fill_cache:

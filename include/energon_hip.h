@@ -137,9 +137,10 @@ int en_ft_transpose_remove(const void *src, void *dst, int valid_word_num, int b
  * n = k_lens[b] when causal == 0, else min(k_lens[b], q + k_lens[b] - q_lens[b] + 1).
  * Rows q >= q_lens[b] are not touched (as in the reference, kernel.cu:14-17).
  * q_lens == NULL means q_lens[b] = min(k_lens[b], Sq).  tail_rows == 0 zeroes the
- * whole tail of every row as the reference does; tail_rows == t > 0 zeroes a row
- * only as far as the last row of its t-row query tile can see, which is all
- * en_attn_pv (t = 128) reads -- the rest of the row is then left untouched.
+ * whole tail of every row as the reference does; tail_rows == t > 0 (a power of
+ * two) zeroes a row only as far as the last row of its t-row query tile can see
+ * and leaves the rest of the row untouched.  t = 1 writes the visible prefix
+ * alone (to the end of its last 16-byte vector), which is all en_attn_pv reads.
  * The reference call is Sq == Sk, scale 1, causal 1, q_lens NULL, tail_rows 0.
  * No limit on Sk; fp32 math. */
 int en_scale_mask_softmax(void *src, const int32_t *k_lens, const int32_t *q_lens, int batch, int head_num,
@@ -180,8 +181,9 @@ int en_attn_qk(const void *q, const void *k, void *scores, const int32_t *k_lens
 
 /* ctx[b,h,i,:] = sum_j p[b,h,i,j] * v[b,h,j,:]  (examples/bert/bert.py:119,
  * examples/gpt/gpt.py:125) over j < visible(i) only; p contiguous [B,H,Sq,Sk]
- * as left by en_scale_mask_softmax, v strided like k above, ctx addressed with
- * its own strides.  Rows i >= q_lens[b] of ctx are written as zero when
+ * as left by en_scale_mask_softmax (any tail_rows: of row i only the 16-byte
+ * vectors that hold a visible entry are read), v strided like k above, ctx
+ * addressed with its own strides.  Rows i >= q_lens[b] of ctx are written as zero when
  * zero_padding != 0 and left untouched otherwise. */
 int en_attn_pv(const void *p, const void *v, void *ctx, const int32_t *k_lens, const int32_t *q_lens, int batch,
                int head_num, int q_seq_len, int k_seq_len, int size_per_head, int64_t v_stride_b,

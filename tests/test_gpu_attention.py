@@ -113,6 +113,35 @@ def test_attn_nan_in_padding_of_v_is_ignored():
         assert torch.isfinite(ctx[b, :, :n]).all()
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.float32])
+@pytest.mark.parametrize("causal", [True, False])
+def test_attn_pv_reads_a_row_only_as_far_as_its_query_sees(dtype, causal):
+    """The score buffer comes from torch.empty and the softmax with tail_rows=1 writes the visible prefix of a
+    row only: NaNs parked everywhere else (past the last 16-byte vector with a visible key, and in the rows of
+    padded queries) must not reach the context."""
+    k = _kernel()
+    B, H, S, D = 3, 2, 328, 64
+    lens = [328, 131, 9]
+    epv = 16 // torch.empty(0, dtype=dtype).element_size()
+    announce("attn pv row extent", dtype, causal)
+    g = torch.Generator().manual_seed(8)
+    p = torch.rand(B, H, S, S, generator=g).to(dtype)
+    v = torch.randn(B, H, S, D, generator=g).to(dtype)
+    clean = torch.zeros_like(p)
+    dirty = torch.full_like(p, float("nan"))
+    for b, n in enumerate(lens):
+        for q in range(n):
+            vis = min(n, q + 1) if causal else n
+            clean[b, :, q, :vis] = p[b, :, q, :vis]
+            dirty[b, :, q, :vis] = p[b, :, q, :vis]
+            dirty[b, :, q, vis:-(-vis // epv) * epv] = 0      # the softmax completes the last vector with zeros
+    lens_t = torch.tensor(lens, dtype=torch.int32).cuda()
+    want = k.attn_pv(clean.cuda(), v.cuda(), lens_t, causal=causal).cpu()
+    got = k.attn_pv(dirty.cuda(), v.cuda(), lens_t, causal=causal).cpu()
+    for b, n in enumerate(lens):
+        assert torch.equal(got[b, :, :n], want[b, :, :n])
+
+
 DECODE_CASES = [
     # B, H, Smax, D, kv lens
     (5, 4, 640, 128, [640, 1, 333, 64, 65]),
