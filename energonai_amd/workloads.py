@@ -142,18 +142,12 @@ def algorithmic_bytes(w: Workload, lens_list) -> Dict[str, float]:
                     scale_mask_softmax=2 * H * kv * e, layernorm_residual=3 * B * hid * e)
     T = sum(lens_list)
     vis = sum(n * (n + 1) // 2 for n in lens_list) if w.causal else sum(n * n for n in lens_list)
-    # softmax with the tail zeroed only as far as attn_pv reads (the extent of each 128-row query tile)
-    tiled = 0
-    for n in lens_list:
-        for q0 in range(0, n, 128):
-            rows = min(128, n - q0)
-            tiled += rows * (min(n, q0 + rows) if w.causal else n)
     return dict(
         depad=2 * T * hid * e,
         transpose_pad=T * H * 3 * D * e + B * S * H * 3 * D * e,
         transpose_depad=2 * T * H * D * e,
         scale_mask_softmax=H * e * vis + H * e * T * S,
-        scale_mask_softmax_tiled=H * e * vis + H * e * tiled,
+        scale_mask_softmax_no_tail=2 * H * e * vis,   # the form in the step: the visible prefix in, the same out
         layernorm_residual=3 * T * hid * e,
         attn_qk=H * e * vis + 2 * T * H * D * e,
         attn_pv=H * e * vis + 2 * T * H * D * e,

@@ -198,25 +198,27 @@ def test_layernorm_module_matches_reference_interface():
         ln(torch.zeros(2, 100, dtype=torch.float16).cuda())
 
 
+@pytest.mark.parametrize("tile", [128, 32, 1])
 @pytest.mark.parametrize("dtype", [torch.float16, torch.float32])
 @pytest.mark.parametrize("causal", [True, False])
-def test_softmax_tiled_tail(dtype, causal):
-    """tail_rows=128: valid entries identical to the full-tail result, zeros up to the extent of the
-    row's 128-row query tile, everything beyond left untouched."""
+def test_softmax_tiled_tail(dtype, causal, tile):
+    """tail_rows=t: valid entries identical to the full-tail result, zeros up to the extent of the row's
+    t-row query tile, everything beyond left untouched.  t = 1 (the form in the step) writes no tail at all."""
     k = _kernel()
     B, H, S = 3, 2, 512
     lens = [512, 130, 300]
-    announce("softmax tiled tail", dtype, causal)
+    announce("softmax tiled tail", dtype, causal, tile)
     g = torch.Generator().manual_seed(21)
     src = (3.0 * torch.randn(B, H, S, S, generator=g)).to(dtype)
     lens_t = torch.tensor(lens, dtype=torch.int32).cuda()
+    epv = 16 // src.element_size()
     full = k.scale_mask_softmax(B, S, H, src.clone().cuda(), lens_t, scale=0.5, causal=causal).cpu()
-    tiled = k.scale_mask_softmax(B, S, H, src.clone().cuda(), lens_t, scale=0.5, causal=causal, tail_rows=128).cpu()
+    tiled = k.scale_mask_softmax(B, S, H, src.clone().cuda(), lens_t, scale=0.5, causal=causal, tail_rows=tile).cpu()
     for b, n in enumerate(lens):
-        for q0 in range(0, n, 128):
-            rows = min(128, n - q0)
+        for q0 in range(0, n, tile):
+            rows = min(tile, n - q0)
             lim = min(n, q0 + rows) if causal else n
-            lim_v = -(-lim // (16 // src.element_size())) * (16 // src.element_size())   # whole vectors are written
+            lim_v = -(-lim // epv) * epv   # whole vectors are written
             assert torch.equal(tiled[b, :, q0:q0 + rows, :lim], full[b, :, q0:q0 + rows, :lim])
             assert torch.equal(tiled[b, :, q0:q0 + rows, lim_v:], src[b, :, q0:q0 + rows, lim_v:])
         assert torch.equal(tiled[b, :, n:], src[b, :, n:])
