@@ -2,7 +2,9 @@
 
 The reference calls ``cublasGemmEx`` with an algorithm id and finds the best id by timing them all.  hipBLASLt
 ranks candidate solutions per problem instead, so ``algo`` is an index into that list (``-1`` = first choice)
-and ``find_algo`` times the candidates of the reference's probe problem.  ``bias`` and ``activation`` are
+and ``find_algo`` times the candidates of the reference's probe problem.  ``algo="auto"`` does that search for
+the problem at hand, once, and remembers the winner (``tuned_algo``): the library's first choice is often not the
+fastest for the skinny GEMMs of a decode step.  ``bias`` and ``activation`` are
 additions: hipBLASLt applies them in the GEMM epilogue, where the reference's callers run separate ops
 (energonai/model/mlp.py:30-35).
 """
@@ -18,6 +20,7 @@ from ... import _lib
 _ACTIVATIONS = {None: 0, "none": 0, "relu": 1, "gelu_tanh": 2}
 _WORKSPACE_BYTES = 64 << 20
 _workspaces: Dict[int, torch.Tensor] = {}
+_tuned: Dict[tuple, int] = {}
 
 
 def _workspace(device: torch.device) -> torch.Tensor:
@@ -45,8 +48,10 @@ def linear(inputs, param, algo=-1, bias=None, activation: Optional[str] = None):
     _lib.require_gpu(param, "param")
     if inputs.dim() != 3 or param.dim() != 2 or inputs.shape[2] != param.shape[1]:
         raise RuntimeError("linear: inputs must be [batch, seq_len, din] and param [dout, din]")
+    if isinstance(algo, str) and algo == "auto":
+        algo = tuned_algo(inputs, param, bias=bias, activation=activation)
     if not isinstance(algo, int) or algo < -1:
-        raise RuntimeError("linear: algo must be -1 or an index below find_algo's candidate count")
+        raise RuntimeError("linear: algo must be -1, \"auto\" or an index below find_algo's candidate count")
     if param.dtype != inputs.dtype or (bias is not None and bias.dtype != inputs.dtype):
         raise RuntimeError("linear: inputs, param and bias must share one dtype")
     if activation not in _ACTIVATIONS:
@@ -74,6 +79,37 @@ def algo_count(rows: int, din: int, dout: int, dtype=torch.float16, has_bias: bo
                                  _lib._DTYPE_TAG[dtype], _WORKSPACE_BYTES)
     _check(n, "algo_count")
     return n
+
+
+@torch.no_grad()
+def tuned_algo(inputs, param, bias=None, activation: Optional[str] = None, inner_loop: int = 5) -> int:
+    """Index of the fastest candidate for ``linear(inputs, param, bias=bias, activation=activation)``.
+
+    Every candidate is timed with HIP events on the given tensors the first time a problem
+    ``(rows, din, dout, dtype, bias, activation)`` is seen on a device (the reference finds its cuBLAS algorithm
+    the same way on one probe problem, linear_func.py:35-92); later calls return the remembered index.  The
+    search launches and synchronises, so the first call of a problem must not sit inside a stream capture.
+    """
+    rows = inputs.shape[0] * inputs.shape[1]
+    key = (inputs.device.index, rows, inputs.shape[2], param.shape[0], inputs.dtype, bias is not None, activation)
+    best = _tuned.get(key)
+    if best is not None:
+        return best
+    n = algo_count(rows, inputs.shape[2], param.shape[0], inputs.dtype, bias is not None, activation)
+    best, best_t = -1, float("inf")
+    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    for algo in range(n):
+        linear(inputs, param, algo, bias=bias, activation=activation)
+        start.record()
+        for _ in range(inner_loop):
+            linear(inputs, param, algo, bias=bias, activation=activation)
+        stop.record()
+        stop.synchronize()
+        dt = start.elapsed_time(stop)
+        if dt < best_t:
+            best, best_t = algo, dt
+    _tuned[key] = best
+    return best
 
 
 @torch.no_grad()

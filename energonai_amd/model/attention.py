@@ -18,6 +18,7 @@ from ..kernel import (attn_fused_varlen, attn_pv, attn_qk, decode_pv, decode_qk,
                       transpose_depad)
 from ..kernel.attention import kv_cache_fill
 from ..seqinfo import SeqInfo, seq_info
+from .gemm import project
 from .kv_cache import KVCache, OutputHistory
 
 
@@ -61,11 +62,11 @@ class MultiHeadAttention1D(nn.Module):
         rows = x.numel() // self.hidden_size
         if self.fused_qkv:
             # the fused output is ordered k, v, q (attention.py:74)
-            kvq = self.query_key_value(x).view(rows, 3 * H, D)
+            kvq = project(self.query_key_value, x).view(rows, 3 * H, D)
             return kvq[:, 2 * H:], kvq[:, :H], kvq[:, H:2 * H], kvq
-        q = self.query_(x).view(rows, H, D)
-        k = self.key_(x).view(rows, H, D)
-        v = self.value_(x).view(rows, H, D)
+        q = project(self.query_, x).view(rows, H, D)
+        k = project(self.key_, x).view(rows, H, D)
+        v = project(self.value_, x).view(rows, H, D)
         return q, k, v, None
 
     # ---- attention over packed tokens --------------------------------------------------------
@@ -95,7 +96,7 @@ class MultiHeadAttention1D(nn.Module):
                 self.kv_cache.fill(kvq, kvq, info, 0, H)
             else:
                 self.kv_cache.fill(k.contiguous(), v.contiguous(), info)
-        return self.dense(ctx.view(1, T, self.hidden_size))
+        return project(self.dense, ctx.view(1, T, self.hidden_size))
 
     # ---- one decode step: newest position only ----------------------------------------------
     def forward_last(self, last: torch.Tensor) -> torch.Tensor:
@@ -112,7 +113,7 @@ class MultiHeadAttention1D(nn.Module):
         probs = scale_mask_softmax(B, 1, H, scores, cache.info, scale=self.scaling, causal=True,
                                    k_seq_len=cache.max_seq_len, q_len_list=ones)
         ctx = decode_pv(probs, cache.v, cache.info)          # [B,H,1,D]
-        return self.dense(ctx.view(B, 1, self.hidden_size))
+        return project(self.dense, ctx.view(B, 1, self.hidden_size))
 
     def forward(self, hidden_states, attention_mask=None, first_cache=False, seq_lens=None):
         B, S, hid = hidden_states.shape

@@ -7,6 +7,7 @@ import torch
 from torch import nn
 
 from ..kernel.cuda_native.linear_func import linear
+from .gemm import gemm_algo
 
 
 def _epilogue_of(activation) -> Optional[str]:
@@ -41,8 +42,9 @@ class MLP1D(nn.Module):
         any other activation runs as its own op between two library GEMMs, as in mlp.py:31-33.
         """
         if self._epilogue is not None and x.is_cuda and x.dim() == 3 and x.is_contiguous():
-            h = linear(x, self.dense_1.weight.detach(), -1, bias=_detached(self.dense_1.bias), activation=self._epilogue)
-            return linear(h, self.dense_2.weight.detach(), -1, bias=_detached(self.dense_2.bias))
+            h = linear(x, self.dense_1.weight.detach(), gemm_algo(), bias=_detached(self.dense_1.bias),
+                       activation=self._epilogue)
+            return linear(h, self.dense_2.weight.detach(), gemm_algo(), bias=_detached(self.dense_2.bias))
         return self.dense_2(self.activation(self.dense_1(x)))
 
     def forward(self, hidden_states, first_cache: Optional[bool] = True):

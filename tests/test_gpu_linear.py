@@ -64,3 +64,25 @@ def test_reference_extension_stand_in_uses_the_same_gemm():
     want = (x.double() @ w.double().T).cpu()
     for algo in (-1, 5, 99, 115):       # the reference's id ranges are accepted
         assert max_abs(ext.mlp_gemm(x, w, algo).cpu(), want) <= 4e-3 * float(want.abs().max())
+
+
+def test_auto_algo_is_searched_once_per_problem_and_gives_the_same_product():
+    lf = _lf()
+    B, S, din, dout = 1, 48, 384, 640          # a skinny problem, as in a decode step
+    announce("linear auto algo")
+    g = torch.Generator().manual_seed(44)
+    x = torch.randn(B, S, din, generator=g).half().cuda()
+    w = (torch.randn(dout, din, generator=g) / din ** 0.5).half().cuda()
+    b = torch.randn(dout, generator=g).half().cuda()
+    lf._tuned.clear()
+    best = lf.tuned_algo(x, w, bias=b, activation="relu", inner_loop=2)
+    assert 0 <= best < lf.algo_count(B * S, din, dout, torch.float16, True, "relu")
+    assert len(lf._tuned) == 1
+    got = lf.linear(x, w, "auto", bias=b, activation="relu").cpu()
+    assert len(lf._tuned) == 1 and lf.tuned_algo(x, w, bias=b, activation="relu") == best    # remembered
+    want = torch.relu(x.double() @ w.double().T + b.double()).cpu()
+    assert max_abs(got, want) <= 4e-3 * float(want.abs().max())
+    lf.linear(x, w, "auto")                      # no bias, no activation: another problem
+    assert len(lf._tuned) == 2
+    with pytest.raises(RuntimeError):
+        lf.linear(x, w, "fastest")

@@ -174,6 +174,43 @@ def test_block_prefill_and_incremental_decode(dtype, post):
         assert max_abs(got[:, -1], want[:, -1]) <= tol, step
 
 
+def test_block_with_tuned_gemms_matches_the_reference_block():
+    """set_gemm_tuning(True): every projection of the block runs on the fastest hipBLASLt candidate for its
+    shape (prefill shapes and the skinny decode shapes are separate problems); same tolerances as untuned."""
+    _, M = _mods()
+    from energonai_amd.kernel.cuda_native import linear_func as lf
+    B, S, hid, heads = 3, 70, 128, 2
+    lens = [70, 9, 41]
+    dtype = torch.float16
+    announce("block tuned gemms")
+    blk = M.Block1D(hid, heads, 4.0, activation=F.relu, dtype=dtype, max_seq_len=96).cuda()
+    _init(blk, 35)
+    p = _fp32_params(blk)
+    x, valid = _padded_batch(B, S, hid, lens, True, dtype, 36)
+    mask = models.additive_mask(valid)
+    lf._tuned.clear()
+    M.set_gemm_tuning(True)
+    try:
+        assert M.gemm_tuning()
+        got = blk(x.cuda(), attention_mask=mask.to(dtype).cuda(), first_cache=True).float().cpu()
+        n_prefill = len(lf._tuned)
+        assert n_prefill == 4                 # qkv, dense, fc1 (+ReLU), fc2 at the packed row count
+        want = models.block_forward(x, p, heads, 1e-5, False, True, mask, activation=F.relu)
+        assert max_abs(_valid_rows(got, lens, True), _valid_rows(want, lens, True)) <= 1.5e-2
+        g = torch.Generator().manual_seed(37)
+        for step in range(2):
+            x = torch.cat((x, torch.randn(B, 1, hid, generator=g).to(dtype)), 1)
+            valid = torch.cat((valid, torch.ones(B, 1)), 1)
+            mask = models.additive_mask(valid)
+            got = blk(x.cuda(), attention_mask=mask.to(dtype).cuda(), first_cache=False).float().cpu()
+            want = models.block_forward(x, p, heads, 1e-5, False, True, mask, activation=F.relu)
+            assert max_abs(got[:, -1], want[:, -1]) <= 1.5e-2, step
+        assert len(lf._tuned) == 2 * n_prefill        # the decode shapes were searched once, not per step
+    finally:
+        M.set_gemm_tuning(False)
+    assert not M.gemm_tuning()
+
+
 @pytest.mark.parametrize("act_name", ["relu", "gelu_tanh", "gelu"])
 @pytest.mark.parametrize("dtype", [torch.float16, torch.float32])
 def test_mlp_with_gemm_epilogues(dtype, act_name):
