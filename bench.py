@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the per-layer padding-removal hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c2] [--no-cpu] [--no-extra]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c2] [--no-cpu] [--no-extra] [--step-only]
 
 A step is one pass of
     depad -> transpose_pad -> QK^T -> scale_mask_softmax -> PV -> transpose_depad -> residual + LayerNorm
@@ -309,7 +309,7 @@ def run_block_decode(torch, w, steps, warmup):
 # ---------------------------------------------------------------------------
 # one workload on the GPU
 # ---------------------------------------------------------------------------
-def run_workload(torch, w, steps, warmup, want_eager=True, want_kernels=True):
+def run_workload(torch, w, steps, warmup, want_eager=True, want_kernels=True, step_only=False):
     from energonai_amd import kernel as K
     from energonai_amd import layer, workloads
     from energonai_amd.seqinfo import seq_info
@@ -345,7 +345,7 @@ def run_workload(torch, w, steps, warmup, want_eager=True, want_kernels=True):
     res["tokens_per_s"] = tokens / (wall_ms * 1e-3)
 
     # the optional fused-attention form of the same step (QK^T + softmax + PV in one kernel); not the headline
-    if not w.decode and w.dtype != torch.float32:
+    if not w.decode and w.dtype != torch.float32 and not step_only:
         def step_fused():
             return layer.padding_removal_layer(d["hidden_padded"], d["qkv_packed"], info, w.heads, w.head_dim,
                                                d["gamma"], d["beta"], workloads.EPS, w.scale, w.causal,
@@ -390,6 +390,8 @@ def run_workload(torch, w, steps, warmup, want_eager=True, want_kernels=True):
 
     # the same step replayed from a HIP graph (launch overhead removed); reported, never the headline
     try:
+        if step_only:
+            raise RuntimeError("skipped (--step-only)")
         g = torch.cuda.CUDAGraph()
         side = torch.cuda.Stream()
         side.wait_stream(torch.cuda.current_stream())
@@ -409,7 +411,7 @@ def run_workload(torch, w, steps, warmup, want_eager=True, want_kernels=True):
     torch.cuda.synchronize()
 
     if want_kernels:
-        res["kernels"] = kernel_table(torch, K, layer, workloads, w, d, info, steps)
+        res["kernels"] = kernel_table(torch, K, layer, workloads, w, d, info, steps, step_only)
     if want_eager:
         add_eager_aux(torch, w, d, dev)
         fn = (lambda: eager_decode_step(torch, w, d)) if w.decode else (lambda: eager_prefill_step(torch, w, d))
@@ -428,7 +430,7 @@ def run_workload(torch, w, steps, warmup, want_eager=True, want_kernels=True):
     return res
 
 
-def kernel_table(torch, K, layer, workloads, w, d, info, steps):
+def kernel_table(torch, K, layer, workloads, w, d, info, steps, step_only=False):
     """Launch-to-launch time of every kernel on its real operands -> GB/s, TFLOP/s, fraction of peak."""
     dt = DTYPE_NAME[str(w.dtype)]
     alg = workloads.algorithmic_bytes(w, d["lens_list"])
@@ -480,6 +482,10 @@ def kernel_table(torch, K, layer, workloads, w, d, info, steps):
         fns["transpose_depad"] = lambda: K.transpose_depad(ctx, B, T, S, info, H, D)
         fns["layernorm_residual"] = lambda: K.layer_norm_forward(attn_out, d["gamma"], d["beta"], (w.hidden,),
                                                                  workloads.EPS, residual=keep["x"])
+    if step_only:   # only the forms the step launches: a profile of the run then holds one form per kernel
+        for name in ("transpose_pad", "scale_mask_softmax", "attn_fused", "attn_fused_packed"):
+            if not w.decode:
+                fns.pop(name, None)
     table = {}
     for name, fn in fns.items():
         for _ in range(3):
@@ -572,6 +578,8 @@ def main(argv=None) -> int:
     ap.add_argument("--workload", default="c2", choices=["c1", "c2", "c3", "c4", "c5"])
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-extra", action="store_true", help="only the headline workload, no eager / other workloads")
+    ap.add_argument("--step-only", action="store_true",
+                    help="with --no-extra: launch nothing but the step and its own kernels (for profiles)")
     ap.add_argument("--copy-yardstick", action="store_true",
                     help="instead of the benchmark, time en_copy_bytes (plain 128-bit copy) at known sizes; "
                          "used as the bandwidth yardstick and to calibrate the FETCH_SIZE / WRITE_SIZE counters")
@@ -595,7 +603,10 @@ def main(argv=None) -> int:
 
     w = workloads.BY_NAME[ns.workload]
     torch.cuda.synchronize()
-    head = run_workload(torch, w, ns.steps, ns.warmup, want_eager=not ns.no_extra, want_kernels=True)
+    if ns.step_only:
+        ns.no_extra = True
+    head = run_workload(torch, w, ns.steps, ns.warmup, want_eager=not ns.no_extra, want_kernels=True,
+                        step_only=ns.step_only)
     torch.cuda.synchronize()
 
     # roofline of the kernel that takes the largest share of the step
