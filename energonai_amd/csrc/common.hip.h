@@ -167,4 +167,11 @@ __device__ __forceinline__ float block_allreduce(float v, float *slots) {
   return r;
 }
 
+// pad.hip: depad and transpose_pad (of all head_num rows per token; valid rows only when zero_padding == 0) in
+// one launch when both move 16-byte multiples, as two launches otherwise.  Same results as en_depad followed
+// by en_transpose_pad_heads.
+int depad_and_transpose_pad(const void *hidden_padded, void *x_packed, const void *qkv_packed, void *qkv_padded,
+                            const int32_t *cu_seqlens, int batch, int max_seq_len, int64_t hidden, int head_num,
+                            int size_per_head, int elem_size, int left_padded, int zero_padding, hipStream_t stream);
+
 }  // namespace en

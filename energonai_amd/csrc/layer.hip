@@ -1,9 +1,10 @@
-// The whole padding-removal step behind one call: the seven launches of
+// The whole padding-removal step behind one call: the seven ops
 //   depad -> transpose_pad -> QK^T -> scale_mask_softmax -> PV -> transpose_depad -> residual + LayerNorm
-// issued back to back on the caller's stream.  Nothing new is computed here -- every launch goes
-// through the entry point of its op -- but a Python caller pays for one foreign call instead of
-// seven, which is what bounds small batches (seven calls cost about 60 us of host time, more than
-// the GPU needs for a BERT-base batch of a few hundred tokens).
+// issued back to back on the caller's stream.  Nothing new is computed here -- every op runs the kernel
+// its entry point runs -- but a Python caller pays for one foreign call instead of seven, which is what
+// bounds small batches (seven calls cost about 60 us of host time, more than the GPU needs for a BERT-base
+// batch of a few hundred tokens), and depad, which depends on nothing before the LayerNorm, shares the
+// launch of transpose_pad: six launches.
 #include "common.hip.h"
 
 extern "C" int en_padding_removal_layer(const void *hidden_padded, const void *qkv_packed, const void *dense_out,
@@ -28,7 +29,9 @@ extern "C" int en_padding_removal_layer(const void *hidden_padded, const void *q
   if (total_tokens == 0) return EN_OK;
   const int B = batch, S = max_seq_len, H = head_num, D = size_per_head;
   int rc = EN_OK;
-  if (!fold_depad_offsets) {
+  // depad depends on nothing the attention chain produces: with transpose_pad to run it shares that launch
+  const bool depad_alone = !fold_depad_offsets && attention_form == 2;
+  if (depad_alone) {
     rc = en_depad(hidden_padded, x_packed, cu_seqlens, B, S, hidden, es, left_padded, stream);
     if (rc) return rc;
   }
@@ -44,7 +47,11 @@ extern "C" int en_padding_removal_layer(const void *hidden_padded, const void *q
     if (rc) return rc;
   } else {
     // the attention entry points never read a row at or past a sequence's length: no zero fill of the padding
-    rc = en_transpose_pad_heads(qkv_packed, qkv_padded, cu_seqlens, B, S, H, 3 * D, H, 0, 0, es, stream);
+    if (fold_depad_offsets)
+      rc = en_transpose_pad_heads(qkv_packed, qkv_padded, cu_seqlens, B, S, H, 3 * D, H, 0, 0, es, stream);
+    else
+      rc = depad_and_transpose_pad(hidden_padded, x_packed, qkv_packed, qkv_padded, cu_seqlens, B, S, hidden, H, 3 * D,
+                                   es, left_padded, 0, (hipStream_t)stream);
     if (rc) return rc;
     // q, k, v are the thirds of the last dimension of the padded [B,H,S,3D] buffer
     const int64_t sb = (int64_t)H * S * 3 * D, sh = (int64_t)S * 3 * D, ss = 3 * D;

@@ -83,7 +83,7 @@ _FORMS = {False: 0, True: 1, "packed": 2}
 
 def _layer_one_call(hidden_padded, qkv_packed, info, B, S, H, D, hid, T, gamma, beta, eps, scale, causal, left_padded,
                     dense_out, fused_attention, fold_depad=False):
-    """The same seven launches through ``en_padding_removal_layer``: one foreign call per step."""
+    """The same seven ops through ``en_padding_removal_layer``: one foreign call per step."""
     dev, dt = hidden_padded.device, hidden_padded.dtype
     form = _FORMS[fused_attention]
     _lib.require_gpu(hidden_padded, "hidden_padded")
