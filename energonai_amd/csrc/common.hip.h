@@ -44,18 +44,21 @@ template <> struct Elem<EN_F32> {
   static constexpr int kSize = 4;
   __device__ static __forceinline__ float to_float(T v) { return v; }
   __device__ static __forceinline__ T from_float(float f) { return f; }
+  static constexpr uint32_t kNegInfWord = 0xff800000u;   // -inf in every element of a 32-bit word
 };
 template <> struct Elem<EN_F16> {
   typedef half_t T;
   static constexpr int kSize = 2;
   __device__ static __forceinline__ float to_float(T v) { return (float)v; }
   __device__ static __forceinline__ T from_float(float f) { return (T)f; }
+  static constexpr uint32_t kNegInfWord = 0xfc00fc00u;
 };
 template <> struct Elem<EN_BF16> {
   typedef uint16_t T;
   static constexpr int kSize = 2;
   __device__ static __forceinline__ float to_float(T v) { return bf16_bits_to_float(v); }
   __device__ static __forceinline__ T from_float(float f) { return float_to_bf16_bits(f); }
+  static constexpr uint32_t kNegInfWord = 0xff80ff80u;
 };
 
 // N elements of T moved as one access (N * sizeof(T) is 4, 8 or 16 bytes).

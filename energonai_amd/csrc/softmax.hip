@@ -108,7 +108,7 @@ __global__ __launch_bounds__(kRowsBlock) void softmax_rows_kernel(SoftmaxArgs a)
 #pragma unroll
     for (int j = 0; j < VPL; ++j) {
       const int e0 = (l + LPR * j) * EPV;
-      raw[i][j] = make_uint4(0u, 0u, 0u, 0u);
+      raw[i][j] = make_uint4(E::kNegInfWord, E::kNegInfWord, E::kNegInfWord, E::kNegInfWord);   // not visible: -inf
       if (ri[i].active && e0 < ri[i].n) raw[i][j] = load16<false>(rowp + e0);
     }
   }
@@ -117,34 +117,42 @@ __global__ __launch_bounds__(kRowsBlock) void softmax_rows_kernel(SoftmaxArgs a)
 #pragma unroll
   for (int i = 0; i < R; ++i) {
     const int n = ri[i].n;
-    // vectors that lie wholly past the visible prefix cost no arithmetic: they are written as zeros
+    // A vector step is skipped when no lane of the wave holds a visible key in it (one scalar branch); in a
+    // step that runs, vectors past a row's prefix hold -inf from the load above and need no masking, so only
+    // the one vector of a row that straddles the end of the prefix is masked element by element.  -inf stays
+    // -inf through the scaling (the scale is positive) and exp2 turns it into the zero it must become.
     float x[VPL][EPV];
+    bool any[VPL];
     float m = -INFINITY;
 #pragma unroll
     for (int j = 0; j < VPL; ++j) {
       const int e0 = (l + LPR * j) * EPV;
-      if (e0 < n) {
+      any[j] = __builtin_amdgcn_ballot_w64(e0 < n) != 0ull;
+      if (any[j]) {
         const Pack<T, EPV> pk = __builtin_bit_cast(Pack<T, EPV>, raw[i][j]);
 #pragma unroll
-        for (int e = 0; e < EPV; ++e) {
-          const float v = (e0 + e < n) ? E::to_float(pk.v[e]) : -INFINITY;
-          x[j][e] = v;
-          m = fmaxf(m, v);
+        for (int e = 0; e < EPV; ++e) x[j][e] = E::to_float(pk.v[e]);
+        const int nv = n - e0;                      // visible elements of this vector
+        if (nv > 0 && nv < EPV) {
+#pragma unroll
+          for (int e = 1; e < EPV; ++e)
+            if (e >= nv) x[j][e] = -INFINITY;
         }
+#pragma unroll
+        for (int e = 0; e < EPV; ++e) m = fmaxf(m, x[j][e]);
       }
     }
     m = group_allreduce<OpMax, LPR>(m);
-    // exp(scale * (x - m)) = exp2(x * c - m * c), c = scale * log2(e) >= 0 (negative scales take the generic kernel)
+    // exp(scale * (x - m)) = exp2(x * c - m * c), c = scale * log2(e) > 0 (other scales take the generic kernel)
     const float c = a.scale * kLog2e;
     const float moff = (m == -INFINITY) ? 0.f : -m * c;  // nothing visible: all zeros, no NaN
     float s = 0.f;
 #pragma unroll
     for (int j = 0; j < VPL; ++j) {
-      const int e0 = (l + LPR * j) * EPV;
-      if (e0 < n) {
+      if (any[j]) {
 #pragma unroll
         for (int e = 0; e < EPV; ++e) {
-          const float ex = (x[j][e] == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(fmaf(x[j][e], c, moff));
+          const float ex = __builtin_amdgcn_exp2f(fmaf(x[j][e], c, moff));
           x[j][e] = ex;
           s += ex;
         }
@@ -156,16 +164,14 @@ __global__ __launch_bounds__(kRowsBlock) void softmax_rows_kernel(SoftmaxArgs a)
 #pragma unroll
     for (int j = 0; j < VPL; ++j) {
       const int e0 = (l + LPR * j) * EPV;
-      if (ri[i].active && e0 < ri[i].lim) {
-        uint4 out = make_uint4(0u, 0u, 0u, 0u);
-        if (e0 < n) {
-          Pack<T, EPV> pk;
+      uint4 out = make_uint4(0u, 0u, 0u, 0u);
+      if (any[j]) {                                 // masked elements are exact zeros by now
+        Pack<T, EPV> pk;
 #pragma unroll
-          for (int e = 0; e < EPV; ++e) pk.v[e] = E::from_float(x[j][e] * inv);
-          out = __builtin_bit_cast(uint4, pk);
-        }
-        store16<false>(rowp + e0, out);
+        for (int e = 0; e < EPV; ++e) pk.v[e] = E::from_float(x[j][e] * inv);
+        out = __builtin_bit_cast(uint4, pk);
       }
+      if (ri[i].active && e0 < ri[i].lim) store16<false>(rowp + e0, out);
     }
   }
 }
@@ -210,7 +216,7 @@ static int dispatch(const SoftmaxArgs &a, hipStream_t s) {
   constexpr int EPV = 16 / Elem<DT>::kSize;
   const bool vec_ok = (a.Sk % EPV) == 0 && aligned_to(a.src, 16);
   const int64_t nvec = vec_ok ? a.Sk / EPV : 0;
-  if (!vec_ok || nvec > 64 * 16 || !(a.scale >= 0.f)) {
+  if (!vec_ok || nvec > 64 * 16 || !(a.scale > 0.f)) {
     softmax_generic_kernel<DT><<<dim3((unsigned)a.rows_per_batch, (unsigned)a.B, 1), kBlock, 0, s>>>(a);
   }
   // Few lanes per row for short rows: a causal row uses on average half of its sequence, so narrow
