@@ -279,6 +279,11 @@ __global__ __launch_bounds__(kBlock, 3) void attn_qk_strip_kernel(AttnArgs a) {
 
   fetch_k();
   stage_k(lds_k[0]);
+  // The Q fragments are used here, before the loop, so that the wait for their loads is placed here too.  Left
+  // to the loop, that wait ("at most the four newest memory operations outstanding") would on every later
+  // iteration also wait for the previous tile's score stores to be acknowledged.
+#pragma unroll
+  for (int vs = 0; vs < NVS; ++vs) asm volatile("" ::"v"(qf[vs].x), "v"(qf[vs].y), "v"(qf[vs].z), "v"(qf[vs].w));
   lds_barrier();
   for (int kt = 0; kt < nkt; ++kt) {
     const int k0 = kt * BK;
