@@ -42,9 +42,15 @@ __global__ __launch_bounds__(STREAM ? kStreamBlock : kBlock) void decode_qk_kern
   const T *kbase = reinterpret_cast<const T *>(a.kv) + (int64_t)b * a.sb + (int64_t)h * a.sh;
   T *srow = reinterpret_cast<T *>(a.out) + ((int64_t)b * a.H + h) * a.Sk;
 
+  // head sizes that are not a power-of-two number of vectors (80, 96) run on the next power of two of
+  // lanes per key; the lanes past the head load nothing and add zeros
+  const bool cv = c * EPV < a.D;
   float qv[EPV];
   {
-    const Pack<T, EPV> pk = load_pack<T, EPV>(q + c * EPV);
+    Pack<T, EPV> pk;
+#pragma unroll
+    for (int e = 0; e < EPV; ++e) pk.v[e] = E::from_float(0.f);
+    if (cv) pk = load_pack<T, EPV>(q + c * EPV);
 #pragma unroll
     for (int e = 0; e < EPV; ++e) qv[e] = E::to_float(pk.v[e]) * a.alpha;
   }
@@ -53,13 +59,13 @@ __global__ __launch_bounds__(STREAM ? kStreamBlock : kBlock) void decode_qk_kern
 #pragma unroll
     for (int u = 0; u < U; ++u) {
       const int key = k0 + u * KPS + slot;
-      if (key < kl) kv[u] = __builtin_bit_cast(Pack<T, EPV>, load16<STREAM>(kbase + (int64_t)key * a.ss + c * EPV));
+      if (key < kl && cv) kv[u] = __builtin_bit_cast(Pack<T, EPV>, load16<STREAM>(kbase + (int64_t)key * a.ss + c * EPV));
     }
 #pragma unroll
     for (int u = 0; u < U; ++u) {
       const int key = k0 + u * KPS + slot;
       float dot = 0.f;
-      if (key < kl) {
+      if (key < kl && cv) {
 #pragma unroll
         for (int e = 0; e < EPV; ++e) dot += qv[e] * E::to_float(kv[u].v[e]);
       }
@@ -85,6 +91,7 @@ __global__ __launch_bounds__(STREAM ? kStreamBlock : kBlock) void decode_pv_kern
   const T *prow = reinterpret_cast<const T *>(a.x) + ((int64_t)b * a.H + h) * a.Sk;
   const T *vbase = reinterpret_cast<const T *>(a.kv) + (int64_t)b * a.sb + (int64_t)h * a.sh;
   T *ctx = reinterpret_cast<T *>(a.out) + ((int64_t)b * a.H + h) * a.D;
+  const bool cv = c * EPV < a.D;     // lanes past the head size idle (head sizes such as 80 and 96)
 
   float acc[EPV];
 #pragma unroll
@@ -96,7 +103,7 @@ __global__ __launch_bounds__(STREAM ? kStreamBlock : kBlock) void decode_pv_kern
     for (int u = 0; u < U; ++u) {
       const int key = k0 + u * KPS;
       p[u] = 0.f;
-      if (key < kl) {
+      if (key < kl && cv) {
         vv[u] = __builtin_bit_cast(Pack<T, EPV>, load16<STREAM>(vbase + (int64_t)key * a.ss + c * EPV));
         p[u] = E::to_float(prow[key]);
       }
@@ -104,7 +111,7 @@ __global__ __launch_bounds__(STREAM ? kStreamBlock : kBlock) void decode_pv_kern
 #pragma unroll
     for (int u = 0; u < U; ++u) {
       const int key = k0 + u * KPS;
-      if (key < kl) {
+      if (key < kl && cv) {
 #pragma unroll
         for (int e = 0; e < EPV; ++e) acc[e] += p[u] * E::to_float(vv[u].v[e]);
       }
@@ -124,7 +131,8 @@ __global__ __launch_bounds__(STREAM ? kStreamBlock : kBlock) void decode_pv_kern
 template <int DT, template <int, int> class Launcher>
 static int dispatch_lpk(const DecodeArgs &a, int batch, hipStream_t s) {
   constexpr int EPV = 16 / Elem<DT>::kSize;
-  const int lpk = a.D / EPV;
+  int lpk = 4;                                 // lanes per key: vectors in a head, rounded up to a power of two
+  while (lpk * EPV < a.D) lpk *= 2;
   dim3 grid((unsigned)a.H, (unsigned)batch, 1);
   switch (lpk) {
     case 4: Launcher<DT, 4>::go(a, grid, s); break;

@@ -195,7 +195,8 @@ int en_attn_pv(const void *p, const void *v, void *ctx, const int32_t *k_lens, c
  * square each step, energonai/model/attention.py:61-71,106-118).
  * q [B,H,D] contiguous, k_cache/v_cache [B,H,Smax,D] with strides as above,
  * scores/p [B,H,Smax] contiguous, ctx [B,H,D] contiguous.  Streaming kernels:
- * bound by the K/V bytes read. */
+ * bound by the K/V bytes read.  D a multiple of 8 (16-bit) / 4 (fp32), up to
+ * 512 / 256; head sizes such as 80 and 96 are supported. */
 int en_decode_qk(const void *q, const void *k_cache, void *scores, const int32_t *kv_lens, int batch, int head_num,
                  int k_seq_len, int size_per_head, int64_t k_stride_b, int64_t k_stride_h, int64_t k_stride_s,
                  float alpha, int dtype, en_stream_t stream);

@@ -147,6 +147,7 @@ DECODE_CASES = [
     (5, 4, 640, 128, [640, 1, 333, 64, 65]),
     (3, 2, 100, 64, [100, 17, 2]),
     (2, 3, 77, 32, [77, 40]),
+    (3, 4, 200, 80, [200, 1, 77]),        # OPT-2.7B head size: ten vectors per key, run on sixteen lanes
     (4, 72, 2048, 128, [2048, 3, 1024, 1989]),
 ]
 

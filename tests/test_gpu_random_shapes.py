@@ -120,3 +120,76 @@ def test_layernorm_random_shapes(seed):
     assert max_abs(y.cpu(), wy) <= tol * max(1.0, float(wy.abs().max()))
     assert max_abs(mean.cpu(), wmean) <= 1e-5 * max(1.0, float(wmean.abs().max()))
     assert max_abs(invvar.cpu(), winv) <= 2e-5 * max(1.0, float(winv.abs().max()))
+
+
+@pytest.mark.parametrize("seed", list(range(10)))
+def test_decode_random_shapes(seed):
+    """Single-query QK^T -> softmax -> PV against a ragged cache whose unused rows hold NaN."""
+    k = _kernel()
+    ri = _draw(7300 + seed)
+    B, H = ri(1, 7), ri(1, 6)
+    D = [32, 64, 80, 96, 128][ri(0, 4)]
+    S = 8 * ri(1, 150)
+    dtype = [torch.float16, torch.bfloat16, torch.float32][ri(0, 2)]
+    kv = [ri(1, S) for _ in range(B)]
+    kv[ri(0, B - 1)] = S
+    announce("decode random", seed, B, H, S, D, dtype, kv)
+    g = torch.Generator().manual_seed(seed)
+    q = torch.randn(B, H, 1, D, generator=g).to(dtype)
+    kc = torch.randn(B, H, S, D, generator=g).to(dtype)
+    vc = torch.randn(B, H, S, D, generator=g).to(dtype)
+    for b, n in enumerate(kv):
+        kc[b, :, n:] = float("nan")
+        vc[b, :, n:] = float("nan")
+    kv_t = torch.tensor(kv, dtype=torch.int32).cuda()
+    scale = D ** -0.5
+    _, want_probs, want_ctx = eager.decode_attention(q, torch.nan_to_num(kc, nan=0.0), torch.nan_to_num(vc, nan=0.0),
+                                                     kv, scale, acc_dtype=torch.float64)
+    scores = k.decode_qk(q.cuda(), kc.cuda(), kv_t)
+    probs = k.scale_mask_softmax(B, 1, H, scores, kv_t, scale=scale, k_seq_len=S,
+                                 q_len_list=torch.ones(B, dtype=torch.int32).cuda())
+    tol = {torch.float16: 2e-3, torch.bfloat16: 1.6e-2, torch.float32: 1e-5}[dtype]
+    assert max_abs(probs.cpu(), want_probs) <= tol
+    ctx = k.decode_pv(probs, vc.cuda(), kv_t).cpu()
+    assert torch.isfinite(ctx).all()
+    assert max_abs(ctx, want_ctx) <= tol * max(1.0, float(want_ctx.abs().max()))
+
+
+@pytest.mark.parametrize("seed", list(range(10)))
+def test_ft_family_random_shapes(seed):
+    """The offset-based helpers: offsets, remove / rebuild, the three-tensor transposing pair; bit-exact."""
+    k = _kernel()
+    ri = _draw(7400 + seed)
+    B, S, H = ri(1, 8), ri(1, 200), ri(1, 6)
+    D = [2, 4, 8, 24, 64, 128][ri(0, 5)]
+    dtype = [torch.float16, torch.float32][ri(0, 1)]
+    lens = _lens(ri, B, S)
+    lens[0] = max(lens[0], 1)                    # at least one token
+    hid = H * D
+    announce("ft random", seed, B, S, H, D, dtype, lens)
+    want_valid, want_off = eager.ft_build_padding_offsets(lens, B, S)
+    T = int(want_valid[0])
+    tmp_off = torch.full((B, S), -7, dtype=torch.int32).cuda()
+    mask_off = torch.full((B, S), -9, dtype=torch.int32).cuda()
+    valid = torch.zeros(1, dtype=torch.int32).cuda()
+    k.ft_build_padding_offsets(torch.tensor(lens, dtype=torch.int32).cuda(), B, S, valid, tmp_off)
+    assert int(valid[0].item()) == T and torch.equal(tmp_off.flatten()[:T].cpu(), want_off)
+    g = torch.Generator().manual_seed(seed)
+    hq, hk, hv = (torch.rand(B, S, hid, generator=g).to(dtype) for _ in range(3))
+    q = k.ft_remove_padding(hq.cuda(), tmp_off, mask_off, T, hid)
+    want_q, want_mask = eager.ft_remove_padding(hq, want_off, T, hid)
+    assert torch.equal(q.cpu(), want_q) and torch.equal(mask_off.flatten()[:T].cpu(), want_mask)
+    kk = k.ft_remove_padding(hk.cuda(), tmp_off, mask_off, T, hid)
+    v = k.ft_remove_padding(hv.cuda(), tmp_off, mask_off, T, hid)
+    bufs = [torch.full((B, H, S, D), 3.0, dtype=dtype).cuda() for _ in range(3)]
+    k.ft_transpose_rebuild_padding(q.view(T, H, D), kk.view(T, H, D), v.view(T, H, D), bufs[0], bufs[1], bufs[2],
+                                   B, S, H, D, T, mask_off)
+    want_bufs = [torch.full((B, H, S, D), 3.0, dtype=dtype) for _ in range(3)]
+    eager.ft_transpose_rebuild_padding(q.cpu().view(T, H, D), kk.cpu().view(T, H, D), v.cpu().view(T, H, D),
+                                       *want_bufs, B, S, H, D, T, want_mask)
+    for got, want in zip(bufs, want_bufs):
+        assert torch.equal(got.cpu(), want)
+    back = k.ft_transpose_remove_padding(bufs[1], T, B, S, H, D, mask_off)
+    assert torch.equal(back, kk)
+    rebuilt = k.ft_rebuild_padding(back, mask_off, T, hid, B, S)
+    assert torch.equal(rebuilt.cpu(), eager.ft_rebuild_padding(back.cpu(), want_mask, T, hid, B, S))
