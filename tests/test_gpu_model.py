@@ -267,3 +267,41 @@ def test_packed_stack_prefill_and_decode(dtype):
         want = reference(x, valid)
         assert got.shape == want.shape
         assert max_abs(got[:, -1].float().cpu(), want[:, -1]) <= tol * scale, step
+
+
+@pytest.mark.parametrize("seed", list(range(10)))
+def test_block_random_shapes(seed):
+    """Block1D on drawn shapes (head sizes 32 / 64 / 80 / 128, pre- or post-LN, ReLU / tanh-GELU / erf-GELU,
+    fused or separate projections): prefill, then two incremental steps, against the reference block."""
+    import functools
+    _, M = _mods()
+    g = torch.Generator().manual_seed(9100 + seed)
+    ri = lambda lo, hi: int(torch.randint(lo, hi + 1, (1,), generator=g))
+    heads, D = ri(1, 4), [32, 64, 80, 128][ri(0, 3)]
+    hid = heads * D
+    B, S = ri(1, 5), ri(2, 90)
+    dtype = [torch.float16, torch.float32, torch.bfloat16][ri(0, 2)]
+    post, fused_qkv = bool(ri(0, 1)), bool(ri(0, 1))
+    act_name = ["relu", "gelu_tanh", "gelu"][ri(0, 2)]
+    act = {"relu": F.relu, "gelu_tanh": functools.partial(F.gelu, approximate="tanh"), "gelu": F.gelu}[act_name]
+    lens = [ri(1, S) for _ in range(B)]
+    lens[ri(0, B - 1)] = S
+    announce("block random", seed, B, S, heads, D, dtype, post, fused_qkv, act_name, lens)
+    blk = M.Block1D(hid, heads, 4.0, activation=act, dtype=dtype, apply_post_layernorm=post, max_seq_len=S + 8,
+                    fused_qkv=fused_qkv).cuda()
+    _init(blk, 9200 + seed)
+    p = _fp32_params(blk)
+    x, valid = _padded_batch(B, S, hid, lens, True, dtype, 9300 + seed)
+    tol = {torch.float16: 2e-2, torch.bfloat16: 1.5e-1, torch.float32: 1e-3}[dtype]
+    mask = models.additive_mask(valid)
+    got = blk(x.cuda(), attention_mask=mask.to(dtype).cuda(), first_cache=True).float().cpu()
+    want = models.block_forward(x, p, heads, 1e-5, post, True, mask, activation=act, fused_qkv=fused_qkv)
+    ref_scale = max(1.0, float(want.abs().max()))
+    assert max_abs(_valid_rows(got, lens, True), _valid_rows(want, lens, True)) <= tol * ref_scale
+    for step in range(2):
+        x = torch.cat((x, torch.randn(B, 1, hid, generator=g).to(dtype)), 1)
+        valid = torch.cat((valid, torch.ones(B, 1)), 1)
+        mask = models.additive_mask(valid)
+        got = blk(x.cuda(), attention_mask=mask.to(dtype).cuda(), first_cache=False).float().cpu()
+        want = models.block_forward(x, p, heads, 1e-5, post, True, mask, activation=act, fused_qkv=fused_qkv)
+        assert max_abs(got[:, -1], want[:, -1]) <= tol * ref_scale, step

@@ -193,3 +193,50 @@ def test_ft_family_random_shapes(seed):
     assert torch.equal(back, kk)
     rebuilt = k.ft_rebuild_padding(back, mask_off, T, hid, B, S)
     assert torch.equal(rebuilt.cpu(), eager.ft_rebuild_padding(back.cpu(), want_mask, T, hid, B, S))
+
+
+@pytest.mark.parametrize("seed", list(range(14)))
+def test_layer_random_shapes(seed):
+    """The whole step on drawn shapes (LayerNorm width equal to or different from heads x head size, either
+    padding side, causal or not, every attention form, depad folded or not) against the oracle's layer."""
+    from energonai_amd import layer
+    ri = _draw(7500 + seed)
+    B, S, H = ri(1, 6), 8 * ri(1, 40), ri(1, 4)
+    D = [32, 64, 80, 128][ri(0, 3)]
+    dtype = [torch.float16, torch.bfloat16, torch.float32][ri(0, 2)]
+    wide = bool(ri(0, 1))                       # a dense projection between attention and LayerNorm
+    hid = 8 * ri(4, 160) if wide else H * D
+    causal, left = bool(ri(0, 1)), bool(ri(0, 1))
+    lens = _lens(ri, B, S)
+    if sum(lens) == 0:
+        lens[0] = S
+    T = sum(lens)
+    announce("layer random", seed, B, S, H, D, hid, dtype, causal, left, lens)
+    g = torch.Generator().manual_seed(seed)
+    x = torch.randn(B, S, hid, generator=g).to(dtype)
+    qkv = torch.randn(1, T, H, 3 * D, generator=g).to(dtype)
+    dense = torch.randn(1, T, hid, generator=g).to(dtype) if wide else None
+    gamma = (1.0 + 0.05 * torch.randn(hid, generator=g)).to(dtype)
+    beta = (0.05 * torch.randn(hid, generator=g)).to(dtype)
+    scale = D ** -0.5
+    want = eager.layer_unpadded(x, qkv, lens, H, D, gamma, beta, 1e-5, scale, causal, left, dense_out=dense,
+                                acc_dtype=torch.float64)
+    args = (x.cuda(), qkv.cuda(), torch.tensor(lens, dtype=torch.int32).cuda(), H, D, gamma.cuda(), beta.cuda(),
+            1e-5, scale, causal, left)
+    dense_g = None if dense is None else dense.cuda()
+    tol_ctx = {torch.float16: 3e-3, torch.bfloat16: 2.5e-2, torch.float32: 2e-5}[dtype]
+    tol_y = {torch.float16: 8e-3, torch.bfloat16: 6e-2, torch.float32: 5e-5}[dtype]
+    kept = layer.padding_removal_layer(*args, dense_out=dense_g, keep=True)
+    assert torch.equal(kept["x"].cpu(), want["x"].to(dtype))
+    scale_c = max(1.0, float(want["ctx_packed"].abs().max()))
+    assert max_abs(kept["ctx_packed"].cpu(), want["ctx_packed"]) <= tol_ctx * scale_c
+    scale_y = max(1.0, float(want["y"].abs().max()))
+    forms = [(False, False), (False, True)]
+    if dtype != torch.float32:
+        forms += [(True, False), ("packed", False), ("packed", True)]
+    for form, fold in forms:
+        y = layer.padding_removal_layer(*args, dense_out=dense_g, fused_attention=form, fold_depad=fold)
+        assert y.shape == (1, T, hid)
+        assert max_abs(y.cpu(), want["y"]) <= tol_y * scale_y, (form, fold)
+        if not form:
+            assert torch.equal(y, kept["y"]), (form, fold)      # the one-call step gives the op-by-op bits
