@@ -595,6 +595,8 @@ def main(argv=None) -> int:
         print("bench.py needs a GPU", file=sys.stderr)
         return 2
     torch.cuda.set_device(0)
+    from energonai_amd import build as hip_build
+    hip_build.ensure_built()      # loads what is built; compiles only when nothing is
     from energonai_amd import workloads
 
     if ns.copy_yardstick:

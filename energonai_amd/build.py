@@ -99,6 +99,13 @@ def build_linear() -> str:
     return LINEAR_LIB_PATH
 
 
+def ensure_built() -> None:
+    """Builds the two libraries if, and only if, one of them is missing (tests, the smoke run and the
+    benchmark load what is there; they compile only when nothing is)."""
+    if not (os.path.exists(LIB_PATH) and os.path.exists(LINEAR_LIB_PATH)):
+        build(force=False)
+
+
 def main(argv=None) -> int:
     ap = argparse.ArgumentParser(description=__doc__)
     ap.add_argument("--force", action="store_true", help="recompile every source")

@@ -12,6 +12,13 @@ def pytest_configure(config):
     config.addinivalue_line("markers", "gpu: needs a real MI355X (run with -m gpu on the GPU box)")
 
 
+@pytest.fixture(scope="session", autouse=True)
+def _libraries_are_built():
+    """The tests load the libraries that are in the tree; they are compiled here only when none is."""
+    from energonai_amd import build
+    build.ensure_built()
+
+
 def _has_gpu() -> bool:
     try:
         import torch
