@@ -22,6 +22,7 @@ _DTYPE_TAG = {torch.float32: EN_F32, torch.float16: EN_F16, torch.bfloat16: EN_B
 # name -> (restype, argtypes); must list every symbol the header declares
 SIGNATURES = {
     "en_version": (c_int, []),
+    "en_source_hash": (c_char_p, []),
     "en_status_string": (c_char_p, [c_int]),
     "en_last_hip_error": (c_int, []),
     "en_last_hip_error_string": (c_char_p, []),
@@ -56,10 +57,23 @@ LINEAR_SIGNATURES = {
     "en_linear": (c_int, [c_void_p] * 4 + [c_int64] * 3 + [c_int] * 3 + [c_void_p, c_int64, c_void_p]),
     "en_linear_algo_count": (c_int, [c_int64] * 3 + [c_int] * 3 + [c_int64]),
     "en_linear_status_string": (ctypes.c_char_p, [c_int]),
+    "en_linear_source_hash": (ctypes.c_char_p, []),
 }
 
 _lib = None
 _linear_lib = None
+
+
+def _refuse_stale(lib, symbol: str, expected: str, path: str) -> None:
+    """A library compiled from other sources than the ones beside it would make every test and measurement
+    speak for code that is not in the tree."""
+    fn_ = getattr(lib, symbol)
+    fn_.restype = c_char_p
+    fn_.argtypes = []
+    built = fn_().decode()
+    if built != expected:
+        raise RuntimeError(f"energonai_amd requires cuda extensions: {path} was built from other sources "
+                           f"(library {built}, tree {expected}); run `python -m energonai_amd.build`")
 
 
 def load_linear() -> ctypes.CDLL:
@@ -73,6 +87,8 @@ def load_linear() -> ctypes.CDLL:
             lib = ctypes.CDLL(LINEAR_LIB_PATH)
         except OSError as exc:
             raise RuntimeError(f"energonai_linear_func requires cuda extensions: cannot load {LINEAR_LIB_PATH}: {exc}") from exc
+        from . import build
+        _refuse_stale(lib, "en_linear_source_hash", build.linear_source_hash(), LINEAR_LIB_PATH)
         for name, (restype, argtypes) in LINEAR_SIGNATURES.items():
             fn = getattr(lib, name)
             fn.restype = restype
@@ -93,6 +109,8 @@ def load() -> ctypes.CDLL:
             lib = ctypes.CDLL(LIB_PATH)
         except OSError as exc:
             raise RuntimeError(f"energonai_amd requires cuda extensions: cannot load {LIB_PATH}: {exc}") from exc
+        from . import build
+        _refuse_stale(lib, "en_source_hash", build.source_hash(), LIB_PATH)
         for name, (restype, argtypes) in SIGNATURES.items():
             fn = getattr(lib, name)
             fn.restype = restype

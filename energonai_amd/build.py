@@ -11,6 +11,7 @@ for gfx950 without a GPU present.
 from __future__ import annotations
 
 import argparse
+import hashlib
 import os
 import shutil
 import subprocess
@@ -50,6 +51,28 @@ def sources() -> list:
     return sorted(os.path.join(CSRC, f) for f in os.listdir(CSRC) if f.endswith(".hip"))
 
 
+def _digest(paths) -> str:
+    h = hashlib.sha256()
+    for path in sorted(paths, key=os.path.basename):
+        h.update(os.path.basename(path).encode() + b"\0")
+        with open(path, "rb") as f:
+            h.update(f.read())
+        h.update(b"\0")
+    return h.hexdigest()[:32]
+
+
+def source_hash() -> str:
+    """Digest of every file libenergon_hip.so is compiled from.  The build stores it in the library
+    (``en_source_hash``); loading compares the two, so a library older than the sources next to it is
+    refused instead of silently tested."""
+    return _digest(sources() + [os.path.join(CSRC, f) for f in os.listdir(CSRC) if f.endswith(".h")] +
+                   [os.path.join(INCLUDE, "energon_hip.h")])
+
+
+def linear_source_hash() -> str:
+    return _digest([LINEAR_SRC, os.path.join(INCLUDE, "energon_linear.h")])
+
+
 def _stale(src: str, obj: str) -> bool:
     if not os.path.exists(obj):
         return True
@@ -61,8 +84,10 @@ def _stale(src: str, obj: str) -> bool:
 
 def _compile(src: str, force: bool, verbose: bool) -> str:
     obj = os.path.join(OBJ_DIR, os.path.basename(src) + ".o")
-    if force or _stale(src, obj):
-        cmd = [_hipcc()] + HIPCC_FLAGS + ["-c", src, "-o", obj]
+    carries_hash = os.path.basename(src) == "abi.hip"     # recompiled every time: the digest changes with any source
+    if force or carries_hash or _stale(src, obj):
+        cmd = [_hipcc()] + HIPCC_FLAGS + ([f'-DEN_SOURCE_HASH="{source_hash()}"'] if carries_hash else []) + \
+              ["-c", src, "-o", obj]
         proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
         out = "\n".join(l for l in proc.stdout.splitlines() if "packed-fp32-ops" not in l)
         if proc.returncode != 0:
@@ -90,7 +115,8 @@ def build(force: bool = True, verbose: bool = False, jobs: int = 4) -> str:
 def build_linear() -> str:
     rocm_lib = os.path.join(os.path.dirname(os.path.dirname(os.path.realpath(_hipcc()))), "lib")
     tmp = LINEAR_LIB_PATH + ".tmp"
-    cmd = [_hipcc(), "-O2", "-std=c++17", "-fPIC", "-shared", f"-I{INCLUDE}", LINEAR_SRC, "-o", tmp,
+    cmd = [_hipcc(), "-O2", "-std=c++17", "-fPIC", "-shared", f"-I{INCLUDE}",
+           f'-DEN_SOURCE_HASH="{linear_source_hash()}"', LINEAR_SRC, "-o", tmp,
            f"-L{rocm_lib}", "-L/opt/rocm/lib", "-lhipblaslt", "-lamdhip64"]
     proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
     if proc.returncode != 0:

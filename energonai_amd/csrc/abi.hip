@@ -71,7 +71,12 @@ __global__ __launch_bounds__(kBlock) void copy_kernel(const uint4 *__restrict__ 
 
 extern "C" {
 
-int en_version(void) { return 100; }
+int en_version(void) { return 200; }
+
+#ifndef EN_SOURCE_HASH
+#define EN_SOURCE_HASH "unknown"
+#endif
+const char *en_source_hash(void) { return EN_SOURCE_HASH; }
 
 const char *en_status_string(int status) {
   switch (status) {

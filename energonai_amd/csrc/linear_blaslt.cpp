@@ -204,4 +204,9 @@ const char *en_linear_status_string(int status) {
   }
 }
 
+#ifndef EN_SOURCE_HASH
+#define EN_SOURCE_HASH "unknown"
+#endif
+const char *en_linear_source_hash(void) { return EN_SOURCE_HASH; }
+
 }  // extern "C"

@@ -198,7 +198,12 @@ __global__ __launch_bounds__(kBlock) void softmax_generic_kernel(SoftmaxArgs a) 
   for (int i = threadIdx.x; i < n; i += kBlock) s += __expf(E::to_float(rowp[i]) * a.scale - msafe);
   s = block_allreduce<OpSum, kBlock / kWave>(s, s_sum);
   const float inv = s > 0.f ? 1.0f / s : 0.f;
-  for (int i = threadIdx.x; i < ri.lim; i += kBlock) {
+  // The contraction that wrote the scores stored whole 16-byte vectors, and the one that reads the probabilities
+  // loads whole vectors as far as the row can see, with no mask inside a vector: like the register kernel, clear
+  // the vector that straddles the end of what is written, or its raw scores would be multiplied with real V rows.
+  constexpr int EPV = 16 / E::kSize;
+  const int lim = min((ri.lim + EPV - 1) / EPV * EPV, a.Sk);
+  for (int i = threadIdx.x; i < lim; i += kBlock) {
     const float p = (i < n) ? __expf(E::to_float(rowp[i]) * a.scale - msafe) * inv : 0.f;
     rowp[i] = E::from_float(p);
   }

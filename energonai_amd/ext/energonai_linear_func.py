@@ -7,8 +7,7 @@ from ..kernel.cuda_native import linear_func as _lf
 
 
 def mlp_gemm(tensor1, tensor2, algo=-1):
-    n = _lf.algo_count(tensor1.shape[0] * tensor1.shape[1], tensor1.shape[2], tensor2.shape[0], tensor1.dtype)
-    return _lf.linear(tensor1, tensor2, algo if 0 <= algo < n else -1)
+    return _lf.linear(tensor1, tensor2, algo)
 
 
 def get_start_algo():

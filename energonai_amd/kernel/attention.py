@@ -29,11 +29,12 @@ def _bhsd(t: torch.Tensor, name: str):
 
 
 def _lens_ptrs(seq_len_list, q_len_list, batch_size, device):
+    """Key lengths, query lengths (or None) and the raw pointer of the latter.  The caller keeps both objects
+    until its kernel is launched: lengths given as a list live in a device tensor that only they own, and a
+    tensor allocated in between could otherwise be handed the same memory."""
     k_info = seq_info(seq_len_list, batch_size, device)
-    q_ptr = 0
-    if q_len_list is not None:
-        q_ptr = seq_info(q_len_list, batch_size, device).lens.data_ptr()
-    return k_info, q_ptr
+    q_info = None if q_len_list is None else seq_info(q_len_list, batch_size, device)
+    return k_info, q_info, (0 if q_info is None else q_info.lens.data_ptr())
 
 
 def attn_qk(q, k, seq_len_list, *, alpha: float = 1.0, causal: bool = True, q_len_list=None,
@@ -50,7 +51,7 @@ def attn_qk(q, k, seq_len_list, *, alpha: float = 1.0, causal: bool = True, q_le
     if k.shape[0] != B or k.shape[1] != H or k.shape[3] != D or k.dtype != q.dtype:
         raise RuntimeError("attn_qk: q and k disagree in batch, heads, size_per_head or dtype")
     Sk = k.shape[2]
-    k_info, q_ptr = _lens_ptrs(seq_len_list, q_len_list, B, q.device)
+    k_info, q_info, q_ptr = _lens_ptrs(seq_len_list, q_len_list, B, q.device)
     if out is None:
         out = torch.empty((B, H, Sq, Sk), dtype=q.dtype, device=q.device)
     else:
@@ -78,7 +79,7 @@ def attn_pv(p, v, seq_len_list, *, causal: bool = True, q_len_list=None, zero_pa
     D = v.shape[3]
     if v.shape[0] != B or v.shape[1] != H or v.shape[2] != Sk or v.dtype != p.dtype:
         raise RuntimeError("attn_pv: p and v disagree in batch, heads, key length or dtype")
-    k_info, q_ptr = _lens_ptrs(seq_len_list, q_len_list, B, p.device)
+    k_info, q_info, q_ptr = _lens_ptrs(seq_len_list, q_len_list, B, p.device)
     if out is None:
         out = torch.empty((B, H, Sq, D), dtype=p.dtype, device=p.device)
     else:
@@ -110,7 +111,7 @@ def attn_fused(q, k, v, seq_len_list, *, scale: Optional[float] = None, causal: 
         raise RuntimeError("attn_fused: q, k, v disagree in batch, heads, size_per_head, key length or dtype")
     if q.dtype not in (torch.float16, torch.bfloat16):
         raise RuntimeError("attn_fused: Datatype not implemented (float16 and bfloat16 only)")
-    k_info, q_ptr = _lens_ptrs(seq_len_list, q_len_list, B, q.device)
+    k_info, q_info, q_ptr = _lens_ptrs(seq_len_list, q_len_list, B, q.device)
     if out is None:
         out = torch.empty((B, H, Sq, D), dtype=q.dtype, device=q.device)
     else:

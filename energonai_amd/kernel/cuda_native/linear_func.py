@@ -62,6 +62,12 @@ def linear(inputs, param, algo=-1, bias=None, activation: Optional[str] = None):
             raise RuntimeError("linear: bias must be [dout]")
     B, S, din = inputs.shape
     dout = param.shape[0]
+    if algo >= 0 and (algo <= 23 or 99 <= algo <= 115):
+        # every id the reference accepts (cuBLAS constants -1..23 and 99..115, csrc/linear_wrapper.cpp:133-140)
+        # is valid here too: one that lies past this problem's candidate list means the first choice
+        with _lib.device_guard(inputs):
+            if algo >= algo_count(B * S, din, dout, inputs.dtype, bias is not None, activation):
+                algo = -1
     out = torch.empty((B, S, dout), dtype=inputs.dtype, device=inputs.device)
     ws = _workspace(inputs.device)
     with _lib.device_guard(inputs):

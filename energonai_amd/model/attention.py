@@ -91,11 +91,14 @@ class MultiHeadAttention1D(nn.Module):
             ctx = transpose_depad(attn_pv(probs, pads[2], info, causal=self.is_decoder), batch_size, T, max_seq_len,
                                   info, H, D)
         if fill_cache:
+            if max_seq_len > self.max_seq_len:
+                raise RuntimeError(f"the batch is padded to {max_seq_len} positions but the K/V cache was planned for "
+                                   f"max_seq_len = {self.max_seq_len}")
             self.kv_cache = KVCache(batch_size, H, self.max_seq_len, D, x.dtype, x.device)
             if kvq is not None:
-                self.kv_cache.fill(kvq, kvq, info, 0, H)
+                self.kv_cache.fill(kvq, kvq, info, 0, H, longest=max_seq_len)
             else:
-                self.kv_cache.fill(k.contiguous(), v.contiguous(), info)
+                self.kv_cache.fill(k.contiguous(), v.contiguous(), info, longest=max_seq_len)
         return project(self.dense, ctx.view(1, T, self.hidden_size))
 
     # ---- one decode step: newest position only ----------------------------------------------

@@ -10,6 +10,8 @@ valid prefix.
 """
 from __future__ import annotations
 
+from typing import Optional
+
 import torch
 
 from ..kernel import kv_cache_append, kv_cache_fill
@@ -23,20 +25,31 @@ class KVCache:
         self.lens = torch.zeros(batch_size, dtype=torch.int32, device=device)
         self.batch_size = batch_size
         self.max_seq_len = max_seq_len
+        self._longest = 0       # host-side bound of the longest cached sequence (no device read per step)
         # lengths are advanced in place, so the kernels are handed this fixed view instead of
         # going through the per-tensor offset cache
         self.info = SeqInfo(self.lens, None, batch_size, None, self.lens)
 
     def fill(self, k_src: torch.Tensor, v_src: torch.Tensor, info: SeqInfo, k_head_first: int = 0,
-             v_head_first: int = 0) -> None:
-        """Prefill from packed projections seen as ``[T,Hs,D]`` (see ``kv_cache_fill``)."""
+             v_head_first: int = 0, longest: Optional[int] = None) -> None:
+        """Prefill from packed projections seen as ``[T,Hs,D]`` (see ``kv_cache_fill``).  ``longest`` is the
+        longest sequence length if the caller knows it on the host (the bucket length is an upper bound)."""
         # the buffers were zeroed when they were allocated and no reader goes past the lengths
         kv_cache_fill(k_src, self.k, self.batch_size, info, k_head_first, zero_padding=False)
         kv_cache_fill(v_src, self.v, self.batch_size, info, v_head_first, zero_padding=False)
         self.lens.copy_(info.lens)
+        # the fill kernel is given at most max_seq_len rows per sequence; the bound is tightened when the
+        # caller has the true maximum on the host
+        self._longest = self.max_seq_len if longest is None else min(int(longest), self.max_seq_len)
 
     def append(self, k_new: torch.Tensor, v_new: torch.Tensor) -> None:
-        """One new ``[B,H,D]`` row per sequence; lengths advance by one."""
+        """One new ``[B,H,D]`` row per sequence; lengths advance by one.  Raises when a sequence may already
+        fill the cache: the kernel would drop its new row and decoding would go on without the newest token
+        (the reference's torch.cat cache grows instead, energonai/model/attention.py:66-71)."""
+        if self._longest >= self.max_seq_len:
+            raise RuntimeError(f"KVCache.append: the cache holds max_seq_len = {self.max_seq_len} positions and a "
+                               f"sequence may already be that long; allocate the cache for prompt + generated tokens")
+        self._longest += 1
         kv_cache_append(k_new, v_new, self.k, self.v, self.info)
         self.lens.add_(1)
 

@@ -22,7 +22,7 @@ _CACHE_SIZE = 16
 class SeqInfo:
     """Device-resident int32 lengths and exclusive prefix for one batch."""
 
-    __slots__ = ("lens", "cu_seqlens", "batch_size", "_total", "_source", "_row_offsets")
+    __slots__ = ("lens", "cu_seqlens", "batch_size", "_total", "_source", "_row_offsets", "_ready", "_ordered")
 
     def __init__(self, lens: torch.Tensor, cu_seqlens: torch.Tensor, batch_size: int, total: Optional[int], source):
         self.lens = lens                # int32 [B] on the device
@@ -31,6 +31,31 @@ class SeqInfo:
         self._total = total
         self._source = source           # keeps the caller's tensor alive while cached
         self._row_offsets = {}          # (max_seq_len, left_padded) -> int32 [T]
+        self._ready = []                # events recorded behind the kernels that produced the arrays above
+        self._ordered = set()           # raw streams already ordered behind every event of _ready
+
+    def produced_on_current_stream(self) -> None:
+        """Call right after launching a kernel that writes one of this object's arrays: remembers the point
+        in the launching stream where they are complete."""
+        if not self.lens.is_cuda:
+            return
+        ev = torch.cuda.Event()
+        ev.record(torch.cuda.current_stream(self.lens.device))
+        self._ready.append(ev)
+        self._ordered = {_lib.stream_of(self.lens)}
+
+    def order_current_stream(self) -> None:
+        """Makes torch's current stream wait for the kernels that produced the offsets when they were launched
+        on another stream (the arrays are cached and reused by later calls, whichever stream those run on)."""
+        if not self._ready:
+            return
+        raw = _lib.stream_of(self.lens)
+        if raw in self._ordered:
+            return
+        cur = torch.cuda.current_stream(self.lens.device)
+        for ev in self._ready:
+            cur.wait_event(ev)
+        self._ordered.add(raw)
 
     @property
     def device(self) -> torch.device:
@@ -52,11 +77,13 @@ class SeqInfo:
         112-131, made aware of left padding)."""
         key = (int(max_seq_len), bool(left_padded))
         off = self._row_offsets.get(key)
+        self.order_current_stream()
         if off is None:
             off = torch.empty(max(self.total, 1), dtype=torch.int32, device=self.lens.device)
             with _lib.device_guard(self.lens):
                 _lib.check(_lib.fn.en_padding_offsets(self.lens.data_ptr(), self.batch_size, key[0], int(key[1]),
                                                       off.data_ptr(), _lib.stream_of(self.lens)), "padding_offsets")
+                self.produced_on_current_stream()
             self._row_offsets[key] = off
         return off
 
@@ -87,7 +114,9 @@ def build_seq_info(seq_lens, batch_size: int, device=None, total: Optional[int] 
         lens32 = torch.empty(batch_size, dtype=torch.int32, device=seq_lens.device)
         _lib.check(lib.en_prefix_sum(seq_lens.data_ptr(), int(seq_lens.dtype == torch.int64), batch_size,
                                      cu.data_ptr(), lens32.data_ptr(), _lib.stream_of(seq_lens)), "prefix_sum")
-    return SeqInfo(lens32, cu, batch_size, total, source)
+        info = SeqInfo(lens32, cu, batch_size, total, source)
+        info.produced_on_current_stream()
+    return info
 
 
 def seq_info(seq_lens, batch_size: int, device=None) -> SeqInfo:
@@ -96,18 +125,25 @@ def seq_info(seq_lens, batch_size: int, device=None) -> SeqInfo:
     A SeqInfo passes through unchanged.  Tensors are cached by identity and
     version counter, and the cache holds a reference to the tensor so its
     storage cannot be recycled under a stale entry; in-place edits through torch
-    bump the version and miss the cache.
+    bump the version and miss the cache.  Tensors created inside
+    ``torch.inference_mode()`` (the reference worker runs the whole forward there,
+    energonai/worker.py:79) carry no version counter, so an edit could not be
+    noticed: they are never cached and the prefix kernel runs on every call.
+    A cached entry used on another stream than the one its kernels were launched
+    on makes that stream wait for them first.
     """
     if isinstance(seq_lens, SeqInfo):
         if seq_lens.batch_size != batch_size:
             raise RuntimeError(f"SeqInfo was built for batch {seq_lens.batch_size}, call passes {batch_size}")
+        seq_lens.order_current_stream()
         return seq_lens
-    if not isinstance(seq_lens, torch.Tensor):
+    if not isinstance(seq_lens, torch.Tensor) or torch.is_inference(seq_lens):
         return build_seq_info(seq_lens, batch_size, device)
     key = (id(seq_lens), seq_lens._version, seq_lens.data_ptr(), batch_size, str(device))
     hit = _cache.get(key)
     if hit is not None and hit._source is seq_lens:
         _cache.move_to_end(key)
+        hit.order_current_stream()
         return hit
     info = build_seq_info(seq_lens, batch_size, device)
     _cache[key] = info

@@ -35,6 +35,10 @@ enum en_status {
 
 /* Library version (major*10000 + minor*100 + patch). */
 int en_version(void);
+/* Digest of the source files this library was compiled from (set by the build; "unknown" otherwise).  The
+ * Python binding compares it with the sources beside it and refuses a library that is older than they are.
+ * No counterpart in the reference, whose extensions are rebuilt by setup.py. */
+const char *en_source_hash(void);
 /* Static description of an en_status value. */
 const char *en_status_string(int status);
 /* hipError_t (as int) recorded by the last EN_ERR_HIP on this thread, and its text. */
@@ -173,7 +177,7 @@ int en_layernorm_fwd(void *out, float *mean, float *invvar, void *sum_out, const
  * scores is contiguous [B,H,Sq,Sk].  Only entries softmax will read are
  * written: rows i < q_lens[b], columns j < visible(i) rounded up to 16 bytes;
  * everything else in scores is left untouched.  q_lens NULL as above.
- * fp32 accumulation on MFMA; D a multiple of 8 (16-bit) / 4 (fp32), D <= 256. */
+ * fp32 accumulation on MFMA; D a multiple of 8 (16-bit) / 4 (fp32), D <= 128. */
 int en_attn_qk(const void *q, const void *k, void *scores, const int32_t *k_lens, const int32_t *q_lens, int batch,
                int head_num, int q_seq_len, int k_seq_len, int size_per_head, int64_t q_stride_b,
                int64_t q_stride_h, int64_t q_stride_s, int64_t k_stride_b, int64_t k_stride_h, int64_t k_stride_s,

@@ -38,6 +38,9 @@ int en_linear_algo_count(int64_t rows, int64_t din, int64_t dout, int has_bias, 
 
 const char *en_linear_status_string(int status);
 
+/* Digest of the source files this library was compiled from (set by the build); see en_source_hash. */
+const char *en_linear_source_hash(void);
+
 #ifdef __cplusplus
 }
 #endif

@@ -53,7 +53,8 @@ def test_linear_library_exports_every_declared_symbol():
     for name, (_, argtypes) in _lib.LINEAR_SIGNATURES.items():
         assert hasattr(lib, name)
         m = re.search(r"\b%s\s*\((.*?)\)\s*;" % re.escape(name), text, flags=re.S)
-        assert len(argtypes) == len(m.group(1).split(",")), name
+        args = m.group(1).strip()
+        assert len(argtypes) == (0 if args in ("", "void") else len(args.split(","))), name
     assert lib.en_linear_status_string(0) == b"ok"
     # argument errors are found before any hipBLASLt or GPU call
     assert lib.en_linear(None, None, None, None, 1, 1, 1, 0, 1, -1, None, 0, None) == -1
@@ -160,6 +161,23 @@ def test_missing_library_fails_loudly(tmp_path, monkeypatch):
     monkeypatch.setattr(_lib, "LIB_PATH", str(tmp_path / "libenergon_hip.so"))
     with pytest.raises(RuntimeError, match="requires cuda extensions"):
         _lib.load()
+
+
+def test_library_built_from_other_sources_is_refused(monkeypatch):
+    """The libraries carry a digest of their sources; one that differs from the sources in the tree (an edited
+    kernel without a rebuild) is refused at load instead of being tested in place of the code beside it."""
+    from energonai_amd import _lib, build
+    lib = _lib.load()
+    assert lib.en_source_hash().decode() == build.source_hash()
+    assert _lib.load_linear().en_linear_source_hash().decode() == build.linear_source_hash()
+    monkeypatch.setattr(_lib, "_lib", None)
+    monkeypatch.setattr(build, "source_hash", lambda: "0" * 32)
+    with pytest.raises(RuntimeError, match="built from other sources"):
+        _lib.load()
+    monkeypatch.setattr(_lib, "_linear_lib", None)
+    monkeypatch.setattr(build, "linear_source_hash", lambda: "0" * 32)
+    with pytest.raises(RuntimeError, match="built from other sources"):
+        _lib.load_linear()
 
 
 def test_product_never_imports_the_oracle():

@@ -379,3 +379,36 @@ def test_attention_long_bucket(causal):
         assert max_abs(ctx_b[b, :, :n], ref) <= 2e-3
         assert max_abs(ctx_c[t0:t0 + n].permute(1, 0, 2), ref) <= 2e-3
         t0 += n
+
+
+@pytest.mark.parametrize("tail_rows", [1, 128])
+@pytest.mark.parametrize("dtype,S", [(torch.float32, 4104), (torch.float16, 8200)])
+def test_attention_rows_past_the_register_limit(dtype, S, tail_rows):
+    """Score rows too long for the register softmax (the three-pass kernel runs) whose length is a multiple of
+    the 16-byte vector: QK^T stores whole vectors and PV loads whole vectors, so the softmax must clear the
+    vector that straddles the end of a row's prefix.  Causal, one full-length and one short sequence, score
+    buffer pre-filled with a large value that would wreck the context if it leaked."""
+    k = _kernel()
+    B, H, D = 2, 1, 64
+    lens = [S, 1029]
+    announce("attn past register limit", dtype, S, tail_rows)
+    T = sum(lens)
+    qkv_packed = packed_randn(T, H * 3 * D, dtype, 77 + S).reshape(T, H, 3 * D)
+    qkv = pad_bhsd(qkv_packed, lens, S, H, 3 * D)
+    q, kk, v = torch.chunk(qkv, 3, dim=-1)
+    scale = D ** -0.5
+    lens_t = torch.tensor(lens, dtype=torch.int32).cuda()
+    qg, kg, vg = torch.chunk(qkv.cuda(), 3, dim=-1)
+    out = torch.full((B, H, S, S), 1000.0, dtype=dtype, device="cuda")
+    s_gpu = k.attn_qk(qg, kg, lens_t, causal=True, out=out)
+    p_gpu = k.scale_mask_softmax(B, S, H, s_gpu, lens_t, scale=scale, causal=True, tail_rows=tail_rows)
+    ctx = k.attn_pv(p_gpu, vg, lens_t, causal=True).cpu()
+    del out, s_gpu, p_gpu
+    tol = {torch.float16: 2e-3, torch.float32: 1e-5}[dtype]
+    for b, n in enumerate(lens):
+        # the oracle one sequence at a time keeps the float32 score tensor of the CPU side small
+        sc = eager.attn_qk(q[b:b + 1, :, :n], kk[b:b + 1, :, :n], torch.float32)
+        pr = eager.scale_mask_softmax(1, n, H, sc, [n], scale=scale, causal=True, acc_dtype=torch.float32,
+                                      out_dtype=torch.float32)
+        want = eager.attn_pv(pr, v[b:b + 1, :, :n], torch.float32)
+        assert max_abs(ctx[b:b + 1, :, :n], want) <= tol * max(1.0, float(want.abs().max()))

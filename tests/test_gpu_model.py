@@ -76,7 +76,7 @@ def test_kv_cache_fill_and_append_bit_exact(dtype):
     cache = M.KVCache(B, H, Smax, D, dtype, "cuda")
     from energonai_amd.seqinfo import seq_info
     info = seq_info(info_lens, B, torch.device("cuda"))
-    cache.fill(kvq.cuda(), kvq.cuda(), info, 0, H)
+    cache.fill(kvq.cuda(), kvq.cuda(), info, 0, H, longest=max(lens))
     want_k = torch.zeros(B, H, Smax, D, dtype=dtype)
     want_v = torch.zeros_like(want_k)
     start = 0
@@ -95,6 +95,15 @@ def test_kv_cache_fill_and_append_bit_exact(dtype):
             want_v[b, :, n + step] = new[b, H:2 * H]
         assert torch.equal(cache.k.cpu(), want_k) and torch.equal(cache.v.cpu(), want_v)
         assert cache.lens.cpu().tolist() == [n + step + 1 for n in lens]
+    # a cache that may be full refuses the next row instead of dropping it silently
+    small = M.KVCache(B, H, max(lens) + 2, D, dtype, "cuda")
+    small.fill(kvq.cuda(), kvq.cuda(), info, 0, H, longest=max(lens))
+    new_g = torch.randn(B, 3 * H, D, generator=g).to(dtype).cuda()
+    small.append(new_g[:, :H], new_g[:, H:2 * H])
+    small.append(new_g[:, :H], new_g[:, H:2 * H])
+    with pytest.raises(RuntimeError, match="max_seq_len"):
+        small.append(new_g[:, :H], new_g[:, H:2 * H])
+    assert small.lens.cpu().tolist() == [n + 2 for n in lens]
 
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.float32])

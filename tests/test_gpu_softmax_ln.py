@@ -201,24 +201,31 @@ def test_layernorm_module_matches_reference_interface():
 @pytest.mark.parametrize("tile", [128, 32, 1])
 @pytest.mark.parametrize("dtype", [torch.float16, torch.float32])
 @pytest.mark.parametrize("causal", [True, False])
-def test_softmax_tiled_tail(dtype, causal, tile):
+@pytest.mark.parametrize("scale", [0.5, -0.5])
+def test_softmax_tiled_tail(dtype, causal, tile, scale):
     """tail_rows=t: valid entries identical to the full-tail result, zeros up to the extent of the row's
-    t-row query tile, everything beyond left untouched.  t = 1 (the form in the step) writes no tail at all."""
+    t-row query tile (completed to a whole 16-byte vector), everything beyond left untouched.  t = 1 (the form
+    in the step) writes no tail beyond that vector.  A negative scale takes the three-pass kernel, which must
+    leave the same bytes."""
     k = _kernel()
     B, H, S = 3, 2, 512
     lens = [512, 130, 300]
-    announce("softmax tiled tail", dtype, causal, tile)
+    announce("softmax tiled tail", dtype, causal, tile, scale)
     g = torch.Generator().manual_seed(21)
     src = (3.0 * torch.randn(B, H, S, S, generator=g)).to(dtype)
     lens_t = torch.tensor(lens, dtype=torch.int32).cuda()
     epv = 16 // src.element_size()
-    full = k.scale_mask_softmax(B, S, H, src.clone().cuda(), lens_t, scale=0.5, causal=causal).cpu()
-    tiled = k.scale_mask_softmax(B, S, H, src.clone().cuda(), lens_t, scale=0.5, causal=causal, tail_rows=tile).cpu()
+    full = k.scale_mask_softmax(B, S, H, src.clone().cuda(), lens_t, scale=scale, causal=causal).cpu()
+    tiled = k.scale_mask_softmax(B, S, H, src.clone().cuda(), lens_t, scale=scale, causal=causal, tail_rows=tile).cpu()
+    want = eager.scale_mask_softmax(B, S, H, src.float(), lens, scale=scale, causal=causal, out_dtype=torch.float32)
+    valid = _valid_row_mask(B, H, S, S, lens)
+    assert max_abs(full[valid].float(), want[valid]) <= TOL[dtype]
     for b, n in enumerate(lens):
         for q0 in range(0, n, tile):
             rows = min(tile, n - q0)
             lim = min(n, q0 + rows) if causal else n
             lim_v = -(-lim // epv) * epv   # whole vectors are written
             assert torch.equal(tiled[b, :, q0:q0 + rows, :lim], full[b, :, q0:q0 + rows, :lim])
+            assert bool((tiled[b, :, q0:q0 + rows, lim:lim_v] == 0).all())
             assert torch.equal(tiled[b, :, q0:q0 + rows, lim_v:], src[b, :, q0:q0 + rows, lim_v:])
         assert torch.equal(tiled[b, :, n:], src[b, :, n:])
