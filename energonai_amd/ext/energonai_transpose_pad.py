@@ -1,6 +1,9 @@
 """Same symbol table as the reference's ``energonai_transpose_pad`` extension
 (csrc/transpose_pad_fusion_wrapper.cpp:246-263)."""
-from ..kernel.cuda_native import transpose_pad as _k
+import importlib
+
+# the package re-exports a function of the same name, which hides the module from a plain "from ... import"
+_k = importlib.import_module("energonai_amd.kernel.cuda_native.transpose_pad")
 
 
 def transpose_pad_wrapper(src, batch_size, max_seq_len, seq_len_list, head_num, size_per_head):
