@@ -87,6 +87,7 @@ const char *en_status_string(int status) {
     case EN_ERR_ALIGN: return "pointer or stride not aligned to the element size";
     case EN_ERR_UNSUPPORTED: return "no kernel in this build for the requested shape";
     case EN_ERR_HIP: return "HIP runtime error (see en_last_hip_error_string)";
+    case EN_ERR_SCRATCH: return "the call needs more than the library's static scratch array holds (EN_LAYER_SCRATCH_BYTES)";
     default: return "unknown status";
   }
 }

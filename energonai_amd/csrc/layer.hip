@@ -7,6 +7,52 @@
 // launch of transpose_pad: six launches.
 #include "common.hip.h"
 
+#include <mutex>
+
+namespace en {
+
+// Scratch of en_padding_removal_layer_noalloc: every intermediate that en_padding_removal_layer takes from its
+// caller lives here instead.  One copy per GPU the library runs on, held until the process ends.
+constexpr int64_t kLayerScratchBytes = EN_LAYER_SCRATCH_BYTES;
+static __device__ __align__(256) unsigned char scratch[kLayerScratchBytes];
+
+// In host code `scratch` is only a handle for hipGetSymbolAddress; the array's device address differs per GPU
+// and is looked up once per device, with that device current.
+constexpr int kMaxDevices = 64;
+static unsigned char *g_scratch_ptr[kMaxDevices];
+static std::mutex g_scratch_mutex;
+
+static int scratch_for_current_device(unsigned char **out) {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return record_hip_error(e);
+  if (dev < 0 || dev >= kMaxDevices) return EN_ERR_UNSUPPORTED;
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (!g_scratch_ptr[dev]) {
+    void *p = nullptr;
+    e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (e != hipSuccess) return record_hip_error(e);
+    if (!p) return EN_ERR_UNSUPPORTED;
+    g_scratch_ptr[dev] = static_cast<unsigned char *>(p);
+  }
+  *out = g_scratch_ptr[dev];
+  return EN_OK;
+}
+
+// Lays out 256-byte aligned pieces of the scratch array: take() returns a piece's offset, or -1 for a piece the
+// call does not need; `used` may run past the end (checked by the caller before anything is launched).
+struct Layout {
+  int64_t used = 0;
+  int64_t take(bool wanted, int64_t bytes) {
+    if (!wanted) return -1;
+    const int64_t at = used;
+    used += (bytes + 255) / 256 * 256;
+    return at;
+  }
+};
+
+}  // namespace en
+
 extern "C" int en_padding_removal_layer(const void *hidden_padded, const void *qkv_packed, const void *dense_out,
                                         const void *gamma, const void *beta, void *x_packed, void *qkv_padded,
                                         void *scores, void *ctx, void *ctx_packed, void *y,
@@ -80,4 +126,48 @@ extern "C" int en_padding_removal_layer(const void *hidden_padded, const void *q
   return en_layernorm_fwd(y, nullptr, nullptr, nullptr, dense_out ? dense_out : ctx_packed,
                           fold_depad_offsets ? hidden_padded : x_packed, fold_depad_offsets, gamma, beta, total_tokens,
                           hidden, eps, dtype, dtype, stream);
+}
+
+extern "C" int en_padding_removal_layer_noalloc(const void *hidden_padded, const void *qkv_packed, const void *dense_out,
+                                                const void *gamma, const void *beta, void *y, const void *seq_lens,
+                                                int lens_are_i64, int batch, int max_seq_len, int head_num,
+                                                int size_per_head, int64_t hidden, int64_t total_tokens, float scale,
+                                                float eps, int causal, int left_padded, int attention_form,
+                                                int fold_depad, int dtype, en_stream_t stream) {
+  using namespace en;
+  if (!hidden_padded || !qkv_packed || !gamma || !beta || !y || !seq_lens) return EN_ERR_NULL;
+  if (attention_form < 0 || attention_form > 2) return EN_ERR_UNSUPPORTED;
+  const int64_t es = dtype_size(dtype);
+  if (!es) return EN_ERR_DTYPE;
+  if (batch < 1 || batch > 65536 || max_seq_len < 1 || head_num < 1 || size_per_head < 1 || hidden < 1 ||
+      total_tokens < 0 || total_tokens > (int64_t)batch * max_seq_len)
+    return EN_ERR_SHAPE;
+  if (total_tokens == 0) return EN_OK;
+  const int64_t B = batch, S = max_seq_len, H = head_num, D = size_per_head, T = total_tokens;
+  // the same pieces, in the same roles, as the caller-owned buffers of en_padding_removal_layer
+  Layout l;
+  const bool padded = attention_form != 2;
+  const int64_t o_cu = l.take(true, (B + 1) * 4), o_lens = l.take(true, B * 4);
+  const int64_t o_offs = l.take(fold_depad != 0, T * 4), o_x = l.take(fold_depad == 0, T * hidden * es);
+  const int64_t o_qkv = l.take(padded, B * H * S * 3 * D * es), o_scores = l.take(attention_form == 0, B * H * S * S * es);
+  const int64_t o_ctx = l.take(padded, B * H * S * D * es), o_ctxp = l.take(true, T * H * D * es);
+  if (l.used > kLayerScratchBytes) return EN_ERR_SCRATCH;
+  unsigned char *base = nullptr;   // the array's address on the current device; never the array's name
+  int rc = scratch_for_current_device(&base);
+  if (rc) return rc;
+  auto at = [&](int64_t off) -> void * { return off < 0 ? nullptr : base + off; };
+  int32_t *cu = static_cast<int32_t *>(at(o_cu)), *lens32 = static_cast<int32_t *>(at(o_lens));
+  int32_t *offs = static_cast<int32_t *>(at(o_offs));
+  rc = en_prefix_sum(seq_lens, lens_are_i64, batch, cu, lens32, stream);
+  if (rc) return rc;
+  if (fold_depad) {
+    rc = en_padding_offsets(lens32, batch, max_seq_len, left_padded, offs, stream);
+    if (rc) return rc;
+  }
+  // Nothing here has to start at zero: every kernel of the step writes what the next one reads, and reads are
+  // bounded by the sequence lengths, so what an earlier (larger) call left in the array is never looked at.
+  return en_padding_removal_layer(hidden_padded, qkv_packed, dense_out, gamma, beta, at(o_x), at(o_qkv), at(o_scores),
+                                  at(o_ctx), at(o_ctxp), y, cu, lens32, batch, max_seq_len, head_num,
+                                  size_per_head, hidden, total_tokens, scale, eps, causal, left_padded, attention_form,
+                                  offs, dtype, stream);
 }

@@ -118,6 +118,51 @@ def _layer_one_call(hidden_padded, qkv_packed, info, B, S, H, D, hid, T, gamma, 
     return y
 
 
+def padding_removal_layer_noalloc(hidden_padded: torch.Tensor, qkv_packed: torch.Tensor, seq_lens: torch.Tensor,
+                                  head_num: int, size_per_head: int, gamma: torch.Tensor, beta: torch.Tensor,
+                                  out: torch.Tensor, sum_seq: int, eps: float = 1e-5, scale: Optional[float] = None,
+                                  causal: bool = True, left_padded: bool = False,
+                                  dense_out: Optional[torch.Tensor] = None, fused_attention=False,
+                                  fold_depad: bool = False) -> torch.Tensor:
+    """The same step for callers that may not allocate device memory (a step recorded into a HIP graph, a tight
+    serving loop): ``en_padding_removal_layer_noalloc`` keeps every intermediate, the sequence offsets included,
+    in a static array inside the library (64 MiB per GPU; larger steps raise).  Nothing is allocated here
+    either: ``seq_lens`` must already be a contiguous int32/int64 tensor on the device, ``sum_seq`` its total
+    and ``out`` the ``[1,T,hid]`` result tensor.  Calls that overlap on one GPU share the array and race.
+    """
+    B, S, hid = hidden_padded.shape
+    H, D = head_num, size_per_head
+    T = int(sum_seq)
+    dt = hidden_padded.dtype
+    for t, name in ((hidden_padded, "hidden_padded"), (qkv_packed, "qkv_packed"), (seq_lens, "seq_lens"), (out, "out"),
+                    (gamma, "gamma"), (beta, "beta")):
+        _lib.require_gpu(t, name)
+    if seq_lens.dtype not in (torch.int32, torch.int64) or seq_lens.numel() < B:
+        raise RuntimeError("padding_removal_layer_noalloc: seq_lens must hold batch int32 or int64 lengths")
+    if qkv_packed.numel() != T * H * 3 * D or qkv_packed.dtype != dt:
+        raise RuntimeError("padding_removal_layer_noalloc: qkv_packed must be [1,T,H,3D] of the activation dtype")
+    if out.numel() != T * hid or out.dtype != dt:
+        raise RuntimeError("padding_removal_layer_noalloc: out must be [1,T,hidden] of the activation dtype")
+    if gamma.dtype != dt or beta.dtype != dt or gamma.numel() != hid or beta.numel() != hid:
+        raise RuntimeError("padding_removal_layer_noalloc: gamma and beta must be [hidden] of the activation dtype")
+    if dense_out is not None:
+        _lib.require_gpu(dense_out, "dense_out")
+        if dense_out.numel() != T * hid or dense_out.dtype != dt:
+            raise RuntimeError("padding_removal_layer_noalloc: dense_out must be [1,T,hidden] of the activation dtype")
+    elif hid != H * D:
+        raise RuntimeError("padding_removal_layer_noalloc: without dense_out the LayerNorm width must equal "
+                           "heads * size_per_head")
+    scale = float(D) ** -0.5 if scale is None else scale
+    with _lib.device_guard(hidden_padded):
+        _lib.check(_lib.fn.en_padding_removal_layer_noalloc(
+            hidden_padded.data_ptr(), qkv_packed.data_ptr(), _lib.ptr(dense_out), gamma.data_ptr(), beta.data_ptr(),
+            out.data_ptr(), seq_lens.data_ptr(), int(seq_lens.dtype == torch.int64), B, S, H, D, hid, T, float(scale),
+            float(eps), int(bool(causal)), int(bool(left_padded)), _FORMS[fused_attention], int(bool(fold_depad)),
+            _lib.dtype_tag(hidden_padded, "padding_removal_layer_noalloc"), _lib.stream_of(hidden_padded)),
+            "padding_removal_layer_noalloc")
+    return out
+
+
 def decode_layer(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, kv_lens, residual: torch.Tensor,
                  gamma: torch.Tensor, beta: torch.Tensor, eps: float = 1e-5, scale: Optional[float] = None,
                  dense_out: Optional[torch.Tensor] = None, keep: bool = False):

@@ -30,7 +30,8 @@ enum en_status {
   EN_ERR_DTYPE = -3,       /* dtype tag or element size not supported by this entry point */
   EN_ERR_ALIGN = -4,       /* pointer or stride not aligned to the element size */
   EN_ERR_UNSUPPORTED = -5, /* valid request this build has no kernel for (message names it) */
-  EN_ERR_HIP = -6          /* the HIP runtime reported an error; see en_last_hip_error() */
+  EN_ERR_HIP = -6,         /* the HIP runtime reported an error; see en_last_hip_error() */
+  EN_ERR_SCRATCH = -7      /* the call needs more than EN_LAYER_SCRATCH_BYTES of the library's static scratch */
 };
 
 /* Library version (major*10000 + minor*100 + patch). */
@@ -261,6 +262,31 @@ int en_padding_removal_layer(const void *hidden_padded, const void *qkv_packed, 
                              int64_t hidden, int64_t total_tokens, float scale, float eps, int causal,
                              int left_padded, int attention_form, const int32_t *fold_depad_offsets, int dtype,
                              en_stream_t stream);
+
+/* en_padding_removal_layer for callers that cannot allocate device memory: code under HIP graph capture,
+ * tight serving loops, harnesses that forbid hipMalloc.  It has no counterpart in the reference.  Every
+ * buffer en_padding_removal_layer takes from its caller besides the inputs and y -- cu_seqlens and the int32
+ * lengths (computed here from seq_lens: int32, or int64 when lens_are_i64 != 0), the fold_depad offsets,
+ * x_packed, qkv_padded, scores, ctx, ctx_packed -- lives in one static device array of
+ * EN_LAYER_SCRATCH_BYTES inside the library, one copy per GPU, held until the process ends.  The pieces a
+ * call needs (each rounded up to 256 bytes; e = element size, T = total_tokens):
+ *   always                 (B+1)*4 + B*4 + T*H*D*e
+ *   fold_depad != 0        + T*4                     else  + T*hidden*e
+ *   attention_form 0 or 1  + B*H*S*3D*e + B*H*S*D*e
+ *   attention_form 0       + B*H*S*S*e
+ * A call that needs more returns EN_ERR_SCRATCH before anything is launched.  Arguments otherwise as
+ * en_padding_removal_layer (fold_depad != 0 stands for passing fold_depad_offsets).  No hipMalloc, hipFree
+ * or other allocating call is made; the first call on a device looks up the array's address
+ * (hipGetSymbolAddress), so make that call outside a stream capture.  Every call on a GPU uses that GPU's one
+ * array: calls that overlap on the same GPU (two streams, two threads) race; calls on one stream do not.
+ * Nothing in the array has to be cleared between calls. */
+#define EN_LAYER_SCRATCH_BYTES (64ll << 20)
+int en_padding_removal_layer_noalloc(const void *hidden_padded, const void *qkv_packed, const void *dense_out,
+                                     const void *gamma, const void *beta, void *y, const void *seq_lens,
+                                     int lens_are_i64, int batch, int max_seq_len, int head_num, int size_per_head,
+                                     int64_t hidden, int64_t total_tokens, float scale, float eps, int causal,
+                                     int left_padded, int attention_form, int fold_depad, int dtype,
+                                     en_stream_t stream);
 
 /* Plain device-to-device copy of nbytes (multiple of 16, 16-byte aligned) with
  * the same 128-bit access pattern the packing kernels use.  Used as the
