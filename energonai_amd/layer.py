@@ -30,7 +30,8 @@ def padding_removal_layer(hidden_padded: torch.Tensor, qkv_packed: torch.Tensor,
                           size_per_head: int, gamma: torch.Tensor, beta: torch.Tensor, eps: float = 1e-5,
                           scale: Optional[float] = None, causal: bool = True, left_padded: bool = False,
                           dense_out: Optional[torch.Tensor] = None, sum_seq: Optional[int] = None,
-                          keep: bool = False, fused_attention=False, fold_depad: bool = False):
+                          keep: bool = False, fused_attention=False, fold_depad: bool = False,
+                          ctx_out: Optional[torch.Tensor] = None):
     """Runs the seven ops on ``hidden_padded`` [B,S,hid] and ``qkv_packed`` [1,T,H,3D].
 
     Returns the normalised ``[1,T,hid]`` output, or a dict of every
@@ -41,6 +42,8 @@ def padding_removal_layer(hidden_padded: torch.Tensor, qkv_packed: torch.Tensor,
     the fused kernel reads the packed projections and writes the packed context.
     ``fold_depad=True`` drops the depad launch as well: the LayerNorm takes its
     residual rows straight from ``hidden_padded`` (not with ``keep``).
+    ``ctx_out`` (``[1,T,H,D]``, not with ``keep``) receives the packed attention
+    context, which is otherwise a temporary of the call.
     """
     B, S, hid = hidden_padded.shape
     H, D = head_num, size_per_head
@@ -49,7 +52,7 @@ def padding_removal_layer(hidden_padded: torch.Tensor, qkv_packed: torch.Tensor,
     scale = float(D) ** -0.5 if scale is None else scale
     if not keep:
         return _layer_one_call(hidden_padded, qkv_packed, info, B, S, H, D, hid, T, gamma, beta, eps, scale, causal,
-                               left_padded, dense_out, fused_attention, fold_depad)
+                               left_padded, dense_out, fused_attention, fold_depad, ctx_out)
     if fold_depad:
         raise RuntimeError("padding_removal_layer: fold_depad has no intermediates to keep")
 
@@ -82,7 +85,7 @@ _FORMS = {False: 0, True: 1, "packed": 2}
 
 
 def _layer_one_call(hidden_padded, qkv_packed, info, B, S, H, D, hid, T, gamma, beta, eps, scale, causal, left_padded,
-                    dense_out, fused_attention, fold_depad=False):
+                    dense_out, fused_attention, fold_depad=False, ctx_out=None):
     """The same seven ops through ``en_padding_removal_layer``: one foreign call per step."""
     dev, dt = hidden_padded.device, hidden_padded.dtype
     form = _FORMS[fused_attention]
@@ -103,7 +106,13 @@ def _layer_one_call(hidden_padded, qkv_packed, info, B, S, H, D, hid, T, gamma, 
     x = None if fold_depad else torch.empty((1, T, hid), dtype=dt, device=dev)
     offs = info.row_offsets(S, left_padded) if fold_depad else None
     y = torch.empty((1, T, hid), dtype=dt, device=dev)
-    ctx_packed = torch.empty((1, T, H, D), dtype=dt, device=dev)
+    if ctx_out is None:
+        ctx_packed = torch.empty((1, T, H, D), dtype=dt, device=dev)
+    else:
+        _lib.require_gpu(ctx_out, "ctx_out")
+        if ctx_out.numel() != T * H * D or ctx_out.dtype != dt:
+            raise RuntimeError("padding_removal_layer: ctx_out must be [1,T,H,D] of the activation dtype")
+        ctx_packed = ctx_out
     qkv = torch.empty((B, H, S, 3 * D), dtype=dt, device=dev) if form != 2 else None
     ctx = torch.empty((B, H, S, D), dtype=dt, device=dev) if form != 2 else None
     scores = torch.empty((B, H, S, S), dtype=dt, device=dev) if form == 0 else None

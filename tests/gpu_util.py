@@ -33,3 +33,35 @@ def pad_bhsd(packed, lens, S, H, D):
 
 def max_abs(a, b):
     return (a.double() - b.double()).abs().max().item()
+
+
+# ---------------------------------------------------------------------------------------------------------------
+# Tolerances, in one place.  The bar is: max-abs error <= BASE[dtype] against the float32 (or float64) oracle, on
+# top of the rounding the result's own storage type forces on it (half a unit in the last place of the stored
+# value: 9.8e-4 for an fp16 value in [2, 4), 1.95e-3 in [4, 8), which no kernel can avoid).  BASE is 2e-3 for
+# fp16 and 1e-5 for fp32; bf16 carries 8 fewer mantissa bits than fp16, hence 8 x 2e-3.
+# ---------------------------------------------------------------------------------------------------------------
+BASE = {torch.float32: 1e-5, torch.float16: 2e-3, torch.bfloat16: 1.6e-2}
+_MANT = {torch.float32: 23, torch.float16: 10, torch.bfloat16: 7}
+_MIN_EXP = {torch.float32: -126, torch.float16: -14, torch.bfloat16: -126}
+
+
+def half_ulp(ref, dtype):
+    """Half the spacing of `dtype` at |ref|, elementwise, as float64."""
+    a = ref.double().abs()
+    e = torch.floor(torch.log2(a.clamp_min(2.0 ** _MIN_EXP[dtype]))).clamp_min(_MIN_EXP[dtype])
+    return 0.5 * torch.pow(torch.tensor(2.0, dtype=torch.float64), e - _MANT[dtype])
+
+
+def excess(got, want, dtype):
+    """max(|got - want| - half_ulp(want)): the error left after the unavoidable rounding of the stored result."""
+    if got.numel() == 0:
+        return 0.0
+    return float(((got.double() - want.double()).abs() - half_ulp(want, dtype)).max())
+
+
+def assert_stored_close(got, want, dtype, base=None, what=""):
+    """|got - want| <= base + half_ulp_dtype(|want|) elementwise; base defaults to BASE[dtype]."""
+    base = BASE[dtype] if base is None else base
+    ex = excess(got, want, dtype)
+    assert ex <= base, f"{what}: error exceeds half an ulp of the stored value by {ex:.3e} > {base:.3e}"

@@ -11,7 +11,7 @@ subset of sequences, so the CPU side stays within seconds.
 import pytest
 import torch
 
-from gpu_util import announce, max_abs
+from gpu_util import BASE, announce, assert_stored_close, max_abs
 from oracle import eager
 
 pytestmark = pytest.mark.gpu
@@ -35,8 +35,11 @@ def _run_and_compare(w, inp, acc_dtype, tol_ctx, tol_y, storage_dtype=None):
     assert torch.equal(got["qkv"].cpu(), want["qkv"].to(w.dtype)), "transpose_pad must be bit-exact"
     err_ctx = max_abs(got["ctx_packed"].cpu(), want["ctx_packed"])
     assert err_ctx <= tol_ctx, err_ctx
-    err_y = max_abs(got["y"].cpu(), want["y"])
-    assert err_y <= tol_y, err_y
+    if tol_y is None:       # 2e-3 (fp16) on top of half an ulp of the stored value
+        assert_stored_close(got["y"].cpu(), want["y"], w.dtype, what="LayerNorm output")
+    else:
+        err_y = max_abs(got["y"].cpu(), want["y"])
+        assert err_y <= tol_y, err_y
     return got, want
 
 
@@ -77,12 +80,36 @@ def test_layer_c2_fp16_full():
     inp = wl.make_inputs(w)
     assert inp["total"] == 8538
     # Against the fp32 oracle that rounds scores / probabilities / context to fp16 where the API stores
-    # them (the reference materialises the same fp16 tensors): the north-star tolerance.  LayerNorm output
-    # |y| reaches ~5, where one fp16 rounding alone is 1.95e-3, on top of the error of its input.
-    _run_and_compare(w, inp, torch.float32, 2e-3, 6e-3, storage_dtype=torch.float16)
-    # Against the oracle with no intermediate rounding at all the fp16 score tensor shows: a score of
-    # magnitude ~32 carries an absolute rounding error of 2^-6, i.e. 2e-3 relative in its probability.
-    _run_and_compare(w, inp, torch.float32, 4e-3, 8e-3)
+    # them (the reference materialises the same fp16 tensors): 2e-3 on the context; 2e-3 plus half an fp16
+    # ulp of the stored value on the LayerNorm output (|y| reaches ~5, where that rounding alone is 1.95e-3).
+    _run_and_compare(w, inp, torch.float32, 2e-3, None, storage_dtype=torch.float16)
+
+
+def test_layer_c2_unfused_path_misses_2e3_against_the_unrounded_oracle_by_the_fp16_score_rounding():
+    """Against the oracle that rounds nothing in between, the three-kernel path cannot meet 2e-3: the score
+    tensor it must materialise in fp16 (as the reference does) perturbs every score by up to half an fp16 ulp,
+    d = half_ulp(max|score|), so every probability by a factor within exp(+-2 * scale * d) and the context by
+    at most 2 * scale * d * max|v|.  The bound below is that worst case on top of the 2e-3; the fused kernel,
+    which stores no scores, meets the plain 2e-3 (test_layer_c2_fused_attention)."""
+    layer, wl = _mods()
+    from gpu_util import half_ulp
+    w = wl.BY_NAME["c2"]
+    announce("layer c2 vs unrounded oracle")
+    inp = wl.make_inputs(w)
+    got = layer.padding_removal_layer(inp["hidden_padded"].cuda(), inp["qkv_packed"].cuda(), inp["lens"].cuda(),
+                                      w.heads, w.head_dim, inp["gamma"].cuda(), inp["beta"].cuda(), 1e-5, w.scale,
+                                      w.causal, w.left_padded, keep=True)
+    want = eager.layer_unpadded(inp["hidden_padded"], inp["qkv_packed"], inp["lens_list"], w.heads, w.head_dim,
+                                inp["gamma"], inp["beta"], 1e-5, w.scale, w.causal, w.left_padded,
+                                acc_dtype=torch.float32)
+    valid = torch.zeros_like(want["scores"], dtype=torch.bool)
+    for b, n in enumerate(inp["lens_list"]):
+        valid[b, :, :n, :n] = True
+    d = float(half_ulp(want["scores"][valid].abs().max(), torch.float16))
+    v_max = float(inp["qkv_packed"][..., 2 * w.head_dim:].abs().max())
+    err = max_abs(got["ctx_packed"].cpu(), want["ctx_packed"])
+    print(f"max|ctx err| vs unrounded oracle {err:.3e}; score rounding allows {2 * w.scale * d * v_max:.3e} more than 2e-3")
+    assert err <= 2e-3 + 2 * w.scale * d * v_max
 
 
 @pytest.mark.parametrize("name,total", [("c3", 9244), ("c4", 20142)])
@@ -133,9 +160,54 @@ def test_layer_large_fp16_properties(name, total):
         sub_hidden = inp["hidden_padded"][b:b + 1]
         sub_dense = None if inp["dense_out"] is None else inp["dense_out"][:, sl]
         want = eager.layer_unpadded(sub_hidden, sub_qkv, [n], H, D, inp["gamma"], inp["beta"], 1e-5, w.scale,
-                                    w.causal, w.left_padded, dense_out=sub_dense, acc_dtype=torch.float32)
-        assert max_abs(got["ctx_packed"][0, sl].cpu(), want["ctx_packed"][0]) <= 2e-3
-        assert max_abs(got["y"][0, sl].cpu(), want["y"][0]) <= 6e-3
+                                    w.causal, w.left_padded, dense_out=sub_dense, acc_dtype=torch.float32,
+                                    storage_dtype=torch.float16)
+        assert_stored_close(got["ctx_packed"][0, sl].cpu(), want["ctx_packed"][0], w.dtype, what="context")
+        assert_stored_close(got["y"][0, sl].cpu(), want["y"][0], w.dtype, what="LayerNorm output")
+
+
+@pytest.mark.parametrize("name,total", [("c3", 9244), ("c4", 20142)])
+def test_layer_large_fp16_one_call_path_against_the_oracle(name, total):
+    """The form the benchmark times (one call into the library: padding rows of the padded tensor not written, no
+    softmax tail, depad paired with transpose_pad on small batches) at full size: context and output of the
+    longest, the median and the shortest sequence against the oracle run on that sequence alone (attention and
+    LayerNorm are independent per sequence), and bit-equality with the op-by-op sequence of public calls.
+
+    Bounds: 2e-3 on top of half an fp16 ulp of the stored value, against the float32 oracle that rounds scores
+    and probabilities to fp16 where the API stores them (the reference materialises the same fp16 tensors,
+    examples/gpt/gpt.py:108-125)."""
+    layer, wl = _mods()
+    w = wl.BY_NAME[name]
+    announce("layer one-call", name)
+    inp = wl.make_inputs(w)
+    assert inp["total"] == total
+    T, B, H, D = total, w.batch, w.heads, w.head_dim
+    lens_l = inp["lens_list"]
+    dense = None if inp["dense_out"] is None else inp["dense_out"].cuda()
+    args = (inp["hidden_padded"].cuda(), inp["qkv_packed"].cuda(), inp["lens"].cuda(), H, D, inp["gamma"].cuda(),
+            inp["beta"].cuda(), 1e-5, w.scale, w.causal, w.left_padded)
+    ctx = torch.full((1, T, H, D), float("nan"), dtype=w.dtype, device="cuda")
+    y = layer.padding_removal_layer(*args, dense_out=dense, sum_seq=T, ctx_out=ctx)
+    steps = layer.padding_removal_layer(*args, dense_out=dense, sum_seq=T, keep=True)
+    assert torch.equal(y, steps["y"]) and torch.equal(ctx, steps["ctx_packed"])
+    del steps
+    y, ctx = y.cpu(), ctx.cpu()
+    order = sorted(range(B), key=lambda b: lens_l[b])
+    cu = [0]
+    for n in lens_l:
+        cu.append(cu[-1] + n)
+    for b in (order[-1], order[B // 2], order[0]):
+        n = lens_l[b]
+        announce("  sequence", b, "length", n)
+        sl = slice(cu[b], cu[b] + n)
+        sub_dense = None if inp["dense_out"] is None else inp["dense_out"][:, sl]
+        want = eager.layer_unpadded(inp["hidden_padded"][b:b + 1], inp["qkv_packed"][:, sl], [n], H, D, inp["gamma"],
+                                    inp["beta"], 1e-5, w.scale, w.causal, w.left_padded, dense_out=sub_dense,
+                                    acc_dtype=torch.float32, storage_dtype=torch.float16)
+        assert_stored_close(ctx[0, sl].reshape(n, H * D), want["ctx_packed"].reshape(n, H * D), w.dtype, what="context")
+        # the LayerNorm passes the error of its input on, scaled by gamma * invvar, and rounds once more
+        amp = max(1.0, float(want["invvar"].max()) * float(inp["gamma"].float().abs().max())) if dense is None else 0.0
+        assert_stored_close(y[0, sl], want["y"][0], w.dtype, base=BASE[w.dtype] * max(amp, 1.0), what="LayerNorm output")
 
 
 def test_decode_layer_c5_reduced_and_full():
@@ -158,14 +230,14 @@ def test_decode_layer_c5_reduced_and_full():
         assert max_abs(got["scores_probs"][b:b + 1].cpu(), probs) <= 2e-3
     want_y, _, _, _ = eager.layer_norm(inp["dense_out"].cpu(), inp["gamma"].cpu(), inp["beta"].cpu(), 1e-5,
                                        residual=inp["residual"].cpu(), out_dtype=torch.float32)
-    assert max_abs(got["y"].cpu(), want_y) <= 6e-3
+    assert_stored_close(got["y"].cpu(), want_y, w.dtype, what="LayerNorm output")
     # the attention output feeds the residual directly when no dense output is given
     got2 = layer.decode_layer(inp["q"], inp["k_cache"], inp["v_cache"], inp["lens"].cuda(), inp["residual"],
                               inp["gamma"], inp["beta"], 1e-5, w.scale, keep=True)
     want2, _, _, _ = eager.layer_norm(got2["ctx_packed"].reshape(1, w.batch, -1).cpu(), inp["gamma"].cpu(),
                                       inp["beta"].cpu(), 1e-5, residual=inp["residual"].cpu(),
                                       out_dtype=torch.float32)
-    assert max_abs(got2["y"].cpu(), want2) <= 6e-3
+    assert_stored_close(got2["y"].cpu(), want2, w.dtype, what="LayerNorm output")
 
 
 @pytest.mark.parametrize("mode", [True, "packed"])
@@ -183,7 +255,7 @@ def test_layer_c2_fused_attention(mode):
                                 inp["gamma"], inp["beta"], 1e-5, w.scale, w.causal, w.left_padded,
                                 acc_dtype=torch.float32)
     assert max_abs(got["ctx_packed"].cpu(), want["ctx_packed"]) <= 2e-3
-    assert max_abs(got["y"].cpu(), want["y"]) <= 6e-3
+    assert_stored_close(got["y"].cpu(), want["y"], w.dtype, what="LayerNorm output")
 
 
 @pytest.mark.parametrize("name,form", [("c1", False), ("c2", False), ("c2", True), ("c2", "packed")])
