@@ -6,10 +6,12 @@
 A step is one pass of
     depad -> transpose_pad -> QK^T -> scale_mask_softmax -> PV -> transpose_depad -> residual + LayerNorm
 over one synthetic batch whose inputs are already resident in HBM.  The headline
-value is tokens/s of that pass on the workload named by --workload (default c2,
-the OPT-125M layer); the other workloads, the per-kernel bandwidths, the
-PyTorch-ROCm eager pipeline and the CPU oracle are reported beside it in the
-same JSON line.
+value is tokens/s of that pass on the workload named by --workload (default c3,
+the OPT-30B-shaped layer: the largest of the five that fits one GPU -- 1.9 GB of
+scores, 45 GFLOP per contraction -- and the one whose kernels are bound by HBM
+bandwidth rather than by launch cost); the other workloads, the per-kernel
+bandwidths, the PyTorch-ROCm eager pipeline and the CPU oracle are reported beside
+it in the same JSON line.
 
 The line also carries
   roofline      achieved vs peak for the kernel that takes the largest share of the step,
@@ -32,21 +34,31 @@ if ROOT not in sys.path:
 
 HBM_PEAK_GBS = 8000.0          # MI355X HBM3E
 MFMA_PEAK_TFLOPS = {"f16": 2500.0, "bf16": 2500.0, "f32": 157.3}
-# HBM bytes per launch on the c2 workload from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this file,
-# each scaled by what the same counter reads for en_copy_bytes of known size (x2.0 for FETCH_SIZE, x1.0
-# for WRITE_SIZE); the counter summary is kept under profiles/.  Counters cannot be read from inside the
-# benchmark, so the figures are carried here and reported with the live timing.
-MEASURED_TRAFFIC_C2 = {
-    "depad": 26.3e6,
-    "transpose_pad": 114.9e6,
-    "transpose_pad_valid_rows": 78.7e6,
-    "attn_qk": 59.5e6,
-    "scale_mask_softmax_no_tail": 71.5e6,
-    "attn_pv": 64.6e6,
-    "transpose_depad": 26.3e6,
-    "layernorm_residual": 39.4e6,
-    "attn_fused": 52.6e6,
-}
+PROFILES = os.path.join(ROOT, "profiles")
+
+
+def measured_traffic(workload: str):
+    """HBM bytes per launch of each kernel of the step, from the counter summary kept under profiles/
+    (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this file, scaled by what the same counters read for
+    en_copy_bytes of known size; written by bench_profiles.py).  Counters cannot be read from inside the
+    benchmark, so the figures of the last profiled tree are reported beside the live timing; {} when the
+    summary is not there."""
+    path = os.path.join(PROFILES, f"bench_{workload}_hbm_traffic.md")
+    out = {}
+    try:
+        with open(path) as f:
+            for line in f:
+                cells = [c.strip() for c in line.strip().strip("|").split("|")]
+                if len(cells) >= 3 and cells[0].startswith("`") and cells[0].endswith("`"):
+                    try:
+                        out[cells[0].strip("`")] = float(cells[-3]) * 1e6      # column "traffic MB"
+                    except ValueError:
+                        pass
+    except OSError:
+        pass
+    return out
+
+
 DTYPE_NAME = {"torch.float16": "f16", "torch.bfloat16": "bf16", "torch.float32": "f32"}
 
 
@@ -344,6 +356,30 @@ def run_workload(torch, w, steps, warmup, want_eager=True, want_kernels=True, st
     res["ms_per_step"] = wall_ms
     res["tokens_per_s"] = tokens / (wall_ms * 1e-3)
 
+    # the same step as an unchanged caller of the reference API issues it (examples/bert/bert.py:100-132): seven
+    # Python calls with the reference's semantics -- transpose_pad writes zeros into the padding rows, the
+    # softmax zeroes the whole tail of every row -- next to the one-call form above
+    if not w.decode and not step_only:
+        def step_api():
+            T = tokens
+            x = K.depad(d["hidden_padded"], w.batch, info, left_padded=w.left_padded, sum_seq=T)
+            qkv = K.transpose_pad(d["qkv_packed"], w.batch, w.seq, info, w.heads, 3 * w.head_dim)
+            q, k, v = torch.chunk(qkv, 3, dim=-1)
+            scores = K.attn_qk(q, k, info, causal=w.causal)
+            probs = K.scale_mask_softmax(w.batch, w.seq, w.heads, scores, info, scale=w.scale, causal=w.causal)
+            ctx = K.attn_pv(probs, v, info, causal=w.causal)
+            ctx_packed = K.transpose_depad(ctx, w.batch, T, w.seq, info, w.heads, w.head_dim)
+            attn_out = ctx_packed.view(1, T, w.heads * w.head_dim) if d["dense_out"] is None else d["dense_out"]
+            return K.layer_norm_forward(attn_out, d["gamma"], d["beta"], (w.hidden,), workloads.EPS, residual=x)
+        for _ in range(max(2, warmup // 2)):
+            step_api()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            step_api()
+        torch.cuda.synchronize()
+        res["api_sequence_ms_per_step"] = (time.perf_counter() - t0) * 1e3 / steps
+
     # the optional fused-attention form of the same step (QK^T + softmax + PV in one kernel); not the headline
     if not w.decode and w.dtype != torch.float32 and not step_only:
         def step_fused():
@@ -504,50 +540,75 @@ def kernel_table(torch, K, layer, workloads, w, d, info, steps, step_only=False)
 # ---------------------------------------------------------------------------
 # CPU baseline: the oracle on this box's host cores, bounded sample
 # ---------------------------------------------------------------------------
-def cpu_baseline(torch, w, budget_s=12.0):
+def host_cpu():
+    """(threads the process may use, os.cpu_count(), CPU model).  A one-GPU box exports OMP_NUM_THREADS for its
+    share of the host's cores; that is what the baseline runs on, and the machine's full count is printed beside it."""
+    total = os.cpu_count() or 1
+    granted = total
+    try:
+        granted = max(1, min(total, int(os.environ.get("OMP_NUM_THREADS", total))))
+    except ValueError:
+        pass
+    model = "unknown"
+    try:
+        with open("/proc/cpuinfo") as f:
+            for line in f:
+                if line.startswith("model name"):
+                    model = line.split(":", 1)[1].strip()
+                    break
+    except OSError:
+        pass
+    return granted, total, model
+
+
+def cpu_baseline(torch, w, full_batch, passes=3):
+    """The oracle's layer (a torch-eager restatement of the reference path) in fp32 on the host cores: the whole
+    batch for the fp32 workload, for the small fp16 one and for the headline workload, the first sequences of
+    the others; one warm-up pass, then the median of `passes` timed ones."""
     from energonai_amd import workloads
     from oracle import eager
-    cores = min(os.cpu_count() or 1, 16)
-    torch.set_num_threads(cores)
+    threads, total, model = host_cpu()
+    torch.set_num_threads(threads)
     if w.decode:
-        lens = workloads.make_lens(w)[:8]
-        sub = workloads.Workload(w.index, w.name, w.title, torch.float32, 8, w.seq, w.heads, w.head_dim, w.hidden,
+        nb = w.batch if full_batch else 8
+        lens = workloads.make_lens(w)[:nb]
+        sub = workloads.Workload(w.index, w.name, w.title, torch.float32, nb, w.seq, w.heads, w.head_dim, w.hidden,
                                  w.len_lo, w.len_hi, w.causal, w.left_padded, decode=True)
         d = workloads.make_decode_inputs(sub, dtype=torch.float32, lens=lens)
-        tokens = 8
-        sample = "first 8 of the 64 sequences, fp32 on the CPU"
+        tokens = nb
 
         def step():
             eager.decode_attention(d["q"], d["k_cache"], d["v_cache"], d["lens_list"], w.scale)
             eager.layer_norm(d["dense_out"], d["gamma"], d["beta"], workloads.EPS, residual=d["residual"])
     else:
-        nb = w.batch if w.name in ("c1", "c2") else 2
+        nb = w.batch if (full_batch or w.name in ("c1", "c2")) else 4
         lens = workloads.make_lens(w)[:nb]
         sub = workloads.Workload(w.index, w.name, w.title, torch.float32, nb, w.seq, w.heads, w.head_dim, w.hidden,
                                  w.len_lo, w.len_hi, w.causal, w.left_padded)
         d = workloads.make_inputs(sub, dtype=torch.float32, lens=lens)
         tokens = d["total"]
-        sample = (f"{'all' if nb == w.batch else 'first ' + str(nb) + ' of the'} {w.batch} sequences "
-                  f"({tokens} tokens), fp32 on the CPU")
 
         def step():
             eager.layer_unpadded(d["hidden_padded"], d["qkv_packed"], d["lens_list"], w.heads, w.head_dim, d["gamma"],
                                  d["beta"], workloads.EPS, w.scale, w.causal, w.left_padded,
                                  dense_out=d["dense_out"])
-    step()  # warm-up
+    which = "all" if nb == w.batch else f"the first {nb} of the"
+    unit = "sequences (one new token each)" if w.decode else f"sequences ({tokens} tokens)"
+    step()  # warm-up (first touch of the fp32 score tensors)
     times = []
-    t_begin = time.perf_counter()
-    while len(times) < 3 or (time.perf_counter() - t_begin < budget_s and len(times) < 50):
+    for _ in range(passes):
         t0 = time.perf_counter()
         step()
         times.append(time.perf_counter() - t0)
-        if time.perf_counter() - t_begin > 3 * budget_s:
-            break
     times.sort()
     med = times[len(times) // 2]
-    return {"value": tokens / med, "unit": "tokens/s", "cores": cores, "kind": "port",
-            "sample": f"{sample}; median of {len(times)} passes, {med * 1e3:.1f} ms each; "
-                      f"oracle.eager.layer_unpadded (torch-eager restatement of the reference path)"}
+    return {"value": tokens / med, "unit": "tokens/s", "cores": threads, "kind": "port",
+            "host_cpu_count": total, "cpu_model": model,
+            "sample": f"{w.name}: {which} {w.batch} {unit}, fp32 on the CPU"
+                      f"{'' if w.dtype == torch.float32 else ' (the GPU path stores ' + DTYPE_NAME[str(w.dtype)] + ')'}; "
+                      f"median of {len(times)} passes after one warm-up, {med * 1e3:.1f} ms each; "
+                      f"{threads} threads on a host of {total} ({model}); "
+                      f"oracle.eager.layer_unpadded, the torch-eager restatement of the reference path"}
 
 
 def copy_yardstick(torch, iters):
@@ -575,7 +636,7 @@ def main(argv=None) -> int:
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--workload", default="c2", choices=["c1", "c2", "c3", "c4", "c5"])
+    ap.add_argument("--workload", default="c3", choices=["c1", "c2", "c3", "c4", "c5"])
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-extra", action="store_true", help="only the headline workload, no eager / other workloads")
     ap.add_argument("--step-only", action="store_true",
@@ -620,7 +681,7 @@ def main(argv=None) -> int:
     row = kt[dom]
     roofline = {"kernel": dom, "bound": "hbm", "achieved": row["GBps"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
                 "frac": row["GBps"] / HBM_PEAK_GBS,
-                "traffic": MEASURED_TRAFFIC_C2.get(dom) if w.name == "c2" else None, "us_per_launch": row["us"],
+                "traffic": measured_traffic(w.name).get(dom), "us_per_launch": row["us"],
                 "alg_bytes_per_launch": row["alg_MB"] * 1e6}
 
     out = {
@@ -630,6 +691,7 @@ def main(argv=None) -> int:
         "config": {"workload": f"{w.name}: {w.title}; batch {w.batch}, bucket {w.seq}, {w.heads}x{w.head_dim} heads, "
                                f"LayerNorm width {w.hidden}, {head['tokens']} valid tokens"},
         "roofline": roofline,
+        "api_sequence_ms_per_step": head.get("api_sequence_ms_per_step"),
         "graph_ms_per_step": head.get("graph_ms_per_step"),
         "fused_attention_ms_per_step": head.get("fused_attention_ms_per_step"),
         "packed_fused_attention_ms_per_step": head.get("packed_fused_attention_ms_per_step"),
@@ -660,7 +722,16 @@ def main(argv=None) -> int:
         except Exception as exc:
             out["model_block_decode"] = {"error": str(exc)[:300]}
     if not ns.no_cpu:
-        out["cpu_baseline"] = cpu_baseline(torch, w)
+        # every GPU tensor is gone by now; the CPU leg runs last so that it cannot disturb the GPU timings
+        out["cpu_baseline"] = cpu_baseline(torch, w, full_batch=True)
+        if not ns.no_extra:
+            out["cpu_baselines"] = {w.name: out["cpu_baseline"]}
+            for ow in workloads.WORKLOADS:
+                if ow.name != w.name:
+                    try:
+                        out["cpu_baselines"][ow.name] = cpu_baseline(torch, ow, full_batch=False)
+                    except Exception as exc:
+                        out["cpu_baselines"][ow.name] = {"error": str(exc)[:300]}
     else:
         out["cpu_baseline"] = None
     print(json.dumps(out))

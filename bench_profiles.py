@@ -1,0 +1,195 @@
+#!/usr/bin/env python3
+"""Profiles of bench.py under rocprofv3, turned into the short summaries kept under profiles/.
+
+    python3 bench_profiles.py trace   --workload c3      # rocprofv3 --kernel-trace --stats of `bench.py --step-only`
+    python3 bench_profiles.py traffic --workload c3      # two --pmc runs (FETCH_SIZE, then WRITE_SIZE) + copy calibration
+
+Each sub-command starts rocprofv3 as a child process with `python3 bench.py ...` after `--`, reads the CSV files it
+leaves under gpurun_out/prof/, and prints a markdown summary (redirect it into profiles/bench_<workload>_*.md).
+`--step-only` makes bench.py launch nothing but the step and the kernels of the step, each op the same number of
+times, so every kernel name in a trace is one op of one workload.
+
+The traffic summary is what bench.py reads `roofline.traffic` from (column "traffic MB" of the row whose first
+cell is the op's name in the bench line).
+"""
+from __future__ import annotations
+
+import argparse
+import collections
+import csv
+import glob
+import json
+import os
+import subprocess
+import sys
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+OUT = os.path.join(ROOT, "gpurun_out", "prof")
+
+# kernel name (substring) -> the op's key in the bench line; first match wins
+KERNEL_KEYS = [
+    ("row_gather_pair_kernel", "depad+transpose_pad_valid_rows"),
+    ("DepadRowsMap", "depad"),
+    ("DepadHeadsMap", "transpose_depad"),
+    ("PadMap", "transpose_pad_valid_rows"),
+    ("attn_qk", "attn_qk"),
+    ("softmax", "scale_mask_softmax_no_tail"),
+    ("attn_pv", "attn_pv"),
+    ("layernorm", "layernorm_residual"),
+    ("decode_qk", "decode_qk"),
+    ("decode_pv", "decode_pv"),
+    ("attn_fused", "attn_fused"),
+    ("copy_kernel", "copy"),
+]
+# in the decode step the softmax keeps its full name in the bench line
+DECODE_KEYS = {"scale_mask_softmax_no_tail": "scale_mask_softmax"}
+
+
+def key_of(kernel: str, decode: bool):
+    for sub, key in KERNEL_KEYS:
+        if sub in kernel:
+            return DECODE_KEYS.get(key, key) if decode else key
+    return None
+
+
+def run_profiler(tag: str, prof_args, bench_args, timeout_s: int):
+    """rocprofv3 <prof_args> -d gpurun_out/prof/<tag> -- python3 bench.py <bench_args>; returns (dir, bench line)."""
+    d = os.path.join(OUT, tag)
+    subprocess.run(["rm", "-rf", d], check=True)
+    os.makedirs(d, exist_ok=True)
+    cmd = ["rocprofv3"] + prof_args + ["--output-format", "csv", "-d", d, "-o", "run", "--",
+                                      "python3", os.path.join(ROOT, "bench.py")] + bench_args
+    env = dict(os.environ, TMPDIR="/tmp")
+    print("[bench_profiles] " + " ".join(cmd), file=sys.stderr, flush=True)
+    proc = subprocess.run(cmd, cwd=ROOT, env=env, stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True,
+                          timeout=timeout_s)
+    if proc.returncode != 0:
+        sys.stderr.write(proc.stderr[-3000:])
+        raise SystemExit(f"rocprofv3 exited with {proc.returncode}")
+    line = None
+    for ln in proc.stdout.splitlines():
+        if ln.startswith("{"):
+            line = json.loads(ln)
+    return d, line, " ".join(cmd[:1] + prof_args + ["--", "python3", "bench.py"] + bench_args)
+
+
+def find_csv(d: str, suffix: str) -> str:
+    hits = glob.glob(os.path.join(d, "**", f"*{suffix}"), recursive=True)
+    if not hits:
+        raise SystemExit(f"no *{suffix} under {d}")
+    return hits[0]
+
+
+def trace_rows(path: str):
+    agg = collections.defaultdict(list)
+    with open(path) as f:
+        for r in csv.DictReader(f):
+            agg[r["Kernel_Name"]].append((int(r["End_Timestamp"]) - int(r["Start_Timestamp"])) / 1e3)
+    return agg
+
+
+def counter_rows(path: str, counter: str):
+    agg = collections.defaultdict(list)
+    with open(path) as f:
+        for r in csv.DictReader(f):
+            if r["Counter_Name"] == counter:
+                agg[r["Kernel_Name"]].append(float(r["Counter_Value"]))
+    return agg
+
+
+def cmd_trace(ns) -> int:
+    bench_args = ["--workload", ns.workload, "--step-only", "--no-cpu", "--steps", str(ns.steps), "--warmup", str(ns.warmup)]
+    d, line, shown = run_profiler(f"kt_{ns.workload}", ["--kernel-trace", "--stats"], bench_args, ns.timeout)
+    agg = trace_rows(find_csv(d, "kernel_trace.csv"))
+    decode = ns.workload == "c5"
+    kt = (line or {}).get("kernels", {})
+    print(f"# rocprofv3 kernel-trace summary: `bench.py --workload {ns.workload} --step-only`\n")
+    print("Command (MI355X box, repo root; the summary below is this command's stdout):\n")
+    print(f"```\npython3 bench_profiles.py trace --workload {ns.workload}\n  -> {shown}\n```\n")
+    if line:
+        print(f"Bench line of the profiled run: {line['ms_per_step'] * 1e3:.1f} us per step "
+              f"({line['config']['workload']}). Event timings of the same run (`us (events)`) are taken by bench.py "
+              f"with HIP events on the launch stream, back-to-back launches; the profiler's own durations are "
+              f"per dispatch.\n")
+    print("| op (key in the bench line) | kernel | calls | avg us | min us | max us | us (events) |\n|---|---|---|---|---|---|---|")
+    for name, v in sorted(agg.items(), key=lambda kv: -sum(kv[1])):
+        key = key_of(name, decode)
+        if key is None:
+            continue
+        ev = kt.get(key, {}).get("us")
+        print(f"| `{key}` | `{name[:100]}` | {len(v)} | {sum(v) / len(v):.1f} | {min(v):.1f} | {max(v):.1f} | "
+              f"{'' if ev is None else format(ev, '.1f')} |")
+    other = sum(sum(v) for n, v in agg.items() if key_of(n, decode) is None)
+    print(f"\nOther kernels in the trace (torch fills and copies while the inputs are made): {other / 1e3:.1f} ms in total.")
+    return 0
+
+
+def cmd_traffic(ns) -> int:
+    bench_args = ["--workload", ns.workload, "--step-only", "--no-cpu", "--steps", str(ns.steps), "--warmup", str(ns.warmup)]
+    decode = ns.workload == "c5"
+    per_counter, shown_cmds, line = {}, [], None
+    calib = {}
+    for counter in ("FETCH_SIZE", "WRITE_SIZE"):
+        d, line, shown = run_profiler(f"pmc_{counter}_{ns.workload}", ["--pmc", counter], bench_args, ns.timeout)
+        shown_cmds.append(shown)
+        per_counter[counter] = counter_rows(find_csv(d, "counter_collection.csv"), counter)
+        d, cline, shown = run_profiler(f"pmc_{counter}_copy", ["--pmc", counter], ["--copy-yardstick", "--steps", "5"],
+                                       ns.timeout)
+        shown_cmds.append(shown)
+        rows = counter_rows(find_csv(d, "counter_collection.csv"), counter)
+        vals = [v for n, vs in rows.items() if "copy_kernel" in n for v in vs]
+        # the copy kernel moves 64 MiB, 256 MiB and 1 GiB each way; the largest launches dominate the maximum
+        calib[counter] = (1 << 30) / max(vals)      # bytes per counter unit
+    alg = {k: v["alg_MB"] * 1e6 for k, v in (line or {}).get("kernels", {}).items()}
+    # every op of the step is launched the same number of times in a --step-only run
+    keys = collections.defaultdict(lambda: {"FETCH_SIZE": 0.0, "WRITE_SIZE": 0.0, "names": set(), "n": 0})
+    for counter, rows in per_counter.items():
+        for name, vals in rows.items():
+            key = key_of(name, decode)
+            if key is None or key == "copy":
+                continue
+            keys[key][counter] += sum(vals)
+            keys[key]["names"].add(name[:70])
+            keys[key]["n"] = max(keys[key]["n"], len(vals))
+    calls = max((v["n"] for k, v in keys.items() if k == "layernorm_residual"), default=0) or \
+        max(v["n"] for v in keys.values())
+    print(f"# HBM traffic per launch, `bench.py --workload {ns.workload} --step-only`, from FETCH_SIZE / WRITE_SIZE\n")
+    print("Command (MI355X box, repo root; the summary below is this command's stdout; one counter per run):\n")
+    print(f"```\npython3 bench_profiles.py traffic --workload {ns.workload}")
+    for c in shown_cmds:
+        print(f"  -> {c}")
+    print("```\n")
+    print(f"Calibration: the same counters over `en_copy_bytes` of 1 GiB (reads 1 GiB, writes 1 GiB) give "
+          f"{calib['FETCH_SIZE']:.1f} bytes per FETCH_SIZE unit and {calib['WRITE_SIZE']:.1f} bytes per WRITE_SIZE unit; "
+          f"the columns below are scaled by that. Each op ran {calls} times; traffic = counter total / {calls}.\n")
+    print("| op (key in the bench line) | kernels | read MB | written MB | traffic MB | algorithmic MB | traffic / algorithmic |\n"
+          "|---|---|---|---|---|---|---|")
+    for key, v in keys.items():
+        rd = v["FETCH_SIZE"] * calib["FETCH_SIZE"] / calls / 1e6
+        wr = v["WRITE_SIZE"] * calib["WRITE_SIZE"] / calls / 1e6
+        a = alg.get(key)
+        if key == "depad+transpose_pad_valid_rows":
+            a = alg.get("depad", 0) + alg.get("transpose_pad_valid_rows", 0)
+        print(f"| `{key}` | {'; '.join(sorted(v['names']))} | {rd:.1f} | {wr:.1f} | {rd + wr:.1f} | "
+              f"{'' if not a else format(a / 1e6, '.1f')} | {'' if not a else format((rd + wr) * 1e6 / a, '.2f')} |")
+    print("\nReads below the algorithmic figure are hits in the 256 MB memory-side cache, which FETCH_SIZE does not count "
+          "as HBM traffic; writes above it are whole 16-byte vectors at ragged row ends.")
+    return 0
+
+
+def main(argv=None) -> int:
+    ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
+    sub = ap.add_subparsers(dest="cmd", required=True)
+    for name, fn in (("trace", cmd_trace), ("traffic", cmd_traffic)):
+        p = sub.add_parser(name)
+        p.add_argument("--workload", default="c3", choices=["c1", "c2", "c3", "c4", "c5"])
+        p.add_argument("--steps", type=int, default=20)
+        p.add_argument("--warmup", type=int, default=5)
+        p.add_argument("--timeout", type=int, default=300, help="seconds allowed for each rocprofv3 run")
+        p.set_defaults(fn=fn)
+    ns = ap.parse_args(argv)
+    return ns.fn(ns)
+
+
+if __name__ == "__main__":
+    sys.exit(main())
