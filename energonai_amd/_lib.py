@@ -42,8 +42,12 @@ SIGNATURES = {
                                       c_int, c_void_p]),
     "en_layernorm_fwd": (c_int, [c_void_p] * 9 + [c_int64, c_int64, c_float, c_int, c_int, c_void_p]),
     "en_padding_offsets": (c_int, [c_void_p, c_int, c_int, c_int, c_void_p, c_void_p]),
-    "en_attn_qk": (c_int, [c_void_p] * 5 + [c_int] * 5 + [c_int64] * 6 + [c_float, c_int, c_int, c_void_p]),
-    "en_attn_pv": (c_int, [c_void_p] * 5 + [c_int] * 5 + [c_int64] * 6 + [c_int, c_int, c_int, c_void_p]),
+    "en_attn_qk": (c_int, [c_void_p] * 5 + [c_int] * 5 + [c_int64] * 6 + [c_float, c_int, c_int, c_void_p, c_void_p,
+                           c_int, c_void_p]),
+    "en_attn_pv": (c_int, [c_void_p] * 5 + [c_int] * 5 + [c_int64] * 6 + [c_int, c_int, c_int, c_void_p, c_void_p,
+                           c_int, c_void_p]),
+    "en_packed_scores_elems": (c_int64, [c_int] * 4),
+    "en_scale_mask_softmax_packed": (c_int, [c_void_p, c_void_p, c_int, c_int, c_int, c_float, c_int, c_void_p]),
     "en_decode_qk": (c_int, [c_void_p] * 4 + [c_int] * 4 + [c_int64] * 3 + [c_float, c_int, c_void_p]),
     "en_decode_pv": (c_int, [c_void_p] * 4 + [c_int] * 4 + [c_int64] * 3 + [c_int, c_void_p]),
     "en_attn_fused": (c_int, [c_void_p] * 6 + [c_int] * 5 + [c_void_p] * 6 + [c_float, c_int, c_int, c_void_p]),

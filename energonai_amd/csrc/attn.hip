@@ -66,15 +66,15 @@ __global__ __launch_bounds__(kBlock) void attn_qk_kernel(AttnArgs a) {
   const int r = lane & 31, g = lane >> 5;
   const int wq = wave & 1, wk = wave >> 1;
 
-  const T *qbase = reinterpret_cast<const T *>(a.a_ptr) + (int64_t)b * a.q_sb + (int64_t)h * a.q_sh;
-  const T *kbase = reinterpret_cast<const T *>(a.b_ptr) + (int64_t)b * a.k_sb + (int64_t)h * a.k_sh;
+  const T *qbase = reinterpret_cast<const T *>(a.a_ptr) + q_unit_offset(a, b, h);
+  const T *kbase = reinterpret_cast<const T *>(a.b_ptr) + k_unit_offset(a, b, h);
   T *sbase = reinterpret_cast<T *>(a.out) + ((int64_t)unit * a.Sq) * a.Sk;
 
   // Q fragments stay in registers for the whole key loop.
   uint4 qf[NT][NVS];
 #pragma unroll
   for (int nt = 0; nt < NT; ++nt) {
-    const int row = min(q0 + wq * 64 + nt * 32 + r, a.Sq - 1);
+    const int row = min(q0 + wq * 64 + nt * 32 + r, ql - 1);    // rows past the last valid one are never stored
     const T *qrow = qbase + (int64_t)row * a.q_ss;
 #pragma unroll
     for (int vs = 0; vs < NVS; ++vs) {
@@ -230,9 +230,9 @@ __global__ __launch_bounds__(kBlock, 3) void attn_qk_strip_kernel(AttnArgs a) {
   const int qw = q0 + wave * 32;                 // first query of this wave
   const int q = qw + r;                          // query whose scores this lane accumulates
 
-  const T *qbase = reinterpret_cast<const T *>(a.a_ptr) + (int64_t)b * a.q_sb + (int64_t)h * a.q_sh;
-  const T *kbase = reinterpret_cast<const T *>(a.b_ptr) + (int64_t)b * a.k_sb + (int64_t)h * a.k_sh;
-  T *sbase = reinterpret_cast<T *>(a.out) + ((int64_t)unit * a.Sq) * a.Sk;
+  const T *qbase = reinterpret_cast<const T *>(a.a_ptr) + q_unit_offset(a, b, h);
+  const T *kbase = reinterpret_cast<const T *>(a.b_ptr) + k_unit_offset(a, b, h);
+  T *sbase = reinterpret_cast<T *>(a.out) + score_unit_offset<EPV>(a, unit);
 
   // Q fragments (B operand): this lane's query row, 8 channels per step; rows >= ql read as zero
   uint4 qf[NVS];
@@ -249,7 +249,7 @@ __global__ __launch_bounds__(kBlock, 3) void attn_qk_strip_kernel(AttnArgs a) {
   // K rows past the last valid key read as zeros through the bounds check (no traffic, no branches);
   // lanes whose channel chunk lies past the head size sit at an offset that stays out of range
   const rsrc_t k_rsrc = make_rsrc(kbase, (uint32_t)(((int64_t)(kl - 1) * a.k_ss + a.D) * E::kSize));
-  const rsrc_t s_rsrc = make_rsrc(sbase, (uint32_t)((int64_t)ql * a.Sk * E::kSize));   // rows >= ql are dropped
+  const rsrc_t s_rsrc = make_rsrc(sbase, (uint32_t)(score_row_offset<EPV>(a, ql) * E::kSize));   // rows >= ql are dropped
   const uint32_t k_row_bytes = (uint32_t)(a.k_ss * E::kSize);
   const int k_row = tid / KVEC_ROW, k_c = tid % KVEC_ROW;
   uint32_t k_off = (k_c * EPV < a.D) ? k_row * k_row_bytes + k_c * EPV * E::kSize : kOutOfRange;
@@ -274,7 +274,7 @@ __global__ __launch_bounds__(kBlock, 3) void attn_qk_strip_kernel(AttnArgs a) {
   for (int i = 0; i < CSTORES; ++i) {
     const int row = qw + sr + i * (kWave / CVEC_ROW);
     k_end[i] = min(a.causal ? min(kl, row + (kl - ql) + 1) : kl, a.Sk);
-    s_off[i] = (uint32_t)(((int64_t)row * a.Sk + sc) * E::kSize);
+    s_off[i] = (uint32_t)((score_row_offset<EPV>(a, row) + sc) * E::kSize);
   }
 
   fetch_k();
@@ -373,7 +373,7 @@ __global__ __launch_bounds__(kBlock) void attn_pv_kernel(AttnArgs a) {
   seq_extents(a, b, kl, ql);
   const int q0 = qi * kQTile;
   const int tid = threadIdx.x;
-  T *cbase = reinterpret_cast<T *>(a.out) + (int64_t)b * a.q_sb + (int64_t)h * a.q_sh;
+  T *cbase = reinterpret_cast<T *>(a.out) + q_unit_offset(a, b, h);
 
   if (q0 >= ql) {
     if (a.zero_padding) {  // whole tile is padding
@@ -393,7 +393,7 @@ __global__ __launch_bounds__(kBlock) void attn_pv_kernel(AttnArgs a) {
   const int wq = wave & 1, wd = wave >> 1;
 
   const T *pbase = reinterpret_cast<const T *>(a.a_ptr) + ((int64_t)unit * a.Sq) * a.Sk;
-  const T *vbase = reinterpret_cast<const T *>(a.b_ptr) + (int64_t)b * a.k_sb + (int64_t)h * a.k_sh;
+  const T *vbase = reinterpret_cast<const T *>(a.b_ptr) + k_unit_offset(a, b, h);
 
   floatx16 acc[MT][NT];
 #pragma unroll
@@ -560,7 +560,7 @@ __global__ __launch_bounds__(kBlock, 3) void attn_pv_strip_kernel(AttnArgs a) {
   seq_extents(a, b, kl, ql);
   const int q0 = qi * kQTile;
   const int tid = threadIdx.x;
-  T *cbase = reinterpret_cast<T *>(a.out) + (int64_t)b * a.q_sb + (int64_t)h * a.q_sh;
+  T *cbase = reinterpret_cast<T *>(a.out) + q_unit_offset(a, b, h);
 
   if (q0 >= ql) {
     if (a.zero_padding) {  // whole tile is padding
@@ -580,10 +580,10 @@ __global__ __launch_bounds__(kBlock, 3) void attn_pv_strip_kernel(AttnArgs a) {
   const int qw = q0 + wave * 32;                 // first query of this wave
   const int q = qw + r;                          // query whose context this lane accumulates
 
-  const T *pbase = reinterpret_cast<const T *>(a.a_ptr) + ((int64_t)unit * a.Sq) * a.Sk;
-  const T *vbase = reinterpret_cast<const T *>(a.b_ptr) + (int64_t)b * a.k_sb + (int64_t)h * a.k_sh;
+  const T *pbase = reinterpret_cast<const T *>(a.a_ptr) + score_unit_offset<EPV>(a, unit);
+  const T *vbase = reinterpret_cast<const T *>(a.b_ptr) + k_unit_offset(a, b, h);
   // rows of padded queries lie past the end of the resource and read as zero; so do V rows >= kl
-  const rsrc_t p_rsrc = make_rsrc(pbase, (uint32_t)((int64_t)ql * a.Sk * E::kSize));
+  const rsrc_t p_rsrc = make_rsrc(pbase, (uint32_t)(score_row_offset<EPV>(a, ql) * E::kSize));
   const uint32_t v_bytes = kl > 0 ? (uint32_t)(((int64_t)(kl - 1) * a.k_ss + a.D) * E::kSize) : 0u;
   const rsrc_t v_rsrc = make_rsrc(vbase, v_bytes);
   const uint32_t v_row_bytes = (uint32_t)(a.k_ss * E::kSize);
@@ -618,7 +618,7 @@ __global__ __launch_bounds__(kBlock, 3) void attn_pv_strip_kernel(AttnArgs a) {
 #pragma unroll
   for (int i = 0; i < PLOADS; ++i) {
     const int row = qw + pr + i * (kWave / PVEC_ROW);
-    p_off[i] = (uint32_t)(((int64_t)row * a.Sk + pc) * E::kSize);
+    p_off[i] = (uint32_t)((score_row_offset<EPV>(a, row) + pc) * E::kSize);
     p_vis[i] = row < ql ? tile_key_extent(a, row, kl, ql) : 0;
   }
   uint4 preg[PLOADS];
@@ -707,11 +707,19 @@ static bool strides_vec_ok(int64_t sb, int64_t sh, int64_t ss, int epv) {
   return (sb % epv) == 0 && (sh % epv) == 0 && (ss % epv) == 0;
 }
 
+// bytes of the score tensor the kernels go through: all of [B,H,Sq,Sk], or the packed causal prefixes
+template <int DT>
+static int64_t score_tensor_bytes(const AttnArgs &a) {
+  constexpr int EPV = 16 / Elem<DT>::kSize;
+  return (int64_t)a.units * (a.packed_scores ? packed_row_start<EPV>(a.Sq) : (int64_t)a.Sq * a.Sk) * Elem<DT>::kSize;
+}
+
 template <int DT>
 static int launch_qk(AttnArgs &a, hipStream_t s) {
   const unsigned grid = (unsigned)(ceil_div(a.units, kXcds) * kXcds * a.ntq);
   // a score tensor too large to stay in the memory-side cache is written with the non-temporal policy
-  const bool stream = (int64_t)a.units * a.Sq * a.Sk * Elem<DT>::kSize >= kStreamScoreBytes;
+  const bool stream = score_tensor_bytes<DT>(a) >= kStreamScoreBytes;
+  if (a.packed_scores && (DT == EN_F32 || !a.vec_out)) return EN_ERR_UNSUPPORTED;
   if constexpr (DT != EN_F32) {
     if (a.vec_out) {   // 16-bit, aligned rows
       if (a.D <= 64) {
@@ -745,7 +753,8 @@ template <int DT>
 static int launch_pv(AttnArgs &a, hipStream_t s) {
   const unsigned grid = (unsigned)(ceil_div(a.units, kXcds) * kXcds * a.ntq);
   // probabilities of a tensor too large to stay cached are read with the non-temporal policy
-  const bool stream = (int64_t)a.units * a.Sq * a.Sk * Elem<DT>::kSize >= kStreamScoreBytes;
+  const bool stream = score_tensor_bytes<DT>(a) >= kStreamScoreBytes;
+  if (a.packed_scores && (DT == EN_F32 || !a.vec_out)) return EN_ERR_UNSUPPORTED;
   if constexpr (DT != EN_F32) {
     if (a.vec_out) {   // 16-bit, aligned rows
       if (a.D <= 64) {
@@ -796,10 +805,13 @@ extern "C" {
 int en_attn_qk(const void *q, const void *k, void *scores, const int32_t *k_lens, const int32_t *q_lens, int batch,
                int head_num, int q_seq_len, int k_seq_len, int size_per_head, int64_t q_stride_b,
                int64_t q_stride_h, int64_t q_stride_s, int64_t k_stride_b, int64_t k_stride_h, int64_t k_stride_s,
-               float alpha, int causal, int dtype, en_stream_t stream) {
+               float alpha, int causal, int dtype, const int32_t *q_row_offsets, const int32_t *k_row_offsets,
+               int packed_scores, en_stream_t stream) {
   using namespace en;
   int rc = check_common(q, k, scores, k_lens, batch, head_num, q_seq_len, k_seq_len, size_per_head, dtype);
   if (rc) return rc;
+  // the packed score layout is that of causal self-attention: row q holds q + 1 scores
+  if (packed_scores && (!causal || q_lens || q_seq_len != k_seq_len)) return EN_ERR_UNSUPPORTED;
   const int es = dtype_size(dtype), epv = 16 / es;
   if (!aligned_to(q, 16) || !aligned_to(k, 16) || !aligned_to(scores, es)) return EN_ERR_ALIGN;
   if (!strides_vec_ok(q_stride_b, q_stride_h, q_stride_s, epv) ||
@@ -813,7 +825,8 @@ int en_attn_qk(const void *q, const void *k, void *scores, const int32_t *k_lens
   a.q_sb = q_stride_b; a.q_sh = q_stride_h; a.q_ss = q_stride_s;
   a.k_sb = k_stride_b; a.k_sh = k_stride_h; a.k_ss = k_stride_s;
   a.alpha = alpha; a.causal = causal ? 1 : 0; a.zero_padding = 0;
-  a.vec_out = ((k_seq_len % epv) == 0 && aligned_to(scores, 16)) ? 1 : 0;
+  a.q_row0 = q_row_offsets; a.k_row0 = k_row_offsets; a.packed_scores = packed_scores ? 1 : 0;
+  a.vec_out = ((packed_scores || (k_seq_len % epv) == 0) && aligned_to(scores, 16)) ? 1 : 0;
   a.ntq = (int)ceil_div(q_seq_len, kQTile);
   a.units = batch * head_num;
   hipStream_t s = (hipStream_t)stream;
@@ -827,10 +840,14 @@ int en_attn_qk(const void *q, const void *k, void *scores, const int32_t *k_lens
 int en_attn_pv(const void *p, const void *v, void *ctx, const int32_t *k_lens, const int32_t *q_lens, int batch,
                int head_num, int q_seq_len, int k_seq_len, int size_per_head, int64_t v_stride_b,
                int64_t v_stride_h, int64_t v_stride_s, int64_t c_stride_b, int64_t c_stride_h, int64_t c_stride_s,
-               int causal, int zero_padding, int dtype, en_stream_t stream) {
+               int causal, int zero_padding, int dtype, const int32_t *c_row_offsets, const int32_t *v_row_offsets,
+               int packed_scores, en_stream_t stream) {
   using namespace en;
   int rc = check_common(p, v, ctx, k_lens, batch, head_num, q_seq_len, k_seq_len, size_per_head, dtype);
   if (rc) return rc;
+  if (packed_scores && (!causal || q_lens || q_seq_len != k_seq_len)) return EN_ERR_UNSUPPORTED;
+  // a packed context has no padding rows: what follows a sequence's last row is the next sequence
+  if (c_row_offsets && zero_padding) return EN_ERR_UNSUPPORTED;
   const int es = dtype_size(dtype), epv = 16 / es;
   if (!aligned_to(p, es) || !aligned_to(v, 16) || !aligned_to(ctx, 4 * es)) return EN_ERR_ALIGN;
   if (!strides_vec_ok(v_stride_b, v_stride_h, v_stride_s, epv) ||
@@ -844,7 +861,8 @@ int en_attn_pv(const void *p, const void *v, void *ctx, const int32_t *k_lens, c
   a.q_sb = c_stride_b; a.q_sh = c_stride_h; a.q_ss = c_stride_s;
   a.k_sb = v_stride_b; a.k_sh = v_stride_h; a.k_ss = v_stride_s;
   a.alpha = 1.f; a.causal = causal ? 1 : 0; a.zero_padding = zero_padding ? 1 : 0;
-  a.vec_out = ((k_seq_len % epv) == 0 && aligned_to(p, 16)) ? 1 : 0;
+  a.q_row0 = c_row_offsets; a.k_row0 = v_row_offsets; a.packed_scores = packed_scores ? 1 : 0;
+  a.vec_out = ((packed_scores || (k_seq_len % epv) == 0) && aligned_to(p, 16)) ? 1 : 0;
   a.ntq = (int)ceil_div(q_seq_len, kQTile);
   a.units = batch * head_num;
   hipStream_t s = (hipStream_t)stream;

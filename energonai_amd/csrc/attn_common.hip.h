@@ -66,7 +66,29 @@ struct AttnArgs {
   int vec_out;   // output rows may be written with 128-bit stores
   int ntq;       // query tiles per unit
   int units;     // B * H
+  // Packed operands: batch b's rows start at row q_row0[b] (q in QK, ctx in PV) / k_row0[b] (k in QK, v in PV)
+  // of a tensor that holds the valid rows of all sequences back to back; null = rows start at b * batch stride.
+  const int32_t *q_row0;
+  const int32_t *k_row0;
+  int packed_scores;   // scores / probabilities are the packed causal prefixes (common.hip.h), not [B,H,Sq,Sk]
 };
+
+// first element of (batch b, head h) in q / ctx and in k / v
+__device__ __forceinline__ int64_t q_unit_offset(const AttnArgs &a, int b, int h) {
+  return (int64_t)b * a.q_sb + (a.q_row0 ? (int64_t)a.q_row0[b] * a.q_ss : 0) + (int64_t)h * a.q_sh;
+}
+__device__ __forceinline__ int64_t k_unit_offset(const AttnArgs &a, int b, int h) {
+  return (int64_t)b * a.k_sb + (a.k_row0 ? (int64_t)a.k_row0[b] * a.k_ss : 0) + (int64_t)h * a.k_sh;
+}
+// scores of a unit: first element, elements up to the start of row q, elements of the rows below ql
+template <int EPV>
+__device__ __forceinline__ int64_t score_unit_offset(const AttnArgs &a, int unit) {
+  return (int64_t)unit * (a.packed_scores ? packed_row_start<EPV>(a.Sq) : (int64_t)a.Sq * a.Sk);
+}
+template <int EPV>
+__device__ __forceinline__ int64_t score_row_offset(const AttnArgs &a, int q) {
+  return a.packed_scores ? packed_row_start<EPV>(q) : (int64_t)q * a.Sk;
+}
 
 // workgroup id -> (unit, query tile): see the header comment.
 __device__ __forceinline__ bool map_block(const AttnArgs &a, int &unit, int &qi) {

@@ -170,6 +170,19 @@ __device__ __forceinline__ float block_allreduce(float v, float *slots) {
   return r;
 }
 
+// ---- packed causal scores -------------------------------------------------------------------------------
+// Under a causal mask of a self-attention batch row q of a (batch, head) unit holds q + 1 visible scores.  In the
+// padded [B,H,S,S] layout those prefixes start a whole row pitch apart: a kernel that streams them touches short,
+// ragged pieces of memory (measured: 4.7 TB/s for an in-place pass over them against 6.5 TB/s over one
+// contiguous range).  The packed layout keeps only the prefixes, each rounded up to one 16-byte vector of V
+// elements, back to back: row q starts at packed_row_start(q) elements into its unit and holds V * (q / V + 1)
+// elements; every unit owns a slot of packed_row_start(S) elements, S the bucket length, whatever its length.
+template <int V>
+__host__ __device__ __forceinline__ int64_t packed_row_start(int64_t q) {
+  const int64_t t = q / V;
+  return V * (V * t * (t + 1) / 2 + (q - V * t) * (t + 1));
+}
+
 // pad.hip: depad and transpose_pad (of all head_num rows per token; valid rows only when zero_padding == 0) in
 // one launch when both move 16-byte multiples, as two launches otherwise.  Same results as en_depad followed
 // by en_transpose_pad_heads.

@@ -65,9 +65,9 @@ extern "C" int en_padding_removal_layer(const void *hidden_padded, const void *q
   if (!hidden_padded || !qkv_packed || !gamma || !beta || !ctx_packed || !y || !cu_seqlens || !seq_lens)
     return EN_ERR_NULL;
   if (!x_packed && !fold_depad_offsets) return EN_ERR_NULL;
-  if (attention_form < 0 || attention_form > 2) return EN_ERR_UNSUPPORTED;
-  if (attention_form != 2 && (!qkv_padded || !ctx)) return EN_ERR_NULL;
-  if (attention_form == 0 && !scores) return EN_ERR_NULL;
+  if (attention_form < 0 || attention_form > 4) return EN_ERR_UNSUPPORTED;
+  if (attention_form < 2 && (!qkv_padded || !ctx)) return EN_ERR_NULL;
+  if ((attention_form == 0 || attention_form >= 3) && !scores) return EN_ERR_NULL;
   const int es = dtype_size(dtype);
   if (!es) return EN_ERR_DTYPE;
   if (total_tokens < 0 || hidden < 1) return EN_ERR_SHAPE;
@@ -76,7 +76,7 @@ extern "C" int en_padding_removal_layer(const void *hidden_padded, const void *q
   const int B = batch, S = max_seq_len, H = head_num, D = size_per_head;
   int rc = EN_OK;
   // depad depends on nothing the attention chain produces: with transpose_pad to run it shares that launch
-  const bool depad_alone = !fold_depad_offsets && attention_form == 2;
+  const bool depad_alone = !fold_depad_offsets && attention_form >= 2;
   if (depad_alone) {
     rc = en_depad(hidden_padded, x_packed, cu_seqlens, B, S, hidden, es, left_padded, stream);
     if (rc) return rc;
@@ -90,6 +90,23 @@ extern "C" int en_padding_removal_layer(const void *hidden_padded, const void *q
     rc = en_attn_fused(pk, pk + (int64_t)D * es, pk + (int64_t)2 * D * es, ctx_packed, seq_lens, nullptr, B, H, S, S, D,
                        in_strides, in_strides, in_strides, out_strides, cu_seqlens, cu_seqlens, scale, causal, dtype,
                        stream);
+    if (rc) return rc;
+  } else if (attention_form >= 3) {
+    // The three kernels on the packed projections: q, k, v are read where the projection left them (batch b at
+    // row cu_seqlens[b], token pitch 3*H*D) and the context is written as packed [T,H,D] rows, so neither
+    // transpose_pad nor transpose_depad runs and no padded tensor exists.  Form 4 also keeps the scores packed.
+    const unsigned char *pk = static_cast<const unsigned char *>(qkv_packed);
+    const void *q = pk, *k = pk + (int64_t)D * es, *v = pk + (int64_t)2 * D * es;
+    const int64_t th = 3 * D, ts = (int64_t)3 * H * D;
+    const int packed_scores = attention_form == 4;
+    rc = en_attn_qk(q, k, scores, seq_lens, nullptr, B, H, S, S, D, 0, th, ts, 0, th, ts, 1.0f, causal, dtype, cu_seqlens,
+                    cu_seqlens, packed_scores, stream);
+    if (rc) return rc;
+    if (packed_scores) rc = en_scale_mask_softmax_packed(scores, seq_lens, B, H, S, scale, dtype, stream);
+    else rc = en_scale_mask_softmax(scores, seq_lens, nullptr, B, H, S, S, scale, causal, 1, dtype, stream);
+    if (rc) return rc;
+    rc = en_attn_pv(scores, v, ctx_packed, seq_lens, nullptr, B, H, S, S, D, 0, th, ts, 0, D, (int64_t)H * D, causal, 0,
+                    dtype, cu_seqlens, cu_seqlens, packed_scores, stream);
     if (rc) return rc;
   } else {
     // the attention entry points never read a row at or past a sequence's length: no zero fill of the padding
@@ -111,12 +128,13 @@ extern "C" int en_padding_removal_layer(const void *hidden_padded, const void *q
       if (rc) return rc;
     } else {
       rc = en_attn_qk(q, k, scores, seq_lens, nullptr, B, H, S, S, D, sb, sh, ss, sb, sh, ss, 1.0f, causal, dtype,
-                      stream);
+                      nullptr, nullptr, 0, stream);
       if (rc) return rc;
       // the PV kernel reads a probability row only as far as its own query sees: no tail is written
       rc = en_scale_mask_softmax(scores, seq_lens, nullptr, B, H, S, S, scale, causal, 1, dtype, stream);
       if (rc) return rc;
-      rc = en_attn_pv(scores, v, ctx, seq_lens, nullptr, B, H, S, S, D, sb, sh, ss, cb, ch, cs, causal, 0, dtype, stream);
+      rc = en_attn_pv(scores, v, ctx, seq_lens, nullptr, B, H, S, S, D, sb, sh, ss, cb, ch, cs, causal, 0, dtype, nullptr,
+                      nullptr, 0, stream);
       if (rc) return rc;
     }
     rc = en_transpose_depad(ctx, ctx_packed, cu_seqlens, B, S, H, D, es, stream);
@@ -136,7 +154,7 @@ extern "C" int en_padding_removal_layer_noalloc(const void *hidden_padded, const
                                                 int fold_depad, int dtype, en_stream_t stream) {
   using namespace en;
   if (!hidden_padded || !qkv_packed || !gamma || !beta || !y || !seq_lens) return EN_ERR_NULL;
-  if (attention_form < 0 || attention_form > 2) return EN_ERR_UNSUPPORTED;
+  if (attention_form < 0 || attention_form > 4) return EN_ERR_UNSUPPORTED;
   const int64_t es = dtype_size(dtype);
   if (!es) return EN_ERR_DTYPE;
   if (batch < 1 || batch > 65536 || max_seq_len < 1 || head_num < 1 || size_per_head < 1 || hidden < 1 ||
@@ -146,10 +164,12 @@ extern "C" int en_padding_removal_layer_noalloc(const void *hidden_padded, const
   const int64_t B = batch, S = max_seq_len, H = head_num, D = size_per_head, T = total_tokens;
   // the same pieces, in the same roles, as the caller-owned buffers of en_padding_removal_layer
   Layout l;
-  const bool padded = attention_form != 2;
+  const bool padded = attention_form < 2;
   const int64_t o_cu = l.take(true, (B + 1) * 4), o_lens = l.take(true, B * 4);
   const int64_t o_offs = l.take(fold_depad != 0, T * 4), o_x = l.take(fold_depad == 0, T * hidden * es);
-  const int64_t o_qkv = l.take(padded, B * H * S * 3 * D * es), o_scores = l.take(attention_form == 0, B * H * S * S * es);
+  const int64_t score_elems = attention_form == 4 ? en_packed_scores_elems(batch, head_num, max_seq_len, dtype) : B * H * S * S;
+  const int64_t o_qkv = l.take(padded, B * H * S * 3 * D * es);
+  const int64_t o_scores = l.take(attention_form == 0 || attention_form >= 3, score_elems * es);
   const int64_t o_ctx = l.take(padded, B * H * S * D * es), o_ctxp = l.take(true, T * H * D * es);
   if (l.used > kLayerScratchBytes) return EN_ERR_SCRATCH;
   unsigned char *base = nullptr;   // the array's address on the current device; never the array's name

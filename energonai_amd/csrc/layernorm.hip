@@ -57,11 +57,11 @@ __global__ __launch_bounds__(TPR < kBlock ? kBlock : TPR) void layernorm_rows_ke
   for (int j = 0; j < VPL; ++j) {
     const int v = t + TPR * j;
     if (v < nvec) {
-      const Pack<TI, EPV> pk = __builtin_bit_cast(Pack<TI, EPV>, load16<false>(in + v * EPV));
+      const Pack<TI, EPV> pk = __builtin_bit_cast(Pack<TI, EPV>, load16<STREAM>(in + v * EPV));
 #pragma unroll
       for (int e = 0; e < EPV; ++e) x[j][e] = EI::to_float(pk.v[e]);
       if (res) {
-        const Pack<TI, EPV> rk = __builtin_bit_cast(Pack<TI, EPV>, load16<false>(res + v * EPV));
+        const Pack<TI, EPV> rk = __builtin_bit_cast(Pack<TI, EPV>, load16<STREAM>(res + v * EPV));
 #pragma unroll
         for (int e = 0; e < EPV; ++e) x[j][e] += EI::to_float(rk.v[e]);
       }

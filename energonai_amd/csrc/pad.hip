@@ -186,10 +186,15 @@ template <> __device__ __forceinline__ uint2 zero_vec<uint2>() { return make_uin
 template <> __device__ __forceinline__ uint32_t zero_vec<uint32_t>() { return 0u; }
 template <> __device__ __forceinline__ uint16_t zero_vec<uint16_t>() { return (uint16_t)0; }
 
-// stores of the mover; the 16-byte path has a non-temporal form for outputs too large to stay cached
+// loads and stores of the mover; the 16-byte path has a non-temporal form for tensors too large to stay cached
+// (a plain copy of 0.5 GB runs at 5.3 TB/s with the default policy, at 6.4 TB/s with non-temporal loads and stores)
 template <typename Vec, bool STREAM> __device__ __forceinline__ void put(Vec *p, const Vec &v) {
   if constexpr (sizeof(Vec) == 16) store16<STREAM>(p, v);
   else *p = v;
+}
+template <typename Vec, bool STREAM> __device__ __forceinline__ Vec get(const Vec *p) {
+  if constexpr (sizeof(Vec) == 16) return load16<STREAM>(p);
+  else return *p;
 }
 
 // One tile of one operation: the first lanes evaluate the map for the tile's rows, then every lane streams
@@ -227,7 +232,7 @@ __device__ __forceinline__ void gather_tile(const Map &map, const Ptrs3 &p, int 
           const int64_t dn = s_dst[r];
           if (dn >= 0) {
             d[u] = dn + c;
-            v[u] = (so >= 0) ? src[so + c] : zero_vec<Vec>();
+            v[u] = (so >= 0) ? get<Vec, STREAM>(src + so + c) : zero_vec<Vec>();
           }
         }
       }

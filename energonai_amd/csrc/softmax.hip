@@ -11,10 +11,6 @@
 
 #include <math.h>
 
-#ifndef EN_SOFTMAX_LPR_A
-#define EN_SOFTMAX_LPR_A 16  // lanes per row for rows of 33..128 vectors
-#endif
-
 namespace en {
 
 struct SoftmaxArgs {
@@ -27,6 +23,7 @@ struct SoftmaxArgs {
   int tail_shift; // < 0: zero the whole tail of a row; s: only up to the extent of its 2^s-row query tile
   int rows_per_batch;  // H * Sq
   float inv_sq;        // 1 / Sq
+  int packed;          // rows are the packed causal prefixes of common.hip.h instead of Sk elements apart
 };
 
 __device__ __forceinline__ int visible_keys(int q, int ql, int kl, int Sk, int causal) {
@@ -69,47 +66,29 @@ __device__ __forceinline__ RowInfo row_info(const SoftmaxArgs &a, int r, int kl,
 // One wave per workgroup: rows differ in length, and a wave that is done frees its slot at once instead of
 // waiting for the longest row among four waves (c3, tile-bounded form: 214 us with 256 threads, 163 us with 64).
 constexpr int kRowsBlock = kWave;
+// a score tensor at least this large is read and written with the non-temporal policy (1.9 GB of scores, 1024-key
+// rows: 157 -> 146 us; on tensors that fit the 256 MB memory-side cache the policy costs time)
+constexpr int64_t kStreamSoftmaxBytes = 512ll << 20;
 
-// LPR lanes share a row, each lane holds VPL vectors of it, and every lane
-// group works on R consecutive rows at once: all R*VPL loads are issued before
-// the first reduction, so one wave keeps R rows of traffic in flight and the
-// R independent reduction chains interleave.
-template <int DT, int VPL, int LPR, int R>
-__global__ __launch_bounds__(kRowsBlock) void softmax_rows_kernel(SoftmaxArgs a) {
+// The work of one lane group: LPR lanes share a row, each lane holds VPL vectors of it, and the group works on
+// R rows at once: all R*VPL loads are issued before the first reduction, so one wave keeps R rows of traffic in
+// flight and the R independent reduction chains interleave.  rowp[i] is row i's first element, ri[i] its
+// geometry, l the lane's index inside its group.  Rows whose write extent lies past the LPR*VPL vectors the
+// registers hold get the rest of their zero tail from a store loop (TAIL_LOOP).
+template <int DT, int VPL, int LPR, int R, bool STREAM, bool TAIL_LOOP>
+__device__ __forceinline__ void softmax_lane_group(const SoftmaxArgs &a, typename Elem<DT>::T *const (&rowp)[R],
+                                                   const RowInfo (&ri)[R], int l) {
   typedef Elem<DT> E;
   typedef typename E::T T;
   constexpr int EPV = 16 / E::kSize;          // elements per 128-bit vector
-  constexpr int GROUPS_PER_WAVE = kWave / LPR;
-  constexpr int GROUPS_PER_BLOCK = GROUPS_PER_WAVE * (kRowsBlock / kWave);
-
-  const int lane = threadIdx.x & (kWave - 1);
-  const int wave = threadIdx.x >> 6;
-  const int sub = lane / LPR;
-  const int l = lane % LPR;
-  const int b = blockIdx.y;
-  const int kl = a.k_lens[b];
-  const int ql = min(a.q_lens ? a.q_lens[b] : min(kl, a.Sq), a.Sq);
-  const int row0 = (blockIdx.x * GROUPS_PER_BLOCK + wave * GROUPS_PER_WAVE + sub) * R;  // inside the batch
-
-  RowInfo ri[R];
-  bool any = false;
-#pragma unroll
-  for (int i = 0; i < R; ++i) {
-    ri[i] = row_info(a, row0 + i, kl, ql);
-    any |= ri[i].active;
-  }
-  if (__ballot(any) == 0ull) return;  // whole wave has nothing to do
-
-  T *base = reinterpret_cast<T *>(a.src) + (int64_t)b * a.rows_per_batch * a.Sk;
   uint4 raw[R][VPL];
 #pragma unroll
   for (int i = 0; i < R; ++i) {
-    const T *rowp = base + (int64_t)(row0 + i) * a.Sk;
 #pragma unroll
     for (int j = 0; j < VPL; ++j) {
       const int e0 = (l + LPR * j) * EPV;
       raw[i][j] = make_uint4(E::kNegInfWord, E::kNegInfWord, E::kNegInfWord, E::kNegInfWord);   // not visible: -inf
-      if (ri[i].active && e0 < ri[i].n) raw[i][j] = load16<false>(rowp + e0);
+      if (ri[i].active && e0 < ri[i].n) raw[i][j] = load16<STREAM>(rowp[i] + e0);
     }
   }
 
@@ -127,7 +106,7 @@ __global__ __launch_bounds__(kRowsBlock) void softmax_rows_kernel(SoftmaxArgs a)
 #pragma unroll
     for (int j = 0; j < VPL; ++j) {
       const int e0 = (l + LPR * j) * EPV;
-      any[j] = __builtin_amdgcn_ballot_w64(e0 < n) != 0ull;
+      any[j] = __builtin_amdgcn_ballot_w64(ri[i].active && e0 < n) != 0ull;
       if (any[j]) {
         const Pack<T, EPV> pk = __builtin_bit_cast(Pack<T, EPV>, raw[i][j]);
 #pragma unroll
@@ -160,7 +139,6 @@ __global__ __launch_bounds__(kRowsBlock) void softmax_rows_kernel(SoftmaxArgs a)
     }
     s = group_allreduce<OpSum, LPR>(s);
     const float inv = s > 0.f ? 1.0f / s : 0.f;
-    T *rowp = base + (int64_t)(row0 + i) * a.Sk;
 #pragma unroll
     for (int j = 0; j < VPL; ++j) {
       const int e0 = (l + LPR * j) * EPV;
@@ -171,9 +149,181 @@ __global__ __launch_bounds__(kRowsBlock) void softmax_rows_kernel(SoftmaxArgs a)
         for (int e = 0; e < EPV; ++e) pk.v[e] = E::from_float(x[j][e] * inv);
         out = __builtin_bit_cast(uint4, pk);
       }
-      if (ri[i].active && e0 < ri[i].lim) store16<false>(rowp + e0, out);
+      if (ri[i].active && e0 < ri[i].lim) store16<STREAM>(rowp[i] + e0, out);
+    }
+    if (TAIL_LOOP && ri[i].active) {
+      for (int e0 = (l + LPR * VPL) * EPV; e0 < ri[i].lim; e0 += LPR * EPV)
+        store16<STREAM>(rowp[i] + e0, make_uint4(0u, 0u, 0u, 0u));
     }
   }
+}
+
+// Rows of up to 64 * 16 vectors, one lane-group shape for the whole launch (chosen from the row length Sk).
+template <int DT, int VPL, int LPR, int R>
+__global__ __launch_bounds__(kRowsBlock) void softmax_rows_kernel(SoftmaxArgs a) {
+  typedef typename Elem<DT>::T T;
+  constexpr int GROUPS_PER_WAVE = kWave / LPR;
+  const int lane = threadIdx.x & (kWave - 1);
+  const int sub = lane / LPR;
+  const int l = lane % LPR;
+  const int b = blockIdx.y;
+  const int kl = a.k_lens[b];
+  const int ql = min(a.q_lens ? a.q_lens[b] : min(kl, a.Sq), a.Sq);
+  const int row0 = (blockIdx.x * GROUPS_PER_WAVE + sub) * R;  // inside the batch
+
+  RowInfo ri[R];
+  T *rowp[R];
+  bool any = false;
+  T *base = reinterpret_cast<T *>(a.src) + (int64_t)b * a.rows_per_batch * a.Sk;
+#pragma unroll
+  for (int i = 0; i < R; ++i) {
+    ri[i] = row_info(a, row0 + i, kl, ql);
+    rowp[i] = base + (int64_t)(row0 + i) * a.Sk;
+    any |= ri[i].active;
+  }
+  if (__ballot(any) == 0ull) return;  // whole wave has nothing to do
+  softmax_lane_group<DT, VPL, LPR, R, false, false>(a, rowp, ri, l);
+}
+
+// ---------------------------------------------------------------------------------------------------------
+// Rows of up to 256 vectors (2048 16-bit or 1024 fp32 keys): the lane-group shape follows each row, not the
+// bucket.  Under a causal mask a row sees from one key to the whole sequence, and sequences are shorter than
+// the bucket; with one shape per launch most lanes of most waves hold nothing, and what a wave keeps in
+// flight -- which is what hides the memory latency -- shrinks with them.  Here every lane holds four vectors and
+// a row is given 4, 8, 16, 32 or 64 lanes by the number of keys it sees, so a wave of 64 lanes works on 16, 8,
+// 4, 2 or 1 rows (times R) and moves about the same number of bytes whichever band its rows are in.
+//
+// The rows of one (batch, head) are cut into bands by what they see; band k holds rows that see more than
+// cap(k-1) and at most cap(k) = 4 * 2^k vectors.  Under a causal mask what a row sees grows by one key per row,
+// so a band is a range of rows; without one every row of a sequence sees the same keys and all of them fall
+// into one band.  A workgroup (one wave) finds its batch's band layout from the two lengths with a few scalar
+// operations, then its head, band and first row from its index; workgroups past the batch's count exit.  Bands
+// are laid out from the longest rows to the shortest, so the heavy waves start first.
+// ---------------------------------------------------------------------------------------------------------
+constexpr int kBandVpl = 4;
+constexpr int kBands = 5;
+
+struct BandLayout {
+  int first[kBands + 1];   // band k holds rows first[k] .. first[k+1]-1 (k = 0: the shortest rows)
+  int blocks[kBands];      // workgroups band k needs per head
+  int total;               // workgroups per head
+};
+
+// cap(k) in elements; the top band takes every longer row as well (rows are at most 256 vectors long here)
+template <int EPV> __host__ __device__ constexpr int band_cap(int k) { return kBandVpl * EPV * (4 << k); }
+
+template <int EPV, int R>
+__device__ __forceinline__ BandLayout band_layout(const SoftmaxArgs &a, int kl, int ql) {
+  BandLayout L;
+  L.first[0] = 0;
+  L.total = 0;
+  const int vis_all = min(max(kl, 0), a.Sk);       // what every row sees without a causal mask
+#pragma unroll
+  for (int k = 0; k < kBands; ++k) {
+    int end;
+    if (k == kBands - 1) end = ql;
+    else if (a.causal) end = min(max(band_cap<EPV>(k) - (kl - ql), 0), ql);   // row q sees q + (kl - ql) + 1 keys
+    else end = vis_all <= band_cap<EPV>(k) ? ql : 0;
+    end = max(end, L.first[k]);
+    L.first[k + 1] = end;
+    const int rows_per_wave = (16 >> k) * R;
+    L.blocks[k] = (end - L.first[k] + rows_per_wave - 1) / rows_per_wave;
+    L.total += L.blocks[k];
+  }
+  return L;
+}
+
+template <int DT, int K, int R, bool STREAM>
+__device__ __forceinline__ void softmax_band_wave(const SoftmaxArgs &a, typename Elem<DT>::T *unit, int q0, int q_end,
+                                                  int kl, int ql, int lane) {
+  typedef typename Elem<DT>::T T;
+  constexpr int LPR = 4 << K;
+  const int sub = lane / LPR, l = lane % LPR;
+  RowInfo ri[R];
+  T *rowp[R];
+#pragma unroll
+  for (int i = 0; i < R; ++i) {
+    const int q = q0 + sub * R + i;
+    ri[i] = RowInfo{false, 0, 0};
+    constexpr int EPV = 16 / Elem<DT>::kSize;
+    if (q < q_end) {
+      ri[i].active = true;
+      ri[i].n = visible_keys(q, ql, kl, a.Sk, a.causal);
+      ri[i].lim = a.Sk;
+      if (a.packed) {           // the row's slot ends with the vector that holds its last visible key
+        ri[i].lim = (q / EPV + 1) * EPV;
+      } else if (a.tail_shift >= 0) {  // the consumer reads a row only up to what the last row of its query tile sees
+        const int q_last = min(((q >> a.tail_shift) + 1) << a.tail_shift, ql) - 1;
+        ri[i].lim = visible_keys(q_last, ql, kl, a.Sk, a.causal);
+      }
+    }
+    rowp[i] = unit + (a.packed ? packed_row_start<EPV>(q) : (int64_t)q * a.Sk);
+  }
+  softmax_lane_group<DT, kBandVpl, LPR, R, STREAM, true>(a, rowp, ri, l);
+}
+
+template <int DT, int R, bool STREAM>
+__global__ __launch_bounds__(kWave) void softmax_bands_kernel(SoftmaxArgs a) {
+  typedef typename Elem<DT>::T T;
+  constexpr int EPV = 16 / Elem<DT>::kSize;
+  // grid (workgroups per head, heads, batches): the workgroups a shorter sequence does not need are spread over
+  // the heads, a few hundred at a time, instead of forming one long run of empty workgroups per batch, during
+  // which the machine would drain
+  const int b = blockIdx.z, h = blockIdx.y;
+  int i = blockIdx.x;
+  const int kl = min(a.k_lens[b], a.Sk);           // a key length past the row length means the whole row
+  const int ql = min(a.q_lens ? a.q_lens[b] : min(kl, a.Sq), a.Sq);
+  if (ql <= 0) return;
+  const BandLayout L = band_layout<EPV, R>(a, kl, ql);
+  if (i >= L.total) return;
+  T *unit = reinterpret_cast<T *>(a.src) +
+            ((int64_t)b * a.H + h) * (a.packed ? packed_row_start<EPV>(a.Sq) : (int64_t)a.Sq * a.Sk);
+  const int lane = threadIdx.x;
+  // longest rows first
+  if (i < L.blocks[4]) return softmax_band_wave<DT, 4, R, STREAM>(a, unit, L.first[4] + i * 1 * R, L.first[5], kl, ql, lane);
+  i -= L.blocks[4];
+  if (i < L.blocks[3]) return softmax_band_wave<DT, 3, R, STREAM>(a, unit, L.first[3] + i * 2 * R, L.first[4], kl, ql, lane);
+  i -= L.blocks[3];
+  if (i < L.blocks[2]) return softmax_band_wave<DT, 2, R, STREAM>(a, unit, L.first[2] + i * 4 * R, L.first[3], kl, ql, lane);
+  i -= L.blocks[2];
+  if (i < L.blocks[1]) return softmax_band_wave<DT, 1, R, STREAM>(a, unit, L.first[1] + i * 8 * R, L.first[2], kl, ql, lane);
+  i -= L.blocks[1];
+  softmax_band_wave<DT, 0, R, STREAM>(a, unit, L.first[0] + i * 16 * R, L.first[1], kl, ql, lane);
+}
+
+// Upper bound, over all lengths a batch may have, of the workgroups one head needs (host side of band_layout).
+template <int EPV, int R>
+static int band_blocks_bound(const SoftmaxArgs &a, bool square_self_attention) {
+  auto rows_per_wave = [](int k) { return (16 >> k) * R; };
+  if (!a.causal) {
+    // all rows of a sequence share one band; the widest band the row length allows needs the most workgroups
+    int k = 0;
+    while (k < kBands - 1 && band_cap<EPV>(k) < a.Sk) ++k;
+    return (int)ceil_div(a.Sq, rows_per_wave(k));
+  }
+  if (square_self_attention) {
+    // row q sees q + 1 keys: band k holds the rows cap(k-1) .. cap(k)-1, the top band whatever is left
+    int total = 0, prev_cap = 0;
+    for (int k = 0; k < kBands; ++k) {
+      const int hi = (k == kBands - 1 || band_cap<EPV>(k) > a.Sq) ? a.Sq : band_cap<EPV>(k);
+      if (hi > prev_cap) total += (int)ceil_div(hi - prev_cap, rows_per_wave(k));
+      prev_cap = hi > prev_cap ? hi : prev_cap;
+    }
+    return total;
+  }
+  // Any shift between query and key positions (chunked prefill, decode): the Sq rows may fall into the bands in
+  // many ways.  Each band takes at most its span of rows (the two outer ones are open-ended), rows in a higher band
+  // need more workgroups, and every band that holds rows at all may end with a partly filled workgroup.
+  int left = a.Sq;
+  double blocks = 0.0;          // the most whole-and-fractional workgroups any split of the rows can need
+  for (int k = kBands - 1; k >= 0 && left > 0; --k) {
+    const int span = (k == 0 || k == kBands - 1) ? a.Sq : band_cap<EPV>(k) - band_cap<EPV>(k - 1);
+    const int rows = span < left ? span : left;
+    blocks += (double)rows / rows_per_wave(k);
+    left -= rows;
+  }
+  const int bands_with_rows = a.Sq < kBands ? a.Sq : kBands;      // no more bands hold rows than there are rows
+  return (int)(blocks + 0.999999) + bands_with_rows - 1;
 }
 
 // Any Sk, any alignment: one workgroup per row, three strided passes.
@@ -211,9 +361,26 @@ __global__ __launch_bounds__(kBlock) void softmax_generic_kernel(SoftmaxArgs a) 
 
 template <int DT, int VPL, int LPR, int R>
 static void launch_rows(const SoftmaxArgs &a, hipStream_t s) {
-  constexpr int ROWS_PER_BLOCK = (kWave / LPR) * (kRowsBlock / kWave) * R;
+  constexpr int ROWS_PER_BLOCK = (kWave / LPR) * R;
   const dim3 grid((unsigned)ceil_div(a.rows_per_batch, ROWS_PER_BLOCK), (unsigned)a.B, 1);
   softmax_rows_kernel<DT, VPL, LPR, R><<<grid, kRowsBlock, 0, s>>>(a);
+}
+
+template <int DT>
+static int launch_bands(const SoftmaxArgs &a, hipStream_t s) {
+  constexpr int EPV = 16 / Elem<DT>::kSize;
+  constexpr int R = 1;   // rows per lane group; two at once were slower on every workload measured
+  const bool square = a.q_lens == nullptr && a.Sq == a.Sk;      // q_len = k_len <= Sk: row q sees q + 1 keys
+  const int64_t blocks = band_blocks_bound<EPV, R>(a, square);
+  if (a.H > 65535 || a.B > 65535) return EN_ERR_SHAPE;
+  const dim3 grid((unsigned)blocks, (unsigned)a.H, (unsigned)a.B);
+  if (blocks > INT32_MAX) return EN_ERR_SHAPE;
+  // a tensor too large to stay in the memory-side cache is read and written with the non-temporal policy
+  const bool stream = (int64_t)a.B * a.rows_per_batch * a.Sk * Elem<DT>::kSize / (a.packed ? 2 : 1) >= kStreamSoftmaxBytes;
+  if (stream) softmax_bands_kernel<DT, R, true><<<grid, kWave, 0, s>>>(a);
+  else softmax_bands_kernel<DT, R, false><<<grid, kWave, 0, s>>>(a);
+  EN_RETURN_IF_LAUNCH_FAILED();
+  return EN_OK;
 }
 
 template <int DT>
@@ -224,13 +391,11 @@ static int dispatch(const SoftmaxArgs &a, hipStream_t s) {
   if (!vec_ok || nvec > 64 * 16 || !(a.scale > 0.f)) {
     softmax_generic_kernel<DT><<<dim3((unsigned)a.rows_per_batch, (unsigned)a.B, 1), kBlock, 0, s>>>(a);
   }
-  // Few lanes per row for short rows: a causal row uses on average half of its sequence, so narrow
-  // lane groups keep more lanes busy and a wave skips the vector steps none of its rows reach.
-  else if (nvec <= 8) launch_rows<DT, 1, 8, 1>(a, s);
-  else if (nvec <= 16) launch_rows<DT, 1, 16, 1>(a, s);
-  else if (nvec <= 32) launch_rows<DT, 2, 16, 1>(a, s);
-  else if (nvec <= 64) launch_rows<DT, 4, EN_SOFTMAX_LPR_A, 1>(a, s);
-  else if (nvec <= 128) launch_rows<DT, 8, EN_SOFTMAX_LPR_A, 1>(a, s);
+  // Rows of up to 128 vectors (1024 16-bit keys): lane groups sized by what each row sees.  Measured against one
+  // shape per launch: 512-key rows 18.7 -> 16.3 us, 1024-key rows 160 -> 142 us; with 2048-key rows the banded form
+  // is slower (144 -> 183 us: two 512-byte pieces per instruction, a row pitch apart, instead of one 1024-byte piece),
+  // so those keep 64 lanes per row.
+  else if (nvec <= 128) return launch_bands<DT>(a, s);
   else if (nvec <= 256) launch_rows<DT, 4, 64, 1>(a, s);
   else if (nvec <= 512) launch_rows<DT, 8, 64, 1>(a, s);
   else launch_rows<DT, 16, 64, 1>(a, s);
@@ -254,11 +419,40 @@ extern "C" int en_scale_mask_softmax(void *src, const int32_t *k_lens, const int
   if (!aligned_to(src, es)) return EN_ERR_ALIGN;
   if (batch > 65535 || (int64_t)head_num * q_seq_len >= (1 << 24)) return EN_ERR_SHAPE;
   SoftmaxArgs a{src, k_lens, q_lens, batch, head_num, q_seq_len, k_seq_len, scale, causal ? 1 : 0, tail_shift,
-                head_num * q_seq_len, 1.0f / (float)q_seq_len};
+                head_num * q_seq_len, 1.0f / (float)q_seq_len, 0};
   hipStream_t s = (hipStream_t)stream;
   switch (dtype) {
     case EN_F32: return dispatch<EN_F32>(a, s);
     case EN_F16: return dispatch<EN_F16>(a, s);
     default: return dispatch<EN_BF16>(a, s);
+  }
+}
+
+extern "C" int64_t en_packed_scores_elems(int batch, int head_num, int seq_len, int dtype) {
+  using namespace en;
+  const int es = dtype_size(dtype);
+  if (!es || batch < 1 || head_num < 1 || seq_len < 1) return 0;
+  const int64_t unit = es == 4 ? packed_row_start<4>(seq_len) : packed_row_start<8>(seq_len);
+  return (int64_t)batch * head_num * unit;
+}
+
+extern "C" int en_scale_mask_softmax_packed(void *scores, const int32_t *seq_lens, int batch, int head_num, int seq_len,
+                                            float scale, int dtype, en_stream_t stream) {
+  using namespace en;
+  if (!scores || !seq_lens) return EN_ERR_NULL;
+  if (batch < 1 || batch > 65535 || head_num < 1 || head_num > 65535 || seq_len < 1) return EN_ERR_SHAPE;
+  const int es = dtype_size(dtype);
+  if (!es) return EN_ERR_DTYPE;
+  if (!aligned_to(scores, 16)) return EN_ERR_ALIGN;
+  if (!(scale > 0.f)) return EN_ERR_UNSUPPORTED;
+  const int epv = 16 / es;
+  if (seq_len > kBandVpl * 64 * epv) return EN_ERR_UNSUPPORTED;     // rows of up to 256 vectors
+  SoftmaxArgs a{scores, seq_lens, nullptr, batch, head_num, seq_len, seq_len, scale, 1, 0,
+                head_num * seq_len, 1.0f / (float)seq_len, 1};
+  hipStream_t s = (hipStream_t)stream;
+  switch (dtype) {
+    case EN_F32: return launch_bands<EN_F32>(a, s);
+    case EN_F16: return launch_bands<EN_F16>(a, s);
+    default: return launch_bands<EN_BF16>(a, s);
   }
 }

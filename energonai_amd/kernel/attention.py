@@ -61,7 +61,7 @@ def attn_qk(q, k, seq_len_list, *, alpha: float = 1.0, causal: bool = True, q_le
     with _lib.device_guard(q):
         _lib.check(_lib.fn.en_attn_qk(q.data_ptr(), k.data_ptr(), out.data_ptr(), k_info.lens.data_ptr(), q_ptr,
                                           B, H, Sq, Sk, D, *qs, *ks, float(alpha), int(bool(causal)),
-                                          _lib.dtype_tag(q, "attn_qk"), _lib.stream_of(q)), "attn_qk")
+                                          _lib.dtype_tag(q, "attn_qk"), None, None, 0, _lib.stream_of(q)), "attn_qk")
     return out
 
 
@@ -90,7 +90,7 @@ def attn_pv(p, v, seq_len_list, *, causal: bool = True, q_len_list=None, zero_pa
     with _lib.device_guard(p):
         _lib.check(_lib.fn.en_attn_pv(p.data_ptr(), v.data_ptr(), out.data_ptr(), k_info.lens.data_ptr(), q_ptr,
                                           B, H, Sq, Sk, D, *vs, *cs, int(bool(causal)), int(bool(zero_padding)),
-                                          _lib.dtype_tag(p, "attn_pv"), _lib.stream_of(p)), "attn_pv")
+                                          _lib.dtype_tag(p, "attn_pv"), None, None, 0, _lib.stream_of(p)), "attn_pv")
     return out
 
 
@@ -162,6 +162,78 @@ def attn_fused_varlen(q, k, v, batch_size: int, max_seq_len: int, seq_len_list, 
                                          int(max_seq_len), D, arr(*qs), arr(*ks), arr(*vs), arr(0, D, H * D), cu, cu,
                                          scale, int(bool(causal)), _lib.dtype_tag(q, "attn_fused_varlen"),
                                          _lib.stream_of(q)), "attn_fused_varlen")
+    return out
+
+
+def packed_scores_elems(batch_size: int, head_num: int, seq_len: int, dtype) -> int:
+    """Elements of the packed causal score tensor of a self-attention batch: per (batch, head) unit the visible
+    prefix of every row, rounded up to one 16-byte vector, back to back; each unit owns the slot of a full-length one."""
+    n = _lib.fn.en_packed_scores_elems(int(batch_size), int(head_num), int(seq_len), _lib._DTYPE_TAG[dtype])
+    if n <= 0:
+        raise RuntimeError("packed_scores_elems: bad arguments")
+    return n
+
+
+def attn_qk_varlen(q, k, batch_size: int, max_seq_len: int, seq_len_list, *, alpha: float = 1.0, causal: bool = True,
+                   packed_scores: bool = False, out: Optional[torch.Tensor] = None):
+    """QK^T of a self-attention batch straight on packed tokens: ``q`` and ``k`` are ``[T,H,D]`` views of the
+    projection output (batch ``b`` at rows ``cu_seqlens[b]`` ..), so no ``transpose_pad`` is needed first.
+    Returns ``[B,H,S,S]`` scores as ``attn_qk`` does, or with ``packed_scores`` (causal, fp16 / bf16) the flat packed
+    tensor of :func:`packed_scores_elems` elements that ``scale_mask_softmax_packed`` and ``attn_pv_varlen`` read."""
+    qs, ks = _thd(q, "q"), _thd(k, "k")
+    T, H, D = q.shape
+    if k.shape != q.shape or k.dtype != q.dtype:
+        raise RuntimeError("attn_qk_varlen: q and k disagree in shape or dtype")
+    B, S = int(batch_size), int(max_seq_len)
+    info = seq_info(seq_len_list, B, q.device)
+    shape = (packed_scores_elems(B, H, S, q.dtype),) if packed_scores else (B, H, S, S)
+    if out is None:
+        out = torch.empty(shape, dtype=q.dtype, device=q.device)
+    elif out.numel() < (shape[0] if packed_scores else B * H * S * S) or out.dtype != q.dtype or not out.is_contiguous():
+        raise RuntimeError("attn_qk_varlen: out is too small, strided or of another dtype")
+    cu = info.cu_seqlens.data_ptr()
+    with _lib.device_guard(q):
+        _lib.check(_lib.fn.en_attn_qk(q.data_ptr(), k.data_ptr(), out.data_ptr(), info.lens.data_ptr(), None, B, H, S, S, D,
+                                      *qs, *ks, float(alpha), int(bool(causal)), _lib.dtype_tag(q, "attn_qk_varlen"), cu, cu,
+                                      int(bool(packed_scores)), _lib.stream_of(q)), "attn_qk_varlen")
+    return out
+
+
+def scale_mask_softmax_packed(batch_size: int, seq_len: int, head_num: int, scores, seq_len_list, *, scale: float = 1.0):
+    """``scale_mask_softmax`` (causal) in place on the packed scores of :func:`attn_qk_varlen`; returns its input."""
+    _lib.require_gpu(scores, "scores")
+    B, S, H = int(batch_size), int(seq_len), int(head_num)
+    if scores.numel() < packed_scores_elems(B, H, S, scores.dtype):
+        raise RuntimeError("scale_mask_softmax_packed: scores is smaller than the packed tensor of this batch")
+    info = seq_info(seq_len_list, B, scores.device)
+    with _lib.device_guard(scores):
+        _lib.check(_lib.fn.en_scale_mask_softmax_packed(scores.data_ptr(), info.lens.data_ptr(), B, H, S, float(scale),
+                                                        _lib.dtype_tag(scores, "scale_mask_softmax_packed"),
+                                                        _lib.stream_of(scores)), "scale_mask_softmax_packed")
+    return scores
+
+
+def attn_pv_varlen(p, v, batch_size: int, max_seq_len: int, seq_len_list, *, causal: bool = True,
+                   packed_scores: bool = False, out: Optional[torch.Tensor] = None):
+    """PV of a self-attention batch with ``v`` a ``[T,H,D]`` view of the packed projection output and the context
+    written as packed ``[1,T,H,D]`` rows (what ``transpose_depad`` would return).  ``p`` is ``[B,H,S,S]`` as left by
+    ``scale_mask_softmax`` or, with ``packed_scores``, the flat tensor left by ``scale_mask_softmax_packed``."""
+    _lib.require_gpu(p, "p")
+    vs = _thd(v, "v")
+    T, H, D = v.shape
+    B, S = int(batch_size), int(max_seq_len)
+    if p.dtype != v.dtype or p.numel() < (packed_scores_elems(B, H, S, v.dtype) if packed_scores else B * H * S * S):
+        raise RuntimeError("attn_pv_varlen: p is too small for this batch or of another dtype than v")
+    info = seq_info(seq_len_list, B, v.device)
+    if out is None:
+        out = torch.empty((1, T, H, D), dtype=v.dtype, device=v.device)
+    elif out.numel() != T * H * D or out.dtype != v.dtype or not out.is_contiguous():
+        raise RuntimeError("attn_pv_varlen: out must be contiguous [1,T,H,D] of v's dtype")
+    cu = info.cu_seqlens.data_ptr()
+    with _lib.device_guard(v):
+        _lib.check(_lib.fn.en_attn_pv(p.data_ptr(), v.data_ptr(), out.data_ptr(), info.lens.data_ptr(), None, B, H, S, S, D,
+                                      *vs, 0, D, H * D, int(bool(causal)), 0, _lib.dtype_tag(v, "attn_pv_varlen"), cu, cu,
+                                      int(bool(packed_scores)), _lib.stream_of(v)), "attn_pv_varlen")
     return out
 
 

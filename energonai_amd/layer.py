@@ -16,9 +16,11 @@ from typing import Dict, Optional
 
 import torch
 
-from .kernel import (attn_fused, attn_fused_packed, attn_pv, attn_qk, decode_pv, decode_qk, depad, layer_norm_forward, scale_mask_softmax,
-                     transpose_depad, transpose_pad)
+from .kernel import (attn_fused, attn_fused_packed, attn_pv, attn_pv_varlen, attn_qk, attn_qk_varlen, decode_pv, decode_qk,
+                     depad, layer_norm_forward, scale_mask_softmax, scale_mask_softmax_packed, transpose_depad,
+                     transpose_pad)
 from . import _lib
+from .kernel.attention import packed_scores_elems
 from .seqinfo import SeqInfo, seq_info
 
 
@@ -30,26 +32,44 @@ def padding_removal_layer(hidden_padded: torch.Tensor, qkv_packed: torch.Tensor,
                           size_per_head: int, gamma: torch.Tensor, beta: torch.Tensor, eps: float = 1e-5,
                           scale: Optional[float] = None, causal: bool = True, left_padded: bool = False,
                           dense_out: Optional[torch.Tensor] = None, sum_seq: Optional[int] = None,
-                          keep: bool = False, fused_attention=False, fold_depad: bool = False,
+                          keep: bool = False, fused_attention=None, fold_depad: Optional[bool] = None,
                           ctx_out: Optional[torch.Tensor] = None):
-    """Runs the seven ops on ``hidden_padded`` [B,S,hid] and ``qkv_packed`` [1,T,H,3D].
+    """Runs the step on ``hidden_padded`` [B,S,hid] and ``qkv_packed`` [1,T,H,3D].
 
-    Returns the normalised ``[1,T,hid]`` output, or a dict of every
-    intermediate when ``keep`` is set.  ``fused_attention=True`` replaces the
-    three ops QK^T / scale_mask_softmax / PV by the single fused kernel (16-bit
-    dtypes only); the score tensor is then never written.
-    ``fused_attention="packed"`` also drops transpose_pad and transpose_depad:
-    the fused kernel reads the packed projections and writes the packed context.
-    ``fold_depad=True`` drops the depad launch as well: the LayerNorm takes its
-    residual rows straight from ``hidden_padded`` (not with ``keep``).
-    ``ctx_out`` (``[1,T,H,D]``, not with ``keep``) receives the packed attention
-    context, which is otherwise a temporary of the call.
+    Returns the normalised ``[1,T,hid]`` output, or a dict of every intermediate when ``keep`` is set.
+    ``fused_attention`` picks how the attention core runs:
+
+    ``False``            the reference's sequence of ops: transpose_pad, QK^T, scale_mask_softmax, PV,
+                         transpose_depad on padded ``[B,H,S,*]`` tensors;
+    ``"varlen"``         QK^T and PV read the packed projections and write the packed context directly
+                         (row offsets): neither transpose runs, no padded tensor exists;
+    ``"varlen_packed"``  the same with the scores in the packed causal layout (causal, 16-bit dtypes);
+    ``True``             QK^T / softmax / PV in the single fused kernel on the padded buffer (16-bit dtypes
+                         only); the score tensor is then never written;
+    ``"packed"``         the fused kernel on the packed projections;
+    ``None`` (default)   ``"varlen_packed"`` where it applies, else ``"varlen"``; with ``keep`` the
+                         reference's sequence, whose intermediates are the ones a caller can name.
+
+    ``fold_depad`` drops the depad launch: the LayerNorm takes its residual rows straight from
+    ``hidden_padded`` (default: on, unless ``keep`` asks for the packed residual).  ``ctx_out``
+    (``[1,T,H,D]``, not with ``keep``) receives the packed attention context, otherwise a temporary.
+    The three-kernel forms compute every score, probability and context entry with the same arithmetic, so
+    their results are bit-identical as long as the softmax gives a row the same lanes in both layouts (rows of
+    up to 1024 keys); beyond that the row sums are added up in another order and the last bit may differ.
     """
     B, S, hid = hidden_padded.shape
     H, D = head_num, size_per_head
     info = seq_info(seq_lens, B, hidden_padded.device)
     T = info.total if sum_seq is None else int(sum_seq)
     scale = float(D) ** -0.5 if scale is None else scale
+    if fused_attention is None:
+        if keep:
+            fused_attention = False
+        else:
+            packable = causal and hidden_padded.dtype != torch.float32 and S <= 2048 and D % 8 == 0 and D <= 128
+            fused_attention = "varlen_packed" if packable else "varlen"
+    if fold_depad is None:
+        fold_depad = not keep
     if not keep:
         return _layer_one_call(hidden_padded, qkv_packed, info, B, S, H, D, hid, T, gamma, beta, eps, scale, causal,
                                left_padded, dense_out, fused_attention, fold_depad, ctx_out)
@@ -57,13 +77,23 @@ def padding_removal_layer(hidden_padded: torch.Tensor, qkv_packed: torch.Tensor,
         raise RuntimeError("padding_removal_layer: fold_depad has no intermediates to keep")
 
     x = depad(hidden_padded, B, info, left_padded=left_padded, sum_seq=T)
-    if fused_attention == "packed":
-        ctx_packed = attn_fused_packed(qkv_packed, B, S, info, H, D, scale=scale, causal=causal)
+    if fused_attention in ("packed", "varlen", "varlen_packed"):
+        probs = None
+        if fused_attention == "packed":
+            ctx_packed = attn_fused_packed(qkv_packed, B, S, info, H, D, scale=scale, causal=causal)
+        else:
+            pk = fused_attention == "varlen_packed"
+            q, k, v = torch.chunk(qkv_packed.view(-1, H, 3 * D), 3, dim=-1)
+            scores = attn_qk_varlen(q, k, B, S, info, causal=causal, packed_scores=pk)
+            if pk:
+                probs = scale_mask_softmax_packed(B, S, H, scores, info, scale=scale)
+            else:
+                probs = scale_mask_softmax(B, S, H, scores, info, scale=scale, causal=causal,
+                                           tail_rows=SOFTMAX_TAIL_ROWS)
+            ctx_packed = attn_pv_varlen(probs, v, B, S, info, causal=causal, packed_scores=pk)
         attn_out = ctx_packed.view(1, T, H * D) if dense_out is None else dense_out
         y = layer_norm_forward(attn_out, gamma, beta, (hid,), eps, residual=x)
-        if keep:
-            return dict(x=x, qkv=None, probs=None, ctx=None, ctx_packed=ctx_packed, y=y)
-        return y
+        return dict(x=x, qkv=None, probs=probs, ctx=None, ctx_packed=ctx_packed, y=y)
     qkv = transpose_pad(qkv_packed, B, S, info, H, 3 * D)
     q, k, v = torch.chunk(qkv, 3, dim=-1)
     if fused_attention:
@@ -76,12 +106,10 @@ def padding_removal_layer(hidden_padded: torch.Tensor, qkv_packed: torch.Tensor,
     ctx_packed = transpose_depad(ctx, B, T, S, info, H, D)
     attn_out = ctx_packed.view(1, T, H * D) if dense_out is None else dense_out
     y = layer_norm_forward(attn_out, gamma, beta, (hid,), eps, residual=x)
-    if keep:
-        return dict(x=x, qkv=qkv, probs=probs, ctx=ctx, ctx_packed=ctx_packed, y=y)
-    return y
+    return dict(x=x, qkv=qkv, probs=probs, ctx=ctx, ctx_packed=ctx_packed, y=y)
 
 
-_FORMS = {False: 0, True: 1, "packed": 2}
+_FORMS = {False: 0, True: 1, "packed": 2, "varlen": 3, "varlen_packed": 4}
 
 
 def _layer_one_call(hidden_padded, qkv_packed, info, B, S, H, D, hid, T, gamma, beta, eps, scale, causal, left_padded,
@@ -101,8 +129,10 @@ def _layer_one_call(hidden_padded, qkv_packed, info, B, S, H, D, hid, T, gamma, 
             raise RuntimeError("padding_removal_layer: dense_out must be [1,T,hidden] of the activation dtype")
     elif hid != H * D:
         raise RuntimeError("padding_removal_layer: without dense_out the LayerNorm width must equal heads * size_per_head")
-    if form and dt == torch.float32:
-        raise RuntimeError("padding_removal_layer: fused attention is for float16 and bfloat16")
+    if form in (1, 2, 4) and dt == torch.float32:
+        raise RuntimeError("padding_removal_layer: the fused kernel and the packed scores are for float16 and bfloat16")
+    if form == 4 and not causal:
+        raise RuntimeError("padding_removal_layer: the packed score layout is that of a causal mask")
     x = None if fold_depad else torch.empty((1, T, hid), dtype=dt, device=dev)
     offs = info.row_offsets(S, left_padded) if fold_depad else None
     y = torch.empty((1, T, hid), dtype=dt, device=dev)
@@ -113,9 +143,13 @@ def _layer_one_call(hidden_padded, qkv_packed, info, B, S, H, D, hid, T, gamma, 
         if ctx_out.numel() != T * H * D or ctx_out.dtype != dt:
             raise RuntimeError("padding_removal_layer: ctx_out must be [1,T,H,D] of the activation dtype")
         ctx_packed = ctx_out
-    qkv = torch.empty((B, H, S, 3 * D), dtype=dt, device=dev) if form != 2 else None
-    ctx = torch.empty((B, H, S, D), dtype=dt, device=dev) if form != 2 else None
-    scores = torch.empty((B, H, S, S), dtype=dt, device=dev) if form == 0 else None
+    qkv = torch.empty((B, H, S, 3 * D), dtype=dt, device=dev) if form < 2 else None
+    ctx = torch.empty((B, H, S, D), dtype=dt, device=dev) if form < 2 else None
+    scores = None
+    if form in (0, 3):
+        scores = torch.empty((B, H, S, S), dtype=dt, device=dev)
+    elif form == 4:
+        scores = torch.empty(packed_scores_elems(B, H, S, dt), dtype=dt, device=dev)
     with _lib.device_guard(hidden_padded):
         _lib.check(_lib.fn.en_padding_removal_layer(
             hidden_padded.data_ptr(), qkv_packed.data_ptr(), _lib.ptr(dense_out), gamma.data_ptr(), beta.data_ptr(),

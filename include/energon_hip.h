@@ -152,6 +152,22 @@ int en_scale_mask_softmax(void *src, const int32_t *k_lens, const int32_t *q_len
                           int q_seq_len, int k_seq_len, float scale, int causal, int tail_rows, int dtype,
                           en_stream_t stream);
 
+/* Packed causal scores.  Under a causal mask of a self-attention batch row q of a (batch, head) unit holds
+ * q + 1 visible scores; in [B,H,S,S] those prefixes start a whole row pitch apart and every kernel of the
+ * chain QK^T -> softmax -> PV streams short ragged pieces of memory.  The packed layout keeps the prefixes only,
+ * each rounded up to one 16-byte vector of V = 16 / element size entries, back to back: row q of a unit starts
+ * V * (V * t * (t + 1) / 2 + (q - V * t) * (t + 1)) elements into it, t = q / V, and holds V * (t + 1) elements;
+ * every unit owns a slot as large as a full-length one (row_start(seq_len) elements), unit (b, h) the slot
+ * b * head_num + h.  en_packed_scores_elems returns the elements of the whole tensor (0 on bad arguments).
+ * An internal format of the step: the reference's [B,H,S,S] tensor (scale_mask_softmax_wrapper.cpp:25-44) stays
+ * the format of en_scale_mask_softmax. */
+int64_t en_packed_scores_elems(int batch, int head_num, int seq_len, int dtype);
+/* en_scale_mask_softmax on packed causal scores, in place: row q < seq_lens[b] becomes softmax(scale * row[:q+1])
+ * with zeros up to the end of its last vector; rows of padded queries do not exist.  seq_len <= 2048 (16-bit)
+ * / 1024 (fp32); scale > 0. */
+int en_scale_mask_softmax_packed(void *scores, const int32_t *seq_lens, int batch, int head_num, int seq_len,
+                                 float scale, int dtype, en_stream_t stream);
+
 /* ---- LayerNorm forward -------------------------------------------------- */
 
 /* forward_affine (csrc/layer_norm_cuda.cpp:82-103, kernel
@@ -178,22 +194,32 @@ int en_layernorm_fwd(void *out, float *mean, float *invvar, void *sum_out, const
  * scores is contiguous [B,H,Sq,Sk].  Only entries softmax will read are
  * written: rows i < q_lens[b], columns j < visible(i) rounded up to 16 bytes;
  * everything else in scores is left untouched.  q_lens NULL as above.
- * fp32 accumulation on MFMA; D a multiple of 8 (16-bit) / 4 (fp32), D <= 128. */
+ * fp32 accumulation on MFMA; D a multiple of 8 (16-bit) / 4 (fp32), D <= 128.
+ * q_row_offsets / k_row_offsets (device, batch entries, or NULL): q / k hold the valid rows of all sequences
+ * back to back (the [1,T,H,3D] projection output of examples/bert/bert.py:100) and batch b starts at that row
+ * (give stride_b = 0, stride_s = the token pitch): the contraction then needs no transpose_pad before it.
+ * packed_scores != 0 (causal self-attention only: q_lens NULL, q_seq_len == k_seq_len; 16-bit dtypes): scores
+ * are written in the packed layout of en_packed_scores_elems instead of [B,H,Sq,Sk]. */
 int en_attn_qk(const void *q, const void *k, void *scores, const int32_t *k_lens, const int32_t *q_lens, int batch,
                int head_num, int q_seq_len, int k_seq_len, int size_per_head, int64_t q_stride_b,
                int64_t q_stride_h, int64_t q_stride_s, int64_t k_stride_b, int64_t k_stride_h, int64_t k_stride_s,
-               float alpha, int causal, int dtype, en_stream_t stream);
+               float alpha, int causal, int dtype, const int32_t *q_row_offsets, const int32_t *k_row_offsets,
+               int packed_scores, en_stream_t stream);
 
 /* ctx[b,h,i,:] = sum_j p[b,h,i,j] * v[b,h,j,:]  (examples/bert/bert.py:119,
  * examples/gpt/gpt.py:125) over j < visible(i) only; p contiguous [B,H,Sq,Sk]
  * as left by en_scale_mask_softmax (any tail_rows: of row i only the 16-byte
  * vectors that hold a visible entry are read), v strided like k above, ctx
  * addressed with its own strides.  Rows i >= q_lens[b] of ctx are written as zero when
- * zero_padding != 0 and left untouched otherwise. */
+ * zero_padding != 0 and left untouched otherwise.
+ * c_row_offsets / v_row_offsets as q_row_offsets / k_row_offsets of en_attn_qk: with c_row_offsets the context is
+ * written as packed [T,H,D] rows (strides 0, D, H*D), which is what transpose_depad would produce
+ * (zero_padding must then be 0: a packed tensor has no padding rows).  packed_scores as in en_attn_qk. */
 int en_attn_pv(const void *p, const void *v, void *ctx, const int32_t *k_lens, const int32_t *q_lens, int batch,
                int head_num, int q_seq_len, int k_seq_len, int size_per_head, int64_t v_stride_b,
                int64_t v_stride_h, int64_t v_stride_s, int64_t c_stride_b, int64_t c_stride_h, int64_t c_stride_s,
-               int causal, int zero_padding, int dtype, en_stream_t stream);
+               int causal, int zero_padding, int dtype, const int32_t *c_row_offsets, const int32_t *v_row_offsets,
+               int packed_scores, en_stream_t stream);
 
 /* Single-query forms of the two contractions for cached decode (one new token
  * per sequence against a ragged cache; the reference recomputes the whole
@@ -252,7 +278,10 @@ int en_attn_fused(const void *q, const void *k, const void *v, void *ctx, const 
  * the LayerNorm adds to x_packed instead of ctx_packed (the output projection lies between
  * the two in a real layer).  attention_form: 0 = the three separate ops, 1 = en_attn_fused
  * on the padded buffer (scores unused), 2 = en_attn_fused on the packed projections
- * (qkv_padded, scores and ctx unused).  fold_depad_offsets (en_padding_offsets of this
+ * (qkv_padded, scores and ctx unused), 3 = the three separate ops on the packed projections
+ * (row offsets into qkv_packed and ctx_packed: transpose_pad and transpose_depad do not run;
+ * qkv_padded and ctx unused), 4 = form 3 with the scores in the packed causal layout
+ * (causal, 16-bit dtypes; scores needs en_packed_scores_elems elements).  fold_depad_offsets (en_padding_offsets of this
  * batch, or NULL): if given, depad is not run and x_packed may be NULL; the LayerNorm takes
  * its residual rows straight from hidden_padded.  gamma/beta in the activation dtype. */
 int en_padding_removal_layer(const void *hidden_padded, const void *qkv_packed, const void *dense_out,
@@ -273,7 +302,8 @@ int en_padding_removal_layer(const void *hidden_padded, const void *qkv_packed, 
  *   always                 (B+1)*4 + B*4 + T*H*D*e
  *   fold_depad != 0        + T*4                     else  + T*hidden*e
  *   attention_form 0 or 1  + B*H*S*3D*e + B*H*S*D*e
- *   attention_form 0       + B*H*S*S*e
+ *   attention_form 0 or 3  + B*H*S*S*e
+ *   attention_form 4       + en_packed_scores_elems(B, H, S, dtype)*e
  * A call that needs more returns EN_ERR_SCRATCH before anything is launched.  Arguments otherwise as
  * en_padding_removal_layer (fold_depad != 0 stands for passing fold_depad_offsets).  No hipMalloc, hipFree
  * or other allocating call is made; the first call on a device looks up the array's address

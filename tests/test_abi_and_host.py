@@ -75,7 +75,14 @@ def test_entry_points_validate_before_launch():
     assert lib.en_layernorm_fwd(16, None, None, None, 32, None, None, 48, 64, 1, 8, 1e-5, 1, 0, None) == -3  # (f16 -> f32)
     assert lib.en_layernorm_fwd(16, None, None, None, 32, None, 80, 48, 64, 1, 8, 1e-5, 1, 1, None) == -1   # offsets, no residual
     assert lib.en_padding_offsets(16, 0, 8, 0, 32, None) == -2           # batch 0
-    assert lib.en_attn_qk(16, 32, 48, 64, None, 1, 1, 8, 8, 200, 0, 0, 200, 0, 0, 200, 1.0, 1, 1, None) == -5  # D > 128
+    assert lib.en_attn_qk(16, 32, 48, 64, None, 1, 1, 8, 8, 200, 0, 0, 200, 0, 0, 200, 1.0, 1, 1, None, None, 0,
+                          None) == -5                                    # D > 128
+    assert lib.en_attn_qk(16, 32, 48, 64, None, 1, 1, 8, 8, 64, 0, 0, 64, 0, 0, 64, 1.0, 0, 1, None, None, 1,
+                          None) == -5                                    # packed scores are those of a causal mask
+    assert lib.en_attn_pv(16, 32, 48, 64, None, 1, 1, 8, 8, 64, 0, 0, 64, 0, 0, 64, 1, 1, 1, 80, None, 0,
+                          None) == -5                                    # a packed context has no padding rows to zero
+    assert lib.en_packed_scores_elems(2, 3, 16, 1) == 2 * 3 * (64 + 128) and lib.en_packed_scores_elems(0, 3, 16, 1) == 0
+    assert lib.en_scale_mask_softmax_packed(16, 32, 1, 1, 4096, 1.0, 1, None) == -5     # rows of more than 256 vectors
     assert lib.en_copy_bytes(16, 32, 24, None) == -2                     # not a multiple of 16
     # entry points added beside the reference's own surface
     i64x3 = (ctypes.c_int64 * 3)(0, 64, 768)
@@ -91,7 +98,7 @@ def test_entry_points_validate_before_launch():
     assert lib.en_attn_fused(16, 32, 48, 64, 80, None, 1, 1, 8, 8, 200, i64x3, i64x3, i64x3, i64x3, None, None, 1.0, 1, 1,
                              None) == -5                                 # head size above 128
     assert lib.en_padding_removal_layer(16, 32, None, 48, 64, 80, 96, 112, 128, 144, 160, 176, 192, 1, 8, 2, 8, 16, 4,
-                                        1.0, 1e-5, 1, 0, 3, None, 1, None) == -5   # unknown attention form
+                                        1.0, 1e-5, 1, 0, 5, None, 1, None) == -5   # unknown attention form
     assert lib.en_padding_removal_layer(16, 32, None, 48, 64, 80, 96, 112, 128, 144, 160, 176, 192, 1, 8, 2, 8, 32, 4,
                                         1.0, 1e-5, 1, 0, 0, None, 1, None) == -2   # LayerNorm width 32 != 2 heads x 8, no dense_out
     assert lib.en_padding_removal_layer(16, 32, None, 48, 64, 80, None, 112, 128, 144, 160, 176, 192, 1, 8, 2, 8, 16, 4,

@@ -426,3 +426,87 @@ def test_attention_rows_past_the_register_limit(dtype, S, tail_rows):
                                       out_dtype=torch.float32)
         want = eager.attn_pv(pr, v[b:b + 1, :, :n], torch.float32)
         assert max_abs(ctx[b:b + 1, :, :n], want) <= tol * max(1.0, float(want.abs().max()))
+
+
+VARLEN_CASES = [
+    # B, H, S, D, lens
+    (8, 12, 128, 64, [24, 127, 31, 65, 24, 127, 31, 65]),
+    (3, 2, 200, 64, [200, 0, 77]),
+    (2, 3, 256, 128, [256, 129]),
+    (1, 2, 520, 80, [515]),
+    (9, 1, 136, 128, [130, 5, 64, 65, 127, 128, 129, 1, 33]),
+    (2, 2, 2048, 128, [2048, 700]),
+]
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("causal", [True, False])
+@pytest.mark.parametrize("B,H,S,D,lens", VARLEN_CASES)
+def test_contractions_on_packed_tokens_match_the_padded_route(dtype, causal, B, H, S, D, lens):
+    """attn_qk_varlen / attn_pv_varlen read q, k, v where the projection left them ([T,H,3D], batch b at row
+    cu_seqlens[b]) and write the packed context: bit for bit what transpose_pad -> attn_qk -> softmax -> attn_pv ->
+    transpose_depad give.  With packed_scores (causal, 16-bit) the score tensor holds each row's visible prefix
+    only, the same bits as the padded tensor's prefix."""
+    k = _kernel()
+    announce("attn varlen", dtype, causal, B, H, S, D, lens)
+    T = sum(lens)
+    qkv_packed = packed_randn(T, H * 3 * D, dtype, 900 + S).reshape(T, H, 3 * D)
+    lens_t = torch.tensor(lens, dtype=torch.int32).cuda()
+    qkv_g = qkv_packed.cuda()
+    scale = D ** -0.5
+    padded = k.transpose_pad(qkv_g.reshape(1, T, H, 3 * D), B, S, lens_t, H, 3 * D)
+    qp, kp, vp = torch.chunk(padded, 3, dim=-1)
+    s_pad = k.attn_qk(qp, kp, lens_t, causal=causal)
+    scores_raw = s_pad.clone()
+    p_pad = k.scale_mask_softmax(B, S, H, s_pad, lens_t, scale=scale, causal=causal, tail_rows=1)
+    want = k.transpose_depad(k.attn_pv(p_pad, vp, lens_t, causal=causal), B, T, S, lens_t, H, D)
+
+    q, kk, v = torch.chunk(qkv_g, 3, dim=-1)
+    s_var = k.attn_qk_varlen(q, kk, B, S, lens_t, causal=causal)
+    for b, n in enumerate(lens):
+        for qi in (0, n // 2, n - 1):
+            if 0 <= qi < n:
+                vis = (qi + 1) if causal else n
+                assert torch.equal(s_var[b, :, qi, :vis], scores_raw[b, :, qi, :vis])
+    p_var = k.scale_mask_softmax(B, S, H, s_var, lens_t, scale=scale, causal=causal, tail_rows=1)
+    sentinel = torch.full((1, T + 1, H, D), 9.0, dtype=dtype, device="cuda")
+    got = k.attn_pv_varlen(p_var, v, B, S, lens_t, causal=causal, out=sentinel[:, :T])
+    assert torch.equal(got, want)
+    assert bool((sentinel[:, T] == 9.0).all())          # nothing is written past the last token
+    if causal and dtype != torch.float32:
+        epv = 8
+        flat = k.attn_qk_varlen(q, kk, B, S, lens_t, causal=True, packed_scores=True)
+        assert flat.numel() == k.packed_scores_elems(B, H, S, dtype)
+
+        def row_start(r):
+            t = r // epv
+            return epv * (epv * t * (t + 1) // 2 + (r - epv * t) * (t + 1))
+        unit = row_start(S)
+        for b, n in enumerate(lens):
+            for qi in (0, n // 2, n - 1):
+                if 0 <= qi < n:
+                    for h in (0, H - 1):
+                        o = (b * H + h) * unit + row_start(qi)
+                        assert torch.equal(flat[o:o + qi + 1], scores_raw[b, h, qi, :qi + 1])
+        probs = k.scale_mask_softmax_packed(B, S, H, flat, lens_t, scale=scale)
+        assert probs.data_ptr() == flat.data_ptr()
+        for b, n in enumerate(lens):
+            for qi in (0, n // 2, n - 1):
+                if 0 <= qi < n:
+                    o = (b * H + (H - 1)) * unit + row_start(qi)
+                    if S <= 1024:
+                        assert torch.equal(probs[o:o + qi + 1], p_pad[b, H - 1, qi, :qi + 1])
+                    else:
+                        assert max_abs(probs[o:o + qi + 1], p_pad[b, H - 1, qi, :qi + 1]) <= 2.0 ** -11
+                    assert not probs[o + qi + 1:o + (qi // epv + 1) * epv].any()
+        got_p = k.attn_pv_varlen(probs, v, B, S, lens_t, causal=True, packed_scores=True)
+        if S <= 1024:
+            assert torch.equal(got_p, want)
+        else:
+            # rows of more than 1024 keys: the softmax on [B,H,S,S] gives every row 64 lanes, the one on packed
+            # scores sizes the lane group by the row, so the row sums are added up in another order and a
+            # probability may differ in its last bit
+            assert max_abs(got_p, want) <= 2.0 ** -10 * max(1.0, float(want.abs().max()))
+    elif dtype == torch.float32 or not causal:
+        with pytest.raises(RuntimeError):
+            k.attn_qk_varlen(q, kk, B, S, lens_t, causal=causal, packed_scores=True)

@@ -188,10 +188,15 @@ def test_layer_large_fp16_one_call_path_against_the_oracle(name, total):
             inp["beta"].cuda(), 1e-5, w.scale, w.causal, w.left_padded)
     ctx = torch.full((1, T, H, D), float("nan"), dtype=w.dtype, device="cuda")
     y = layer.padding_removal_layer(*args, dense_out=dense, sum_seq=T, ctx_out=ctx)
-    steps = layer.padding_removal_layer(*args, dense_out=dense, sum_seq=T, keep=True)
+    # the same form, op by op through the public functions
+    steps = layer.padding_removal_layer(*args, dense_out=dense, sum_seq=T, keep=True, fused_attention="varlen_packed")
     assert torch.equal(y, steps["y"]) and torch.equal(ctx, steps["ctx_packed"])
-    del steps
-    y, ctx = y.cpu(), ctx.cpu()
+    # the reference's sequence of ops (transpose_pad ... transpose_depad on padded tensors), also checked below
+    ref = layer.padding_removal_layer(*args, dense_out=dense, sum_seq=T, keep=True, fused_attention=False)
+    if w.seq <= 1024:       # same softmax lane grouping in both: the same bits
+        assert torch.equal(y, ref["y"]) and torch.equal(ctx, ref["ctx_packed"])
+    routes = [("one call", y.cpu(), ctx.cpu()), ("reference sequence", ref["y"].cpu(), ref["ctx_packed"].cpu())]
+    del steps, ref
     order = sorted(range(B), key=lambda b: lens_l[b])
     cu = [0]
     for n in lens_l:
@@ -204,10 +209,13 @@ def test_layer_large_fp16_one_call_path_against_the_oracle(name, total):
         want = eager.layer_unpadded(inp["hidden_padded"][b:b + 1], inp["qkv_packed"][:, sl], [n], H, D, inp["gamma"],
                                     inp["beta"], 1e-5, w.scale, w.causal, w.left_padded, dense_out=sub_dense,
                                     acc_dtype=torch.float32, storage_dtype=torch.float16)
-        assert_stored_close(ctx[0, sl].reshape(n, H * D), want["ctx_packed"].reshape(n, H * D), w.dtype, what="context")
         # the LayerNorm passes the error of its input on, scaled by gamma * invvar, and rounds once more
         amp = max(1.0, float(want["invvar"].max()) * float(inp["gamma"].float().abs().max())) if dense is None else 0.0
-        assert_stored_close(y[0, sl], want["y"][0], w.dtype, base=BASE[w.dtype] * max(amp, 1.0), what="LayerNorm output")
+        for route, y_r, ctx_r in routes:
+            assert_stored_close(ctx_r[0, sl].reshape(n, H * D), want["ctx_packed"].reshape(n, H * D), w.dtype,
+                                what=f"context, {route}")
+            assert_stored_close(y_r[0, sl], want["y"][0], w.dtype, base=BASE[w.dtype] * max(amp, 1.0),
+                                what=f"LayerNorm output, {route}")
 
 
 def test_decode_layer_c5_reduced_and_full():
@@ -258,7 +266,8 @@ def test_layer_c2_fused_attention(mode):
     assert_stored_close(got["y"].cpu(), want["y"], w.dtype, what="LayerNorm output")
 
 
-@pytest.mark.parametrize("name,form", [("c1", False), ("c2", False), ("c2", True), ("c2", "packed")])
+@pytest.mark.parametrize("name,form", [("c1", False), ("c1", "varlen"), ("c2", False), ("c2", True), ("c2", "packed"),
+                                       ("c2", "varlen"), ("c2", "varlen_packed"), ("c2", None)])
 def test_layer_single_call_equals_the_op_by_op_sequence(name, form):
     """padding_removal_layer without keep= goes through the one-call entry point of the library; it must give
     bit for bit what the same ops give when called one by one."""
@@ -275,9 +284,13 @@ def test_layer_single_call_equals_the_op_by_op_sequence(name, form):
     assert torch.equal(once, steps["y"])
     twice = layer.padding_removal_layer(*args, dense_out=dense, fused_attention=form, sum_seq=int(inp["lens"].sum()))
     assert torch.equal(twice, once)
+    if form in ("varlen", "varlen_packed", None):
+        # the contractions on packed tokens compute what the reference's sequence of ops computes, bit for bit
+        ref = layer.padding_removal_layer(*args, dense_out=dense, keep=True, fused_attention=False)
+        assert torch.equal(once, ref["y"]) and torch.equal(steps["ctx_packed"], ref["ctx_packed"])
 
 
-@pytest.mark.parametrize("name,form", [("c1", False), ("c2", False), ("c2", "packed")])
+@pytest.mark.parametrize("name,form", [("c1", False), ("c2", False), ("c2", "packed"), ("c2", "varlen_packed")])
 def test_layer_with_depad_folded_into_layernorm(name, form):
     """fold_depad: no depad launch, the LayerNorm reads its residual rows from the padded activations through
     per-token row offsets (right-padded c1, left-padded c2).  Same bits as the step with the depad copy."""
@@ -289,12 +302,12 @@ def test_layer_with_depad_folded_into_layernorm(name, form):
             inp["gamma"].cuda(), inp["beta"].cuda(), 1e-5, w.scale, w.causal, w.left_padded)
     dense = inp.get("dense_out")
     dense = None if dense is None else dense.cuda()
-    plain = layer.padding_removal_layer(*args, dense_out=dense, fused_attention=form)
+    plain = layer.padding_removal_layer(*args, dense_out=dense, fused_attention=form, fold_depad=False)
     folded = layer.padding_removal_layer(*args, dense_out=dense, fused_attention=form, fold_depad=True)
     assert torch.equal(folded, plain)
 
 
-@pytest.mark.parametrize("name,form", [("c1", False), ("c2", False), ("c2", "packed")])
+@pytest.mark.parametrize("name,form", [("c1", False), ("c2", False), ("c2", "packed"), ("c1", None), ("c2", None)])
 def test_layer_recorded_into_a_hip_graph_replays_the_eager_result(name, form):
     """The step allocates through torch only and never synchronises, so a caller may record it into a HIP graph.
     Each of three replays, with eager launches and synchronisations between them, must give the eager bits, and

@@ -237,12 +237,15 @@ def test_layer_random_shapes(seed):
     # between attention and LayerNorm), and adds its own fp32 arithmetic and one rounding
     amp = 0.0 if wide else float(want["invvar"].max()) * float(gamma.float().abs().max())
     base_y = base_c * amp + 1e-5 * max(1.0, float(want["y"].abs().max()))
-    forms = [(False, False), (False, True)]
+    forms = [(False, False), (False, True), ("varlen", False), ("varlen", True), (None, None)]
     if dtype != torch.float32:
         forms += [(True, False), ("packed", False), ("packed", True)]
+        if causal:
+            forms += [("varlen_packed", False), ("varlen_packed", True)]
     for form, fold in forms:
         y = layer.padding_removal_layer(*args, dense_out=dense_g, fused_attention=form, fold_depad=fold)
         assert y.shape == (1, T, hid)
-        assert_stored_close(y.cpu(), (want if form else want_r)["y"], dtype, base=base_y, what=f"y {form} {fold}")
-        if not form:
+        three_kernels = form in (False, None, "varlen", "varlen_packed")
+        assert_stored_close(y.cpu(), (want_r if three_kernels else want)["y"], dtype, base=base_y, what=f"y {form} {fold}")
+        if three_kernels:
             assert torch.equal(y, kept["y"]), (form, fold)      # the one-call step gives the op-by-op bits

@@ -14,6 +14,9 @@ pytestmark = pytest.mark.gpu
 # (workload the shape is cut from, dtype, form, fold_depad, lens of the first call, lens of the second)
 CASES = [
     ("c2", torch.float16, "packed", True, [512, 64, 301, 97, 200, 511], [130, 33]),
+    ("c2", torch.float16, "varlen_packed", True, [512, 64, 301, 97, 200, 511], [130, 33]),
+    ("c2", torch.bfloat16, "varlen", False, [256, 64, 201], [97, 5]),
+    ("c1", torch.float32, "varlen", True, [128, 16, 77, 100], [25, 119]),
     ("c2", torch.float16, False, False, [256, 64, 201], [97, 5]),
     ("c2", torch.bfloat16, True, False, [300, 17, 128], [64]),
     ("c1", torch.float32, False, False, [128, 16, 77, 100], [25, 119]),
@@ -73,7 +76,7 @@ def test_noalloc_layer_refuses_what_does_not_fit():
     with pytest.raises(RuntimeError, match="static scratch"):
         layer.padding_removal_layer_noalloc(d["hidden_padded"], d["qkv_packed"], d["lens"].cuda(), w.heads, w.head_dim,
                                             d["gamma"], d["beta"], out, T, workloads.EPS, w.scale, w.causal,
-                                            w.left_padded)
+                                            w.left_padded, fused_attention=False)
     torch.cuda.synchronize()
     assert not out.any()                   # nothing was launched
     # the same batch fits when the scores never exist and no padded tensor is built
