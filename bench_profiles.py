@@ -33,7 +33,7 @@ KERNEL_KEYS = [
     ("DepadHeadsMap", "transpose_depad"),
     ("PadMap", "transpose_pad_valid_rows"),
     ("attn_qk", "attn_qk"),
-    ("softmax", "scale_mask_softmax_no_tail"),
+    ("softmax", "scale_mask_softmax"),
     ("attn_pv", "attn_pv"),
     ("layernorm", "layernorm_residual"),
     ("decode_qk", "decode_qk"),
@@ -41,14 +41,11 @@ KERNEL_KEYS = [
     ("attn_fused", "attn_fused"),
     ("copy_kernel", "copy"),
 ]
-# in the decode step the softmax keeps its full name in the bench line
-DECODE_KEYS = {"scale_mask_softmax_no_tail": "scale_mask_softmax"}
-
 
 def key_of(kernel: str, decode: bool):
     for sub, key in KERNEL_KEYS:
         if sub in kernel:
-            return DECODE_KEYS.get(key, key) if decode else key
+            return key
     return None
 
 
@@ -102,7 +99,7 @@ def cmd_trace(ns) -> int:
     d, line, shown = run_profiler(f"kt_{ns.workload}", ["--kernel-trace", "--stats"], bench_args, ns.timeout)
     agg = trace_rows(find_csv(d, "kernel_trace.csv"))
     decode = ns.workload == "c5"
-    kt = (line or {}).get("kernels", {})
+    kt = (line or {}).get("step_kernels", {})
     print(f"# rocprofv3 kernel-trace summary: `bench.py --workload {ns.workload} --step-only`\n")
     print("Command (MI355X box, repo root; the summary below is this command's stdout):\n")
     print(f"```\npython3 bench_profiles.py trace --workload {ns.workload}\n  -> {shown}\n```\n")
@@ -140,7 +137,7 @@ def cmd_traffic(ns) -> int:
         vals = [v for n, vs in rows.items() if "copy_kernel" in n for v in vs]
         # the copy kernel moves 64 MiB, 256 MiB and 1 GiB each way; the largest launches dominate the maximum
         calib[counter] = (1 << 30) / max(vals)      # bytes per counter unit
-    alg = {k: v["alg_MB"] * 1e6 for k, v in (line or {}).get("kernels", {}).items()}
+    alg = {k: v["alg_MB"] * 1e6 for k, v in (line or {}).get("step_kernels", {}).items()}
     # every op of the step is launched the same number of times in a --step-only run
     keys = collections.defaultdict(lambda: {"FETCH_SIZE": 0.0, "WRITE_SIZE": 0.0, "names": set(), "n": 0})
     for counter, rows in per_counter.items():

@@ -73,6 +73,10 @@ __device__ __forceinline__ void store_pack(T *p, const Pack<T, N> &x) { *reinter
 // consumer kernel anyway, so they are written with non-temporal stores (measured:
 // +10..25 % on such tensors, -5 % when applied to small, cache-resident ones).
 constexpr int64_t kStreamStoreBytes = 96ll << 20;
+// Inputs are read with non-temporal loads only when the tensor moved is larger than the memory-side cache: a
+// smaller one has often just been written by the kernel before and is served from that cache, and the policy then
+// costs time (133 MB rows: depad 39 -> 47 us, LayerNorm 60 -> 72 us; 495 MB: 181 -> 175 us, 274 -> 268 us).
+constexpr int64_t kStreamLoadBytes = 384ll << 20;
 
 // 128-bit global accesses, optionally non-temporal (streamed once: do not keep in cache).
 typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));

@@ -28,7 +28,7 @@ struct LnArgs {
   float eps;
 };
 
-template <int DTI, int DTO, int VPL, int TPR, bool STREAM>
+template <int DTI, int DTO, int VPL, int TPR, bool STREAM, bool STREAM_LD = false>
 __global__ __launch_bounds__(TPR < kBlock ? kBlock : TPR) void layernorm_rows_kernel(LnArgs a) {
   typedef Elem<DTI> EI;
   typedef Elem<DTO> EO;
@@ -57,11 +57,11 @@ __global__ __launch_bounds__(TPR < kBlock ? kBlock : TPR) void layernorm_rows_ke
   for (int j = 0; j < VPL; ++j) {
     const int v = t + TPR * j;
     if (v < nvec) {
-      const Pack<TI, EPV> pk = __builtin_bit_cast(Pack<TI, EPV>, load16<STREAM>(in + v * EPV));
+      const Pack<TI, EPV> pk = __builtin_bit_cast(Pack<TI, EPV>, load16<STREAM_LD>(in + v * EPV));
 #pragma unroll
       for (int e = 0; e < EPV; ++e) x[j][e] = EI::to_float(pk.v[e]);
       if (res) {
-        const Pack<TI, EPV> rk = __builtin_bit_cast(Pack<TI, EPV>, load16<STREAM>(res + v * EPV));
+        const Pack<TI, EPV> rk = __builtin_bit_cast(Pack<TI, EPV>, load16<STREAM_LD>(res + v * EPV));
 #pragma unroll
         for (int e = 0; e < EPV; ++e) x[j][e] += EI::to_float(rk.v[e]);
       }
@@ -169,7 +169,10 @@ static void launch_rows(const LnArgs &a, hipStream_t s) {
   constexpr int ROWS_PER_BLOCK = BLOCK / TPR;
   const unsigned grid = (unsigned)ceil_div(a.n1, ROWS_PER_BLOCK);
   // outputs too large to stay in the memory-side cache are written with non-temporal stores
-  if (a.n1 * a.n2 * Elem<DTO>::kSize >= kStreamStoreBytes) layernorm_rows_kernel<DTI, DTO, VPL, TPR, true><<<grid, BLOCK, 0, s>>>(a);
+  // and inputs too large to have stayed there are read with non-temporal loads
+  const int64_t bytes = a.n1 * a.n2 * Elem<DTO>::kSize;
+  if (bytes >= kStreamLoadBytes) layernorm_rows_kernel<DTI, DTO, VPL, TPR, true, true><<<grid, BLOCK, 0, s>>>(a);
+  else if (bytes >= kStreamStoreBytes) layernorm_rows_kernel<DTI, DTO, VPL, TPR, true><<<grid, BLOCK, 0, s>>>(a);
   else layernorm_rows_kernel<DTI, DTO, VPL, TPR, false><<<grid, BLOCK, 0, s>>>(a);
 }
 

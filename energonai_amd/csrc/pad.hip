@@ -199,7 +199,7 @@ template <typename Vec, bool STREAM> __device__ __forceinline__ Vec get(const Ve
 
 // One tile of one operation: the first lanes evaluate the map for the tile's rows, then every lane streams
 // 4 x 128-bit loads followed by 4 x 128-bit stores per step, for each of the NT tensors that share the map.
-template <typename Vec, typename Map, int NT, bool STREAM>
+template <typename Vec, typename Map, int NT, bool STREAM, bool STREAM_LD = false>
 __device__ __forceinline__ void gather_tile(const Map &map, const Ptrs3 &p, int vpr, int rows_per_block, int tx, int ty) {
   __shared__ int64_t s_src[kMaxTileRows];
   __shared__ int64_t s_dst[kMaxTileRows];
@@ -232,7 +232,7 @@ __device__ __forceinline__ void gather_tile(const Map &map, const Ptrs3 &p, int 
           const int64_t dn = s_dst[r];
           if (dn >= 0) {
             d[u] = dn + c;
-            v[u] = (so >= 0) ? get<Vec, STREAM>(src + so + c) : zero_vec<Vec>();
+            v[u] = (so >= 0) ? get<Vec, STREAM_LD>(src + so + c) : zero_vec<Vec>();
           }
         }
       }
@@ -243,9 +243,9 @@ __device__ __forceinline__ void gather_tile(const Map &map, const Ptrs3 &p, int 
   }
 }
 
-template <typename Vec, typename Map, int NT, bool STREAM>
+template <typename Vec, typename Map, int NT, bool STREAM, bool STREAM_LD = false>
 __global__ __launch_bounds__(kBlock) void row_gather_kernel(Map map, Ptrs3 p, int vpr, int rows_per_block) {
-  gather_tile<Vec, Map, NT, STREAM>(map, p, vpr, rows_per_block, blockIdx.x, blockIdx.y);
+  gather_tile<Vec, Map, NT, STREAM, STREAM_LD>(map, p, vpr, rows_per_block, blockIdx.x, blockIdx.y);
 }
 
 // Two independent operations in one launch (128-bit rows, default store policy): workgroups [0, first_blocks)
@@ -302,7 +302,8 @@ static int launch_row_gather(int64_t row_bytes, int64_t tile_dim_rows, int64_t o
   if (grid.y > 65535u) return EN_ERR_SHAPE;
   switch (vb) {
     case 16:
-      if (out_bytes >= kStreamStoreBytes) row_gather_kernel<uint4, Map, NT, true><<<grid, kBlock, 0, stream>>>(map, p, vpr, R);
+      if (out_bytes >= kStreamLoadBytes) row_gather_kernel<uint4, Map, NT, true, true><<<grid, kBlock, 0, stream>>>(map, p, vpr, R);
+      else if (out_bytes >= kStreamStoreBytes) row_gather_kernel<uint4, Map, NT, true><<<grid, kBlock, 0, stream>>>(map, p, vpr, R);
       else row_gather_kernel<uint4, Map, NT, false><<<grid, kBlock, 0, stream>>>(map, p, vpr, R);
       break;
     case 8: row_gather_kernel<uint2, Map, NT, false><<<grid, kBlock, 0, stream>>>(map, p, vpr, R); break;

@@ -47,8 +47,10 @@ def padding_removal_layer(hidden_padded: torch.Tensor, qkv_packed: torch.Tensor,
     ``True``             QK^T / softmax / PV in the single fused kernel on the padded buffer (16-bit dtypes
                          only); the score tensor is then never written;
     ``"packed"``         the fused kernel on the packed projections;
-    ``None`` (default)   ``"varlen_packed"`` where it applies, else ``"varlen"``; with ``keep`` the
-                         reference's sequence, whose intermediates are the ones a caller can name.
+    ``None`` (default)   ``"varlen"``; with ``keep`` the reference's sequence, whose intermediates are
+                         the ones a caller can name.  (``"varlen_packed"`` speeds the softmax up -- 2048-key
+                         rows: 148 -> 131 us -- but its rows start on 16-byte instead of 128-byte boundaries,
+                         which costs QK^T and PV more than that: 133 -> 215 us and 134 -> 160 us.)
 
     ``fold_depad`` drops the depad launch: the LayerNorm takes its residual rows straight from
     ``hidden_padded`` (default: on, unless ``keep`` asks for the packed residual).  ``ctx_out``
@@ -66,8 +68,7 @@ def padding_removal_layer(hidden_padded: torch.Tensor, qkv_packed: torch.Tensor,
         if keep:
             fused_attention = False
         else:
-            packable = causal and hidden_padded.dtype != torch.float32 and S <= 2048 and D % 8 == 0 and D <= 128
-            fused_attention = "varlen_packed" if packable else "varlen"
+            fused_attention = "varlen"
     if fold_depad is None:
         fold_depad = not keep
     if not keep:
