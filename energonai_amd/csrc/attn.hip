@@ -210,7 +210,9 @@ __global__ __launch_bounds__(kBlock, 3) void attn_qk_strip_kernel(AttnArgs a) {
   constexpr int CVEC_ROW = BK / EPV;             // 128-bit vectors per score row of a tile
   constexpr int CSTORES = 32 * CVEC_ROW / kWave; // vectors each lane stores per tile
   static_assert(BK * KVEC_ROW % kBlock == 0, "K tile must divide over the block");
-  __shared__ __attribute__((aligned(16))) T lds_k[2][BK * KPITCH];
+  constexpr bool DMA = (DP == 128);              // K tiles go from memory straight into LDS
+  constexpr int KP = DMA ? DP : KPITCH;
+  __shared__ __attribute__((aligned(16))) T lds_k[2][BK * KP];
   __shared__ __attribute__((aligned(16))) T lds_c[kBlock / kWave][32 * CPITCH];
 
   int unit, qi;
@@ -251,12 +253,23 @@ __global__ __launch_bounds__(kBlock, 3) void attn_qk_strip_kernel(AttnArgs a) {
   const rsrc_t k_rsrc = make_rsrc(kbase, (uint32_t)(((int64_t)(kl - 1) * a.k_ss + a.D) * E::kSize));
   const rsrc_t s_rsrc = make_rsrc(sbase, (uint32_t)(score_row_offset<EPV>(a, ql) * E::kSize));   // rows >= ql are dropped
   const uint32_t k_row_bytes = (uint32_t)(a.k_ss * E::kSize);
-  const int k_row = tid / KVEC_ROW, k_c = tid % KVEC_ROW;
+  // direct loads: one instruction of a wave fills 1 KB of LDS, lane i the 16 bytes at 16 i.  Slot c of row r
+  // holds the row's chunk c ^ (r & 15), which keeps the fragment reads of 16 consecutive rows on distinct banks.
+  const int k_row = DMA ? wave * (kWave / KVEC_ROW) + lane / KVEC_ROW : tid / KVEC_ROW;
+  const int k_c = DMA ? (lane % KVEC_ROW) ^ (k_row & (KVEC_ROW - 1)) : tid % KVEC_ROW;
   uint32_t k_off = (k_c * EPV < a.D) ? k_row * k_row_bytes + k_c * EPV * E::kSize : kOutOfRange;
   uint4 kreg[KLOADS];
   auto fetch_k = [&]() {
 #pragma unroll
     for (int i = 0; i < KLOADS; ++i) kreg[i] = buffer_load16(k_rsrc, k_off + i * (kBlock / KVEC_ROW) * k_row_bytes);
+    k_off += BK * k_row_bytes;
+  };
+  const desc_t k_desc = make_desc(kbase, (uint32_t)(((int64_t)(kl - 1) * a.k_ss + a.D) * E::kSize));
+  auto dma_k = [&](T *kdst) {
+    const uint32_t lds0 = lds_address(kdst) + wave * kWave * 16;
+#pragma unroll
+    for (int i = 0; i < KLOADS; ++i)
+      buffer_load16_to_lds(k_desc, lds0 + i * kBlock * 16, k_off + i * (kBlock / KVEC_ROW) * k_row_bytes);
     k_off += BK * k_row_bytes;
   };
   auto stage_k = [&](T *kdst) {
@@ -277,8 +290,13 @@ __global__ __launch_bounds__(kBlock, 3) void attn_qk_strip_kernel(AttnArgs a) {
     s_off[i] = (uint32_t)((score_row_offset<EPV>(a, row) + sc) * E::kSize);
   }
 
-  fetch_k();
-  stage_k(lds_k[0]);
+  if constexpr (DMA) {
+    dma_k(lds_k[0]);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  } else {
+    fetch_k();
+    stage_k(lds_k[0]);
+  }
   // The Q fragments are used here, before the loop, so that the wait for their loads is placed here too.  Left
   // to the loop, that wait ("at most the four newest memory operations outstanding") would on every later
   // iteration also wait for the previous tile's score stores to be acknowledged.
@@ -288,7 +306,8 @@ __global__ __launch_bounds__(kBlock, 3) void attn_qk_strip_kernel(AttnArgs a) {
   for (int kt = 0; kt < nkt; ++kt) {
     const int k0 = kt * BK;
     const T *ksrc = lds_k[kt & 1];
-    fetch_k();                                   // next tile (past the end: out of range, zeros)
+    T *knext = lds_k[(kt + 1) & 1];
+    if constexpr (DMA) dma_k(knext); else fetch_k();   // next tile (past the end: out of range, zeros)
 
     floatx16 s[KB];
 #pragma unroll
@@ -303,7 +322,9 @@ __global__ __launch_bounds__(kBlock, 3) void attn_qk_strip_kernel(AttnArgs a) {
         for (int u = 0; u < 2; ++u)
 #pragma unroll
           for (int kb = 0; kb < KB; ++kb)
-            dst[u][kb] = *reinterpret_cast<const uint4 *>(&ksrc[(kb * 32 + r) * KPITCH + M::k_of(2 * st + u, g, NVS)]);
+            dst[u][kb] = *reinterpret_cast<const uint4 *>(
+                DMA ? &ksrc[(kb * 32 + r) * KP + (((M::k_of(2 * st + u, g, NVS) / EPV) ^ (r & (KVEC_ROW - 1))) * EPV)]
+                    : &ksrc[(kb * 32 + r) * KP + M::k_of(2 * st + u, g, NVS)]);
       };
       load_stage(0, kf[0]);
 #pragma unroll
@@ -337,7 +358,10 @@ __global__ __launch_bounds__(kBlock, 3) void attn_qk_strip_kernel(AttnArgs a) {
     }
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // strip read out before the next tile overwrites it
 
-    stage_k(lds_k[(kt + 1) & 1]);                // waits for the loads of this iteration only
+    // direct loads are not in the compiler's count of outstanding memory operations: the wait is written here.
+    // They were issued before this tile's CSTORES score stores, so the tile has landed once only those are left.
+    if constexpr (DMA) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(CSTORES) : "memory");
+    else stage_k(knext);                         // waits for the loads of this iteration only
     lds_barrier();
   }
 }
@@ -711,7 +735,7 @@ static bool strides_vec_ok(int64_t sb, int64_t sh, int64_t ss, int epv) {
 template <int DT>
 static int64_t score_tensor_bytes(const AttnArgs &a) {
   constexpr int EPV = 16 / Elem<DT>::kSize;
-  return (int64_t)a.units * (a.packed_scores ? packed_row_start<EPV>(a.Sq) : (int64_t)a.Sq * a.Sk) * Elem<DT>::kSize;
+  return (int64_t)a.units * (a.packed_scores ? packed_row_start<EPV * kPackedRowVectors>(a.Sq) : (int64_t)a.Sq * a.Sk) * Elem<DT>::kSize;
 }
 
 template <int DT>

@@ -83,11 +83,11 @@ __device__ __forceinline__ int64_t k_unit_offset(const AttnArgs &a, int b, int h
 // scores of a unit: first element, elements up to the start of row q, elements of the rows below ql
 template <int EPV>
 __device__ __forceinline__ int64_t score_unit_offset(const AttnArgs &a, int unit) {
-  return (int64_t)unit * (a.packed_scores ? packed_row_start<EPV>(a.Sq) : (int64_t)a.Sq * a.Sk);
+  return (int64_t)unit * (a.packed_scores ? packed_row_start<EPV * kPackedRowVectors>(a.Sq) : (int64_t)a.Sq * a.Sk);
 }
 template <int EPV>
 __device__ __forceinline__ int64_t score_row_offset(const AttnArgs &a, int q) {
-  return a.packed_scores ? packed_row_start<EPV>(q) : (int64_t)q * a.Sk;
+  return a.packed_scores ? packed_row_start<EPV * kPackedRowVectors>(q) : (int64_t)q * a.Sk;
 }
 
 // workgroup id -> (unit, query tile): see the header comment.

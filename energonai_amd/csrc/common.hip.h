@@ -120,6 +120,27 @@ __device__ __forceinline__ void buffer_store16(rsrc_t r, uint32_t byte_offset, c
   __builtin_amdgcn_raw_buffer_store_b128(x, r, (int)byte_offset, 0, AUX);
 }
 
+// Loads that go from memory straight into LDS, without passing through registers.  One instruction of a wave
+// writes 64 x 16 bytes to consecutive LDS addresses starting at the (wave-uniform) byte address `lds_addr`:
+// lane i's 16 bytes land at lds_addr + 16 i, whatever offset the lane reads from.  An offset outside the
+// descriptor's range writes zeros.  The compiler does not see the LDS write: the caller waits with
+// `s_waitcnt vmcnt(n)` (these loads count like any other) before a barrier that publishes the data.  A wait the
+// compiler computes for its own loads and stores stays correct: operations it does not know of only make the
+// counter larger, so its waits become stricter, never weaker.
+typedef u32x4 desc_t;
+__device__ __forceinline__ desc_t make_desc(const void *base, uint32_t bytes) {
+  const uint64_t p = (uint64_t)(uintptr_t)base;
+  return desc_t{(uint32_t)p, (uint32_t)(p >> 32), bytes, 0x00020000u};
+}
+__device__ __forceinline__ uint32_t lds_address(const void *p) {
+  return (uint32_t)(uintptr_t)(__attribute__((address_space(3))) const void *)p;
+}
+__device__ __forceinline__ void buffer_load16_to_lds(desc_t d, uint32_t lds_addr, uint32_t byte_offset) {
+  // M0 carries the LDS address; one wait state separates its write from the load that reads it
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds"
+               :: "s"(lds_addr), "v"(byte_offset), "s"(d) : "memory");
+}
+
 // Workgroup barrier that orders LDS traffic only.  __syncthreads() also waits
 // for every outstanding global load and store of the wave, which would cancel
 // any prefetch that is meant to stay in flight across the barrier.
@@ -178,9 +199,13 @@ __device__ __forceinline__ float block_allreduce(float v, float *slots) {
 // Under a causal mask of a self-attention batch row q of a (batch, head) unit holds q + 1 visible scores.  In the
 // padded [B,H,S,S] layout those prefixes start a whole row pitch apart: a kernel that streams them touches short,
 // ragged pieces of memory (measured: 4.7 TB/s for an in-place pass over them against 6.5 TB/s over one
-// contiguous range).  The packed layout keeps only the prefixes, each rounded up to one 16-byte vector of V
-// elements, back to back: row q starts at packed_row_start(q) elements into its unit and holds V * (q / V + 1)
-// elements; every unit owns a slot of packed_row_start(S) elements, S the bucket length, whatever its length.
+// contiguous range).  The packed layout keeps only the prefixes, each rounded up to a whole group of V elements,
+// back to back: row q starts at packed_row_start(q) elements into its unit and holds V * (q / V + 1) elements;
+// every unit owns a slot of packed_row_start(S) elements, S the bucket length, whatever its length.  V is 128
+// bytes' worth of elements (kPackedRowVectors 16-byte vectors): rows then start on cache-line boundaries, and a
+// wave's 128-byte stores of a score tile each fill one line (with 16-byte groups the same stores straddled two
+// lines and QK^T ran at 0.55 of its speed on the padded layout).
+constexpr int kPackedRowVectors = 8;
 template <int V>
 __host__ __device__ __forceinline__ int64_t packed_row_start(int64_t q) {
   const int64_t t = q / V;

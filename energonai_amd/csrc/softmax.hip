@@ -257,7 +257,7 @@ __device__ __forceinline__ void softmax_band_wave(const SoftmaxArgs &a, typename
         ri[i].lim = visible_keys(q_last, ql, kl, a.Sk, a.causal);
       }
     }
-    rowp[i] = unit + (a.packed ? packed_row_start<EPV>(q) : (int64_t)q * a.Sk);
+    rowp[i] = unit + (a.packed ? packed_row_start<EPV * kPackedRowVectors>(q) : (int64_t)q * a.Sk);
   }
   softmax_lane_group<DT, kBandVpl, LPR, R, STREAM, true>(a, rowp, ri, l);
 }
@@ -277,7 +277,7 @@ __global__ __launch_bounds__(kWave) void softmax_bands_kernel(SoftmaxArgs a) {
   const BandLayout L = band_layout<EPV, R>(a, kl, ql);
   if (i >= L.total) return;
   T *unit = reinterpret_cast<T *>(a.src) +
-            ((int64_t)b * a.H + h) * (a.packed ? packed_row_start<EPV>(a.Sq) : (int64_t)a.Sq * a.Sk);
+            ((int64_t)b * a.H + h) * (a.packed ? packed_row_start<EPV * kPackedRowVectors>(a.Sq) : (int64_t)a.Sq * a.Sk);
   const int lane = threadIdx.x;
   // longest rows first
   if (i < L.blocks[4]) return softmax_band_wave<DT, 4, R, STREAM>(a, unit, L.first[4] + i * 1 * R, L.first[5], kl, ql, lane);
@@ -432,7 +432,7 @@ extern "C" int64_t en_packed_scores_elems(int batch, int head_num, int seq_len, 
   using namespace en;
   const int es = dtype_size(dtype);
   if (!es || batch < 1 || head_num < 1 || seq_len < 1) return 0;
-  const int64_t unit = es == 4 ? packed_row_start<4>(seq_len) : packed_row_start<8>(seq_len);
+  const int64_t unit = es == 4 ? packed_row_start<4 * kPackedRowVectors>(seq_len) : packed_row_start<8 * kPackedRowVectors>(seq_len);
   return (int64_t)batch * head_num * unit;
 }
 

@@ -474,13 +474,13 @@ def test_contractions_on_packed_tokens_match_the_padded_route(dtype, causal, B, 
     assert torch.equal(got, want)
     assert bool((sentinel[:, T] == 9.0).all())          # nothing is written past the last token
     if causal and dtype != torch.float32:
-        epv = 8
+        epv, grp = 8, 64       # 16-byte vectors; rows of the packed layout are whole 128-byte groups
         flat = k.attn_qk_varlen(q, kk, B, S, lens_t, causal=True, packed_scores=True)
         assert flat.numel() == k.packed_scores_elems(B, H, S, dtype)
 
         def row_start(r):
-            t = r // epv
-            return epv * (epv * t * (t + 1) // 2 + (r - epv * t) * (t + 1))
+            t = r // grp
+            return grp * (grp * t * (t + 1) // 2 + (r - grp * t) * (t + 1))
         unit = row_start(S)
         for b, n in enumerate(lens):
             for qi in (0, n // 2, n - 1):
