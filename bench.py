@@ -385,13 +385,16 @@ def run_workload(torch, w, steps, warmup, want_eager=True, want_kernels=True, st
 
     # other forms of the same step through the one-call entry point, for comparison; never the headline:
     #   reference_ops_one_call   the seven ops of the reference's sequence (padded tensors, both transposes, depad)
-    #   packed_scores            the headline form with the scores in the packed causal layout
+    #   packed_scores / padded_scores   the three kernels on packed operands with the other score layout than the
+    #                            default form's (the default is packed causal scores for 16-bit causal rows of >= 256 keys)
     #   fused_attention ...      QK^T + softmax + PV in one kernel: on the padded buffer, on the packed projections,
     #                            and with depad folded into the LayerNorm as well
     if not w.decode and not step_only:
         forms = [("reference_ops_one_call_ms_per_step", False, False)]
         if w.dtype != torch.float32:
-            if w.causal:
+            if layer.default_attention_form(w.causal, w.dtype, w.seq) == "varlen_packed":
+                forms += [("padded_scores_ms_per_step", "varlen", True)]
+            elif w.causal:
                 forms += [("packed_scores_ms_per_step", "varlen_packed", True)]
             forms += [("fused_attention_ms_per_step", True, False),
                       ("packed_fused_attention_ms_per_step", "packed", False),
@@ -483,7 +486,7 @@ def kernel_table(torch, K, layer, workloads, w, d, info, steps, step_only=False)
     else:
         T = d["total"]
         # ---- the step's own forms
-        packed_scores = False       # the step's default form keeps [B,H,S,S] scores
+        packed_scores = layer.default_attention_form(w.causal, w.dtype, S) == "varlen_packed"
         qv, kv, vv = torch.chunk(d["qkv_packed"].view(T, H, 3 * D), 3, dim=-1)
         n_scores = K.packed_scores_elems(B, H, S, w.dtype) if packed_scores else B * H * S * S
         s_step = torch.empty(n_scores, dtype=w.dtype, device="cuda")
@@ -712,6 +715,7 @@ def main(argv=None) -> int:
         "api_sequence_ms_per_step": head.get("api_sequence_ms_per_step"),
         "reference_ops_one_call_ms_per_step": head.get("reference_ops_one_call_ms_per_step"),
         "packed_scores_ms_per_step": head.get("packed_scores_ms_per_step"),
+        "padded_scores_ms_per_step": head.get("padded_scores_ms_per_step"),
         "graph_ms_per_step": head.get("graph_ms_per_step"),
         "fused_attention_ms_per_step": head.get("fused_attention_ms_per_step"),
         "packed_fused_attention_ms_per_step": head.get("packed_fused_attention_ms_per_step"),

@@ -28,6 +28,14 @@ from .seqinfo import SeqInfo, seq_info
 SOFTMAX_TAIL_ROWS = 1
 
 
+def default_attention_form(causal: bool, dtype: torch.dtype, max_seq_len: int) -> str:
+    """The form ``padding_removal_layer`` runs when the caller names none: the three kernels on packed operands,
+    with the scores in the packed causal layout where that layout exists and is smaller than ``[B,H,S,S]``."""
+    if causal and dtype in (torch.float16, torch.bfloat16) and max_seq_len >= 256:
+        return "varlen_packed"
+    return "varlen"
+
+
 def padding_removal_layer(hidden_padded: torch.Tensor, qkv_packed: torch.Tensor, seq_lens, head_num: int,
                           size_per_head: int, gamma: torch.Tensor, beta: torch.Tensor, eps: float = 1e-5,
                           scale: Optional[float] = None, causal: bool = True, left_padded: bool = False,
@@ -47,10 +55,11 @@ def padding_removal_layer(hidden_padded: torch.Tensor, qkv_packed: torch.Tensor,
     ``True``             QK^T / softmax / PV in the single fused kernel on the padded buffer (16-bit dtypes
                          only); the score tensor is then never written;
     ``"packed"``         the fused kernel on the packed projections;
-    ``None`` (default)   ``"varlen"``; with ``keep`` the reference's sequence, whose intermediates are
-                         the ones a caller can name.  (``"varlen_packed"`` speeds the softmax up -- 2048-key
-                         rows: 148 -> 131 us -- but its rows start on 16-byte instead of 128-byte boundaries,
-                         which costs QK^T and PV more than that: 133 -> 215 us and 134 -> 160 us.)
+    ``None`` (default)   ``"varlen_packed"`` under a causal mask with a 16-bit dtype and rows of at least 256
+                         keys, else ``"varlen"``; with ``keep`` the reference's sequence, whose intermediates
+                         are the ones a caller can name.  (The packed layout halves the score tensor and keeps
+                         every row on whole 128-byte groups: the three kernels together take 415 -> 349 us on
+                         2048-key rows, 461 -> 457 us on 1024-key rows; short rows would only grow.)
 
     ``fold_depad`` drops the depad launch: the LayerNorm takes its residual rows straight from
     ``hidden_padded`` (default: on, unless ``keep`` asks for the packed residual).  ``ctx_out``
@@ -65,10 +74,7 @@ def padding_removal_layer(hidden_padded: torch.Tensor, qkv_packed: torch.Tensor,
     T = info.total if sum_seq is None else int(sum_seq)
     scale = float(D) ** -0.5 if scale is None else scale
     if fused_attention is None:
-        if keep:
-            fused_attention = False
-        else:
-            fused_attention = "varlen"
+        fused_attention = False if keep else default_attention_form(causal, hidden_padded.dtype, S)
     if fold_depad is None:
         fold_depad = not keep
     if not keep:

@@ -188,18 +188,21 @@ def test_layer_large_fp16_one_call_path_against_the_oracle(name, total):
             inp["beta"].cuda(), 1e-5, w.scale, w.causal, w.left_padded)
     ctx = torch.full((1, T, H, D), float("nan"), dtype=w.dtype, device="cuda")
     y = layer.padding_removal_layer(*args, dense_out=dense, sum_seq=T, ctx_out=ctx)
-    # the same form, op by op through the public functions
+    assert layer.default_attention_form(w.causal, w.dtype, w.seq) == "varlen_packed"
+    # the three kernels on packed operands with [B,H,S,S] scores, in one call and op by op through the public functions
+    ctx_v = torch.full((1, T, H, D), float("nan"), dtype=w.dtype, device="cuda")
+    y_v = layer.padding_removal_layer(*args, dense_out=dense, sum_seq=T, ctx_out=ctx_v, fused_attention="varlen")
     steps = layer.padding_removal_layer(*args, dense_out=dense, sum_seq=T, keep=True, fused_attention="varlen")
-    assert torch.equal(y, steps["y"]) and torch.equal(ctx, steps["ctx_packed"])
+    assert torch.equal(y_v, steps["y"]) and torch.equal(ctx_v, steps["ctx_packed"])
     # the reference's sequence of ops (transpose_pad ... transpose_depad on padded tensors): the same bits
     ref = layer.padding_removal_layer(*args, dense_out=dense, sum_seq=T, keep=True, fused_attention=False)
-    assert torch.equal(y, ref["y"]) and torch.equal(ctx, ref["ctx_packed"])
-    # the form with packed causal scores: the same bits while the softmax gives a row the same lanes in both layouts
-    pk = layer.padding_removal_layer(*args, dense_out=dense, sum_seq=T, fused_attention="varlen_packed")
+    assert torch.equal(y_v, ref["y"]) and torch.equal(ctx_v, ref["ctx_packed"])
+    # the default form keeps the scores in the packed causal layout: the same bits while the softmax gives a row
+    # the same lanes in both layouts
     if w.seq <= 1024:
-        assert torch.equal(pk, y)
-    routes = [("one call", y.cpu(), ctx.cpu()), ("packed scores", pk.cpu(), None)]
-    del steps, ref, pk
+        assert torch.equal(y, y_v) and torch.equal(ctx, ctx_v)
+    routes = [("one call, default form", y.cpu(), ctx.cpu()), ("one call, [B,H,S,S] scores", y_v.cpu(), ctx_v.cpu())]
+    del steps, ref, y_v, ctx_v
     order = sorted(range(B), key=lambda b: lens_l[b])
     cu = [0]
     for n in lens_l:
@@ -215,9 +218,8 @@ def test_layer_large_fp16_one_call_path_against_the_oracle(name, total):
         # the LayerNorm passes the error of its input on, scaled by gamma * invvar, and rounds once more
         amp = max(1.0, float(want["invvar"].max()) * float(inp["gamma"].float().abs().max())) if dense is None else 0.0
         for route, y_r, ctx_r in routes:
-            if ctx_r is not None:
-                assert_stored_close(ctx_r[0, sl].reshape(n, H * D), want["ctx_packed"].reshape(n, H * D), w.dtype,
-                                    what=f"context, {route}")
+            assert_stored_close(ctx_r[0, sl].reshape(n, H * D), want["ctx_packed"].reshape(n, H * D), w.dtype,
+                                what=f"context, {route}")
             assert_stored_close(y_r[0, sl], want["y"][0], w.dtype, base=BASE[w.dtype] * max(amp, 1.0),
                                 what=f"LayerNorm output, {route}")
 
