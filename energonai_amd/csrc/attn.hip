@@ -560,6 +560,7 @@ __global__ __launch_bounds__(kBlock) void attn_pv_kernel(AttnArgs a) {
 template <int DT, int DP, bool STREAM>
 __global__ __launch_bounds__(kBlock, 3) void attn_pv_strip_kernel(AttnArgs a) {
   static_assert(DT != EN_F32, "16-bit storage only");
+  static_assert(DP == 64 || DP == 128, "swizzles are written for 8 or 16 slots per V row");
   typedef Elem<DT> E;
   typedef typename E::T T;
   typedef Mma<DT> M;
@@ -567,15 +568,21 @@ __global__ __launch_bounds__(kBlock, 3) void attn_pv_strip_kernel(AttnArgs a) {
   constexpr int BK = 64;                         // keys per tile
   constexpr int NVS = BK / 16;                   // MFMA steps over a key tile
   constexpr int DMT = DP / 32;                   // 32-channel MFMA tiles of the output
-  constexpr int VPITCH = BK + 4;                 // V^T rows: 34 dwords, conflict-free 64-bit accesses
-  constexpr int PPITCH = BK + EPV;               // probability rows in a wave's strip
-  constexpr int NQUAD = BK / 4, NCHUNK = DP / EPV;
-  constexpr int VUNITS = NQUAD * NCHUNK;         // (four keys, eight channels) units of a V tile
-  constexpr int PVEC_ROW = BK / EPV;
-  constexpr int PLOADS = 32 * PVEC_ROW / kWave;  // vectors each lane fetches per tile
-  static_assert(VUNITS <= kBlock, "one V unit per lane");
-  __shared__ __attribute__((aligned(16))) T lds_v[2][DP * VPITCH];
-  __shared__ __attribute__((aligned(16))) T lds_p[kBlock / kWave][32 * PPITCH];
+  constexpr int VVEC_ROW = DP / EPV;             // 16-byte slots per V row
+  constexpr int VLOADS = BK * VVEC_ROW / kBlock; // direct loads per wave and V tile
+  constexpr int RPL = kWave / VVEC_ROW;          // V rows one direct load of a wave covers
+  constexpr int PVEC_ROW = BK / EPV;             // 16-byte slots per probability row of a tile: 8
+  constexpr int PLOADS = 32 * PVEC_ROW / kWave;  // direct loads per wave and probability strip: 4, eight rows each
+  constexpr uint32_t VROW_BYTES = DP * sizeof(T), PROW_BYTES = BK * sizeof(T);
+  static_assert(BK * VVEC_ROW % kBlock == 0, "V tile must divide over the block");
+  // Both operands travel from memory straight into LDS, unpadded, with their 16-byte chunks in XOR-swizzled slots:
+  //   V tile [key][channel], two buffers: slot c of key k holds chunk c ^ vswz(k), vswz = 4 (k & 3) (16 slots) or
+  //     4 ((k >> 1) & 1) (8 slots).  The transposing read of a 16-lane group takes 32 bytes from each of four
+  //     consecutive keys; a half wave's 64 bytes per key then fall into four distinct quarters of the banks.
+  //   probability strip [query][key] of each wave, 32 x 64: slot c of row q holds chunk c ^ ((q >> 1) & 7), which
+  //     puts the 128-bit reads of 16 consecutive rows at one chunk on all 64 banks once.
+  __shared__ __attribute__((aligned(16))) T lds_v[2][BK * DP];
+  __shared__ __attribute__((aligned(16))) T lds_p[kBlock / kWave][32 * BK];
 
   int unit, qi;
   if (!map_block(a, unit, qi)) return;
@@ -606,57 +613,55 @@ __global__ __launch_bounds__(kBlock, 3) void attn_pv_strip_kernel(AttnArgs a) {
 
   const T *pbase = reinterpret_cast<const T *>(a.a_ptr) + score_unit_offset<EPV>(a, unit);
   const T *vbase = reinterpret_cast<const T *>(a.b_ptr) + k_unit_offset(a, b, h);
-  // rows of padded queries lie past the end of the resource and read as zero; so do V rows >= kl
-  const rsrc_t p_rsrc = make_rsrc(pbase, (uint32_t)(score_row_offset<EPV>(a, ql) * E::kSize));
-  const uint32_t v_bytes = kl > 0 ? (uint32_t)(((int64_t)(kl - 1) * a.k_ss + a.D) * E::kSize) : 0u;
-  const rsrc_t v_rsrc = make_rsrc(vbase, v_bytes);
+  // rows of padded queries lie past the end of the descriptor and arrive as zeros; so do V rows >= kl
+  const desc_t p_desc = make_desc(pbase, (uint32_t)(score_row_offset<EPV>(a, ql) * E::kSize));
+  const desc_t v_desc = make_desc(vbase, kl > 0 ? (uint32_t)(((int64_t)(kl - 1) * a.k_ss + a.D) * E::kSize) : 0u);
+
+  // ---- V: lane i of the wave's n-th load fills slot i % VVEC_ROW of tile row RPL (4n + wave) + i / VVEC_ROW
   const uint32_t v_row_bytes = (uint32_t)(a.k_ss * E::kSize);
-  const int v_c = (tid % 4) + 4 * (tid / (4 * NQUAD)), v_kq = (tid / 4) % NQUAD;
-  uint32_t v_off = (tid < VUNITS && v_c * EPV < a.D) ? v_kq * 4 * v_row_bytes + v_c * EPV * E::kSize : kOutOfRange;
-  uint4 vreg[4];
-  auto fetch_v = [&]() {
+  const int ld_row = wave * RPL + lane / VVEC_ROW, ld_slot = lane % VVEC_ROW;
+  const int v_c = ld_slot ^ (DP == 128 ? 4 * (ld_row & 3) : 4 * ((ld_row >> 1) & 1));
+  uint32_t v_off = (v_c * EPV < a.D) ? ld_row * v_row_bytes + v_c * EPV * E::kSize : kOutOfRange;
+  auto fetch_v = [&](T *vdst) {
+    const uint32_t v_lds = lds_address(vdst) + wave * kWave * 16;
 #pragma unroll
-    for (int x = 0; x < 4; ++x) vreg[x] = buffer_load16(v_rsrc, v_off + x * v_row_bytes);
+    for (int i = 0; i < VLOADS; ++i) buffer_load16_to_lds(v_desc, v_lds + i * kBlock * 16, v_off + i * (kBlock / VVEC_ROW) * v_row_bytes);
     v_off += BK * v_row_bytes;
   };
-  auto stage_v = [&](T *vdst) {
-    if (VUNITS == kBlock || tid < VUNITS) {
-      Pack<T, EPV> rows[4];
+  // transposing read: lane j of a 16-lane group points at key j / 4 of the group's four keys and at channels
+  // 4 (j % 4) .. + 3 of the group's sixteen; the read hands lane i of the group channel i of those sixteen at the
+  // four keys.  Byte offset inside a V buffer for channel tile mt and keys 8g + 0..3 of step 0:
+  const int tj = lane & 15, tg = (lane >> 4) & 1;
+  const int vsw = DP == 128 ? (tj >> 2) : ((tj >> 3) & 1);
+  uint32_t v_frag[DMT];
 #pragma unroll
-      for (int x = 0; x < 4; ++x) rows[x] = __builtin_bit_cast(Pack<T, EPV>, vreg[x]);
-#pragma unroll
-      for (int e = 0; e < EPV; ++e) {
-        Pack<T, 4> col;
-#pragma unroll
-        for (int x = 0; x < 4; ++x) col.v[x] = rows[x].v[e];
-        store_pack<T, 4>(&vdst[(v_c * EPV + e) * VPITCH + v_kq * 4], col);
-      }
-    }
-  };
+  for (int mt = 0; mt < DMT; ++mt)
+    v_frag[mt] = (uint32_t)((8 * g + (tj >> 2)) * VROW_BYTES + (4 * (mt ^ vsw) + 2 * tg + ((tj >> 1) & 1)) * 16 + (tj & 1) * 8);
 
-  // this lane's share of the wave's probability strip: row pr + 8i, eight keys at column pc
+  // ---- probabilities: the wave's n-th load brings rows 8n .. 8n + 7 of its strip, lane i slot i % 8 of row
+  //      8n + i / 8; the chunk it holds is (i % 8) ^ ((row >> 1) & 7) = (i % 8) ^ (i >> 4) ^ 4 (n & 1)
   T *strip = lds_p[wave];
-  const int pr = lane / PVEC_ROW, pc = (lane % PVEC_ROW) * EPV;
+  const uint32_t strip_lds = lds_address(strip);
+  const int p_c0 = (lane & 7) ^ (lane >> 4);
   uint32_t p_off[PLOADS];
-  int p_vis[PLOADS];           // a row is read only as far as its own query sees: the rest need not have been written
+  int p_left[PLOADS];          // keys of the row still visible from this lane's chunk on, in tile 0: a row is read
+                               // only as far as its own query sees, the rest need not have been written
 #pragma unroll
   for (int i = 0; i < PLOADS; ++i) {
-    const int row = qw + pr + i * (kWave / PVEC_ROW);
-    p_off[i] = (uint32_t)((score_row_offset<EPV>(a, row) + pc) * E::kSize);
-    p_vis[i] = row < ql ? tile_key_extent(a, row, kl, ql) : 0;
+    const int row = qw + 8 * i + (lane >> 3);
+    const int c = p_c0 ^ (4 * (i & 1));
+    p_off[i] = (uint32_t)((score_row_offset<EPV>(a, row) + c * EPV) * E::kSize);
+    p_left[i] = (row < ql ? tile_key_extent(a, row, kl, ql) : 0) - c * EPV;
   }
-  uint4 preg[PLOADS];
   auto fetch_p = [&](int kt) {
     const int k0 = kt * BK;
 #pragma unroll
     for (int i = 0; i < PLOADS; ++i)
-      preg[i] = buffer_load16<STREAM ? 2 : 0>(p_rsrc, (k0 + pc < p_vis[i]) ? p_off[i] + (uint32_t)(k0 * E::kSize) : kOutOfRange);
+      buffer_load16_to_lds<STREAM ? 2 : 0>(p_desc, strip_lds + i * kWave * 16,
+                                           (k0 < p_left[i]) ? p_off[i] + (uint32_t)(k0 * E::kSize) : kOutOfRange);
   };
-  auto stage_p = [&]() {
-#pragma unroll
-    for (int i = 0; i < PLOADS; ++i)
-      *reinterpret_cast<uint4 *>(&strip[(pr + i * (kWave / PVEC_ROW)) * PPITCH + pc]) = preg[i];
-  };
+  const uint32_t p_frag = (uint32_t)(r * PROW_BYTES);
+  const int psw = (r >> 1) & 7;
 
   floatx16 o[DMT];
 #pragma unroll
@@ -664,28 +669,30 @@ __global__ __launch_bounds__(kBlock, 3) void attn_pv_strip_kernel(AttnArgs a) {
 #pragma unroll
     for (int x = 0; x < 16; ++x) o[mt][x] = 0.f;
 
-  fetch_v();
+  fetch_v(lds_v[0]);
   fetch_p(0);
-  stage_v(lds_v[0]);
-  stage_p();
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   lds_barrier();
   for (int kt = 0; kt < nkt; ++kt) {
-    const T *vsrc = lds_v[kt & 1];
-    fetch_v();                                   // next tiles (past the end: out of range, no traffic)
-    fetch_p(kt + 1);
+    const char *vsrc = reinterpret_cast<const char *>(lds_v[kt & 1]);
+    fetch_v(lds_v[(kt + 1) & 1]);                // next tile (past the end: out of range, zeros, no traffic)
 
     // B operands: keys 16vs + 8g .. +7 of this lane's query, out of the wave's own strip
     uint4 pf[NVS];
 #pragma unroll
-    for (int vs = 0; vs < NVS; ++vs) pf[vs] = *reinterpret_cast<const uint4 *>(&strip[r * PPITCH + vs * 16 + 8 * g]);
+    for (int vs = 0; vs < NVS; ++vs)
+      pf[vs] = *reinterpret_cast<const uint4 *>(reinterpret_cast<const char *>(strip) + p_frag + (((2 * vs + g) ^ psw) * 16));
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // this wave has read its strip: the next one may arrive
+    fetch_p(kt + 1);
+
     // A operands: V^T at the same keys, read one step ahead of the MFMAs
     uint4 va[2][DMT];
     auto load_step = [&](int vs, uint4 (&dst)[DMT]) {
 #pragma unroll
       for (int mt = 0; mt < DMT; ++mt) {
-        const T *vrow = &vsrc[(mt * 32 + r) * VPITCH + vs * 16 + 8 * g];
-        const uint2 lo = *reinterpret_cast<const uint2 *>(vrow);
-        const uint2 hi = *reinterpret_cast<const uint2 *>(vrow + 4);
+        const char *vt = vsrc + vs * 16 * VROW_BYTES + v_frag[mt];
+        const uint2 lo = lds_read_tr16(vt);                       // keys 16vs + 8g + 0..3
+        const uint2 hi = lds_read_tr16(vt + 4 * VROW_BYTES);      // keys 16vs + 8g + 4..7
         dst[mt] = make_uint4(lo.x, lo.y, hi.x, hi.y);
       }
     };
@@ -699,9 +706,8 @@ __global__ __launch_bounds__(kBlock, 3) void attn_pv_strip_kernel(AttnArgs a) {
       __builtin_amdgcn_sched_barrier(0);
     }
 
-    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // this wave has read its strip: it may be overwritten
-    stage_v(lds_v[(kt + 1) & 1]);
-    stage_p();
+    // direct loads are not in the compiler's count of outstanding memory operations: the wait is written here
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     lds_barrier();
   }
 

@@ -135,10 +135,28 @@ __device__ __forceinline__ desc_t make_desc(const void *base, uint32_t bytes) {
 __device__ __forceinline__ uint32_t lds_address(const void *p) {
   return (uint32_t)(uintptr_t)(__attribute__((address_space(3))) const void *)p;
 }
+// AUX 2 = non-temporal, as for the loads above.
+template <int AUX = 0>
 __device__ __forceinline__ void buffer_load16_to_lds(desc_t d, uint32_t lds_addr, uint32_t byte_offset) {
   // M0 carries the LDS address; one wait state separates its write from the load that reads it
-  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds"
-               :: "s"(lds_addr), "v"(byte_offset), "s"(d) : "memory");
+  if constexpr (AUX == 2)
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, 0 offen nt lds"
+                 :: "s"(lds_addr), "v"(byte_offset), "s"(d) : "memory");
+  else
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds"
+                 :: "s"(lds_addr), "v"(byte_offset), "s"(d) : "memory");
+}
+
+// Transposing LDS read of 16-bit elements.  Within each group of 16 lanes, lane j supplies the address of four
+// consecutive elements; taking those sixteen pieces in lane order as one run of 64 elements, lane i receives
+// elements i, i + 16, i + 32, i + 48 of the run: element i % 4 of the pieces of lanes i / 4, i / 4 + 4,
+// i / 4 + 8 and i / 4 + 12.  Lanes that point at rows of a row-major tile (lane j at row j / 4, columns
+// 4 (j % 4) .. + 3) thus receive a column each: lane i gets column i of rows 0..3.
+typedef short s16x4 __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ uint2 lds_read_tr16(const void *p) {
+  const s16x4 v = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+      (__attribute__((address_space(3))) s16x4 *)(__attribute__((address_space(3))) void *)const_cast<void *>(p));
+  return __builtin_bit_cast(uint2, v);
 }
 
 // Workgroup barrier that orders LDS traffic only.  __syncthreads() also waits
