@@ -40,13 +40,14 @@ MFMA_PEAK_TFLOPS = {"f16": 2500.0, "bf16": 2500.0, "f32": 157.3}
 PROFILES = os.path.join(ROOT, "profiles")
 
 
-def measured_traffic(workload: str):
+def measured_traffic(workload: str, form: str = "default"):
     """HBM bytes per launch of each kernel of the step, from the counter summary kept under profiles/
     (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this file, scaled by what the same counters read for
     en_copy_bytes of known size; written by bench_profiles.py).  Counters cannot be read from inside the
     benchmark, so the figures of the last profiled tree are reported beside the live timing; {} when the
     summary is not there."""
-    path = os.path.join(PROFILES, f"bench_{workload}_hbm_traffic.md")
+    tag = "" if form == "default" else f"_{form}"
+    path = os.path.join(PROFILES, f"bench_{workload}{tag}_hbm_traffic.md")
     out = {}
     try:
         with open(path) as f:
@@ -63,6 +64,7 @@ def measured_traffic(workload: str):
 
 
 DTYPE_NAME = {"torch.float16": "f16", "torch.bfloat16": "bf16", "torch.float32": "f32"}
+PREHEAT_S = 0.1      # untimed load before the warm-up steps, so that the timed steps run at the settled clock
 
 
 def _event_time_ms(fn, iters, torch):
@@ -324,7 +326,7 @@ def run_block_decode(torch, w, steps, warmup):
 # ---------------------------------------------------------------------------
 # one workload on the GPU
 # ---------------------------------------------------------------------------
-def run_workload(torch, w, steps, warmup, want_eager=True, want_kernels=True, step_only=False):
+def run_workload(torch, w, steps, warmup, want_eager=True, want_kernels=True, step_only=False, form="default"):
     from energonai_amd import kernel as K
     from energonai_amd import layer, workloads
     from energonai_amd.seqinfo import seq_info
@@ -342,12 +344,26 @@ def run_workload(torch, w, steps, warmup, want_eager=True, want_kernels=True, st
         d = workloads.make_inputs(w, device=dev)
         info = seq_info(d["lens"], w.batch, dev)
         tokens = d["total"]
+        three = layer.three_kernel_form(w.causal, w.dtype, w.seq)
+        # "default": whatever padding_removal_layer runs when the caller names no form (the product's own choice);
+        # "three_kernel": QK^T, softmax and PV as separate kernels on packed operands (for profiles of those kernels)
+        step_form_name = layer.default_attention_form(w.causal, w.dtype, w.seq, w.head_dim, w.scale) \
+            if form == "default" else three
+        res["step_form"] = step_form_name
 
         def step():
             return layer.padding_removal_layer(d["hidden_padded"], d["qkv_packed"], info, w.heads, w.head_dim,
                                                d["gamma"], d["beta"], workloads.EPS, w.scale, w.causal,
-                                               w.left_padded, dense_out=d["dense_out"], sum_seq=tokens)
+                                               w.left_padded, dense_out=d["dense_out"], sum_seq=tokens,
+                                               fused_attention=None if form == "default" else three)
     res["tokens"] = tokens
+    # the GPU raises its clocks only after some tens of milliseconds of load (measured: 332 us/step after 10 steps,
+    # 295 us after 100, 294 us after 1000): the step is run untimed for PREHEAT_S first, then the W warm-up steps
+    t_heat = time.perf_counter()
+    while time.perf_counter() - t_heat < PREHEAT_S:
+        for _ in range(10):
+            step()
+        torch.cuda.synchronize()
     for _ in range(warmup):
         step()
     torch.cuda.synchronize()
@@ -385,26 +401,26 @@ def run_workload(torch, w, steps, warmup, want_eager=True, want_kernels=True, st
 
     # other forms of the same step through the one-call entry point, for comparison; never the headline:
     #   reference_ops_one_call   the seven ops of the reference's sequence (padded tensors, both transposes, depad)
-    #   packed_scores / padded_scores   the three kernels on packed operands with the other score layout than the
-    #                            default form's (the default is packed causal scores for 16-bit causal rows of >= 256 keys)
+    #   three_kernel             QK^T, softmax, PV as three kernels on packed operands, depad folded into the LayerNorm
+    #                            (the default where the fused kernel does not apply), scores in the layout
+    #                            layer.three_kernel_form picks; three_kernel_other_scores: the other score layout
     #   fused_attention ...      QK^T + softmax + PV in one kernel: on the padded buffer, on the packed projections,
-    #                            and with depad folded into the LayerNorm as well
+    #                            and with depad folded into the LayerNorm as well (the default where it applies)
     if not w.decode and not step_only:
-        forms = [("reference_ops_one_call_ms_per_step", False, False)]
+        forms = [("reference_ops_one_call_ms_per_step", False, False), ("three_kernel_ms_per_step", three, True)]
         if w.dtype != torch.float32:
-            if layer.default_attention_form(w.causal, w.dtype, w.seq) == "varlen_packed":
-                forms += [("padded_scores_ms_per_step", "varlen", True)]
-            elif w.causal:
-                forms += [("packed_scores_ms_per_step", "varlen_packed", True)]
+            if w.causal:
+                forms += [("three_kernel_other_scores_ms_per_step",
+                           "varlen" if three == "varlen_packed" else "varlen_packed", True)]
             forms += [("fused_attention_ms_per_step", True, False),
                       ("packed_fused_attention_ms_per_step", "packed", False),
                       ("packed_fused_folded_depad_ms_per_step", "packed", True)]
-        for key, form, fold in forms:
+        for key, fform, fold in forms:
             def step_form():
                 return layer.padding_removal_layer(d["hidden_padded"], d["qkv_packed"], info, w.heads, w.head_dim,
                                                    d["gamma"], d["beta"], workloads.EPS, w.scale, w.causal,
                                                    w.left_padded, dense_out=d["dense_out"], sum_seq=tokens,
-                                                   fused_attention=form, fold_depad=fold)
+                                                   fused_attention=fform, fold_depad=fold)
             for _ in range(max(2, warmup // 2)):
                 step_form()
             torch.cuda.synchronize()
@@ -437,7 +453,8 @@ def run_workload(torch, w, steps, warmup, want_eager=True, want_kernels=True, st
     torch.cuda.synchronize()
 
     if want_kernels:
-        res["step_kernels"], res["kernels"] = kernel_table(torch, K, layer, workloads, w, d, info, steps, step_only)
+        res["step_kernels"], res["three_kernel_step_kernels"], res["kernels"] = kernel_table(
+            torch, K, layer, workloads, w, d, info, steps, step_only, res.get("step_form"))
     if want_eager:
         add_eager_aux(torch, w, d, dev)
         fn = (lambda: eager_decode_step(torch, w, d)) if w.decode else (lambda: eager_prefill_step(torch, w, d))
@@ -456,20 +473,23 @@ def run_workload(torch, w, steps, warmup, want_eager=True, want_kernels=True, st
     return res
 
 
-def kernel_table(torch, K, layer, workloads, w, d, info, steps, step_only=False):
+def kernel_table(torch, K, layer, workloads, w, d, info, steps, step_only=False, step_form=None):
     """Launch-to-launch time of every kernel on its real operands -> GB/s, TFLOP/s, fraction of peak.
 
-    Two tables: `step` holds the kernels in the form the timed step launches them (prefill: QK^T and PV on the
-    packed projections with row offsets, scores in the packed causal layout where that applies, LayerNorm taking
-    its residual rows from the padded activations); `api` holds every op of the reference's sequence in the form
-    its public function launches it (padded [B,H,S,*] tensors, zero-filled padding, whole-row softmax tails).
+    Three tables: `step` holds the kernels the timed step launches, in its form (prefill default: fused attention
+    on the packed projections, LayerNorm taking its residual rows from the padded activations); `three` holds the
+    kernels of the three-kernel form of the step (QK^T and PV on the packed projections with row offsets, scores in
+    the packed causal layout where that applies, the same LayerNorm) -- it is the `step` table when that form is
+    the one timed, and is left out of a --step-only run otherwise; `api` holds every op of the reference's sequence
+    in the form its public function launches it (padded [B,H,S,*] tensors, zero-filled padding, whole-row softmax
+    tails).
     """
     dt = DTYPE_NAME[str(w.dtype)]
     es = torch.empty(0, dtype=w.dtype).element_size()
     alg = workloads.algorithmic_bytes(w, d["lens_list"])
     flops = workloads.algorithmic_flops(w, d["lens_list"])
     H, D, S, B = w.heads, w.head_dim, w.seq, w.batch
-    api, step = {}, {}
+    api, step, three = {}, {}, {}
     if w.decode:
         ones = layer._ones_info(B, d["q"].device)
         keep = layer.decode_layer(d["q"], d["k_cache"], d["v_cache"], info, d["residual"], d["gamma"], d["beta"],
@@ -485,30 +505,42 @@ def kernel_table(torch, K, layer, workloads, w, d, info, steps, step_only=False)
                                                                   workloads.EPS, residual=d["residual"])
     else:
         T = d["total"]
-        # ---- the step's own forms
-        packed_scores = layer.default_attention_form(w.causal, w.dtype, S) == "varlen_packed"
+        # ---- the kernels of the three-kernel form
+        packed_scores = layer.three_kernel_form(w.causal, w.dtype, S) == "varlen_packed"
         qv, kv, vv = torch.chunk(d["qkv_packed"].view(T, H, 3 * D), 3, dim=-1)
-        n_scores = K.packed_scores_elems(B, H, S, w.dtype) if packed_scores else B * H * S * S
-        s_step = torch.empty(n_scores, dtype=w.dtype, device="cuda")
         ctx_step = torch.empty((1, T, H, D), dtype=w.dtype, device="cuda")
         offs = info.row_offsets(S, w.left_padded)
         attn_out_step = ctx_step.view(1, T, H * D) if d["dense_out"] is None else d["dense_out"]
-        step["attn_qk"] = lambda: K.attn_qk_varlen(qv, kv, B, S, info, causal=w.causal, packed_scores=packed_scores,
-                                                   out=s_step)
-        if packed_scores:
-            step["scale_mask_softmax"] = lambda: K.scale_mask_softmax_packed(B, S, H, s_step, info, scale=w.scale)
-        else:
-            step["scale_mask_softmax"] = lambda: K.scale_mask_softmax(B, S, H, s_step.view(B, H, S, S), info,
-                                                                      scale=w.scale, causal=w.causal,
-                                                                      tail_rows=layer.SOFTMAX_TAIL_ROWS)
-        step["attn_pv"] = lambda: K.attn_pv_varlen(s_step, vv, B, S, info, causal=w.causal,
-                                                   packed_scores=packed_scores, out=ctx_step)
-        step["layernorm_residual"] = lambda: K.layer_norm_forward(attn_out_step, d["gamma"], d["beta"], (w.hidden,),
-                                                                  workloads.EPS, residual=d["hidden_padded"],
-                                                                  residual_row_offsets=offs)
+        fused_step = step_form == "packed"
+        if not (step_only and fused_step):
+            n_scores = K.packed_scores_elems(B, H, S, w.dtype) if packed_scores else B * H * S * S
+            s_step = torch.empty(n_scores, dtype=w.dtype, device="cuda")
+            three["attn_qk"] = lambda: K.attn_qk_varlen(qv, kv, B, S, info, causal=w.causal, packed_scores=packed_scores,
+                                                        out=s_step)
+            if packed_scores:
+                three["scale_mask_softmax"] = lambda: K.scale_mask_softmax_packed(B, S, H, s_step, info, scale=w.scale)
+            else:
+                three["scale_mask_softmax"] = lambda: K.scale_mask_softmax(B, S, H, s_step.view(B, H, S, S), info,
+                                                                           scale=w.scale, causal=w.causal,
+                                                                           tail_rows=layer.SOFTMAX_TAIL_ROWS)
+            three["attn_pv"] = lambda: K.attn_pv_varlen(s_step, vv, B, S, info, causal=w.causal,
+                                                        packed_scores=packed_scores, out=ctx_step)
+        ln_step = lambda: K.layer_norm_forward(attn_out_step, d["gamma"], d["beta"], (w.hidden,), workloads.EPS,
+                                               residual=d["hidden_padded"], residual_row_offsets=offs)
         alg["scale_mask_softmax"] = alg.pop("scale_mask_softmax")       # keep the key order readable
         step_alg = dict(attn_qk=alg["attn_qk"], scale_mask_softmax=alg["scale_mask_softmax_no_tail"],
-                        attn_pv=alg["attn_pv"], layernorm_residual=alg["layernorm_residual"])
+                        attn_pv=alg["attn_pv"], layernorm_residual=alg["layernorm_residual"],
+                        attn_fused_packed=4 * T * H * D * es)   # q, k, v in; ctx out
+        if fused_step:
+            # ---- the kernels of the default form: fused attention on the packed projections, then the LayerNorm
+            step["attn_fused_packed"] = lambda: K.attn_fused_packed(d["qkv_packed"], B, S, info, H, D, scale=w.scale,
+                                                                    causal=w.causal, out=ctx_step)
+            step["layernorm_residual"] = ln_step
+            if three:
+                three["layernorm_residual"] = ln_step
+        else:
+            three["layernorm_residual"] = ln_step
+            step, three = three, {}
         if not step_only:
             # ---- the reference's sequence of ops, each as its public function launches it
             keep = layer.padding_removal_layer(d["hidden_padded"], d["qkv_packed"], info, H, D, d["gamma"], d["beta"],
@@ -557,8 +589,9 @@ def kernel_table(torch, K, layer, workloads, w, d, info, steps, step_only=False)
             table[name] = row
         return table
     step_table = measure(step, alg if w.decode else step_alg)
+    three_table = measure(three, alg if w.decode else step_alg)
     api_table = measure(api, alg)
-    return step_table, api_table
+    return step_table, three_table, api_table
 
 
 # ---------------------------------------------------------------------------
@@ -661,6 +694,8 @@ def main(argv=None) -> int:
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--workload", default="c3", choices=["c1", "c2", "c3", "c4", "c5"])
+    ap.add_argument("--form", default="default", choices=["default", "three_kernel"],
+                    help="the step that is timed: the product's default form, or QK^T / softmax / PV as three kernels")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-extra", action="store_true", help="only the headline workload, no eager / other workloads")
     ap.add_argument("--step-only", action="store_true",
@@ -693,17 +728,25 @@ def main(argv=None) -> int:
     if ns.step_only:
         ns.no_extra = True
     head = run_workload(torch, w, ns.steps, ns.warmup, want_eager=not ns.no_extra, want_kernels=True,
-                        step_only=ns.step_only)
+                        step_only=ns.step_only, form=ns.form)
     torch.cuda.synchronize()
 
     # roofline of the kernel that takes the largest share of the step, in the form the step launches it
     kt = head["step_kernels"]
     dom = max(kt, key=lambda n: kt[n]["us"])
     row = kt[dom]
-    roofline = {"kernel": dom, "bound": "hbm", "achieved": row["GBps"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                "frac": row["GBps"] / HBM_PEAK_GBS,
-                "traffic": measured_traffic(w.name).get(dom), "us_per_launch": row["us"],
-                "alg_bytes_per_launch": row["alg_MB"] * 1e6}
+    if "mfma_frac" in row and dom.startswith("attn_fused"):
+        # fused attention moves 4 T H D bytes and is bound by the matrix and vector pipes, not by HBM
+        roofline = {"kernel": dom, "bound": "mfma", "achieved": row["TFLOPs"], "peak": MFMA_PEAK_TFLOPS[head["dtype"]],
+                    "unit": "TFLOP/s", "frac": row["mfma_frac"],
+                    "traffic": measured_traffic(w.name, ns.form).get(dom), "us_per_launch": row["us"],
+                    "alg_flops_per_launch": row["TFLOPs"] * 1e12 * row["us"] * 1e-6,
+                    "alg_bytes_per_launch": row["alg_MB"] * 1e6, "hbm_frac": row["hbm_frac"]}
+    else:
+        roofline = {"kernel": dom, "bound": "hbm", "achieved": row["GBps"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                    "frac": row["GBps"] / HBM_PEAK_GBS,
+                    "traffic": measured_traffic(w.name, ns.form).get(dom), "us_per_launch": row["us"],
+                    "alg_bytes_per_launch": row["alg_MB"] * 1e6}
 
     out = {
         "metric": "per_layer_tokens_per_s", "value": head["tokens_per_s"], "unit": "tokens/s", "n_gpus": 1,
@@ -712,10 +755,11 @@ def main(argv=None) -> int:
         "config": {"workload": f"{w.name}: {w.title}; batch {w.batch}, bucket {w.seq}, {w.heads}x{w.head_dim} heads, "
                                f"LayerNorm width {w.hidden}, {head['tokens']} valid tokens"},
         "roofline": roofline,
+        "step_form": head.get("step_form"), "preheat_ms": PREHEAT_S * 1e3,
+        "three_kernel_ms_per_step": head.get("three_kernel_ms_per_step"),
+        "three_kernel_other_scores_ms_per_step": head.get("three_kernel_other_scores_ms_per_step"),
         "api_sequence_ms_per_step": head.get("api_sequence_ms_per_step"),
         "reference_ops_one_call_ms_per_step": head.get("reference_ops_one_call_ms_per_step"),
-        "packed_scores_ms_per_step": head.get("packed_scores_ms_per_step"),
-        "padded_scores_ms_per_step": head.get("padded_scores_ms_per_step"),
         "graph_ms_per_step": head.get("graph_ms_per_step"),
         "fused_attention_ms_per_step": head.get("fused_attention_ms_per_step"),
         "packed_fused_attention_ms_per_step": head.get("packed_fused_attention_ms_per_step"),
@@ -723,6 +767,7 @@ def main(argv=None) -> int:
         "eager_gpu_ms_per_step": head.get("eager_gpu_ms_per_step"),
         "speedup_vs_eager_gpu": head.get("speedup_vs_eager_gpu"),
         "step_kernels": kt,
+        "three_kernel_step_kernels": head["three_kernel_step_kernels"],
         "kernels": head["kernels"],
     }
     if not ns.no_extra:

@@ -3,6 +3,7 @@
 
     python3 bench_profiles.py trace   --workload c3      # rocprofv3 --kernel-trace --stats of `bench.py --step-only`
     python3 bench_profiles.py traffic --workload c3      # two --pmc runs (FETCH_SIZE, then WRITE_SIZE) + copy calibration
+    python3 bench_profiles.py counters --workload c3     # one --pmc run of SQ counters: MFMA and VALU busy, LDS, waits
 
 Each sub-command starts rocprofv3 as a child process with `python3 bench.py ...` after `--`, reads the CSV files it
 leaves under gpurun_out/prof/, and prints a markdown summary (redirect it into profiles/bench_<workload>_*.md).
@@ -38,7 +39,7 @@ KERNEL_KEYS = [
     ("layernorm", "layernorm_residual"),
     ("decode_qk", "decode_qk"),
     ("decode_pv", "decode_pv"),
-    ("attn_fused", "attn_fused"),
+    ("attn_fused", "attn_fused_packed"),
     ("copy_kernel", "copy"),
 ]
 
@@ -95,14 +96,15 @@ def counter_rows(path: str, counter: str):
 
 
 def cmd_trace(ns) -> int:
-    bench_args = ["--workload", ns.workload, "--step-only", "--no-cpu", "--steps", str(ns.steps), "--warmup", str(ns.warmup)]
-    d, line, shown = run_profiler(f"kt_{ns.workload}", ["--kernel-trace", "--stats"], bench_args, ns.timeout)
+    bench_args = ["--workload", ns.workload, "--form", ns.form, "--step-only", "--no-cpu", "--steps", str(ns.steps),
+                  "--warmup", str(ns.warmup)]
+    d, line, shown = run_profiler(f"kt_{ns.workload}_{ns.form}", ["--kernel-trace", "--stats"], bench_args, ns.timeout)
     agg = trace_rows(find_csv(d, "kernel_trace.csv"))
     decode = ns.workload == "c5"
     kt = (line or {}).get("step_kernels", {})
-    print(f"# rocprofv3 kernel-trace summary: `bench.py --workload {ns.workload} --step-only`\n")
+    print(f"# rocprofv3 kernel-trace summary: `bench.py --workload {ns.workload} --form {ns.form} --step-only`\n")
     print("Command (MI355X box, repo root; the summary below is this command's stdout):\n")
-    print(f"```\npython3 bench_profiles.py trace --workload {ns.workload}\n  -> {shown}\n```\n")
+    print(f"```\npython3 bench_profiles.py trace --workload {ns.workload} --form {ns.form}\n  -> {shown}\n```\n")
     if line:
         print(f"Bench line of the profiled run: {line['ms_per_step'] * 1e3:.1f} us per step "
               f"({line['config']['workload']}). Event timings of the same run (`us (events)`) are taken by bench.py "
@@ -122,12 +124,13 @@ def cmd_trace(ns) -> int:
 
 
 def cmd_traffic(ns) -> int:
-    bench_args = ["--workload", ns.workload, "--step-only", "--no-cpu", "--steps", str(ns.steps), "--warmup", str(ns.warmup)]
+    bench_args = ["--workload", ns.workload, "--form", ns.form, "--step-only", "--no-cpu", "--steps", str(ns.steps),
+                  "--warmup", str(ns.warmup)]
     decode = ns.workload == "c5"
     per_counter, shown_cmds, line = {}, [], None
     calib = {}
     for counter in ("FETCH_SIZE", "WRITE_SIZE"):
-        d, line, shown = run_profiler(f"pmc_{counter}_{ns.workload}", ["--pmc", counter], bench_args, ns.timeout)
+        d, line, shown = run_profiler(f"pmc_{counter}_{ns.workload}_{ns.form}", ["--pmc", counter], bench_args, ns.timeout)
         shown_cmds.append(shown)
         per_counter[counter] = counter_rows(find_csv(d, "counter_collection.csv"), counter)
         d, cline, shown = run_profiler(f"pmc_{counter}_copy", ["--pmc", counter], ["--copy-yardstick", "--steps", "5"],
@@ -150,9 +153,9 @@ def cmd_traffic(ns) -> int:
             keys[key]["n"] = max(keys[key]["n"], len(vals))
     calls = max((v["n"] for k, v in keys.items() if k == "layernorm_residual"), default=0) or \
         max(v["n"] for v in keys.values())
-    print(f"# HBM traffic per launch, `bench.py --workload {ns.workload} --step-only`, from FETCH_SIZE / WRITE_SIZE\n")
+    print(f"# HBM traffic per launch, `bench.py --workload {ns.workload} --form {ns.form} --step-only`, from FETCH_SIZE / WRITE_SIZE\n")
     print("Command (MI355X box, repo root; the summary below is this command's stdout; one counter per run):\n")
-    print(f"```\npython3 bench_profiles.py traffic --workload {ns.workload}")
+    print(f"```\npython3 bench_profiles.py traffic --workload {ns.workload} --form {ns.form}")
     for c in shown_cmds:
         print(f"  -> {c}")
     print("```\n")
@@ -174,15 +177,66 @@ def cmd_traffic(ns) -> int:
     return 0
 
 
+SQ_COUNTERS = ["SQ_WAVE_CYCLES", "SQ_VALU_MFMA_BUSY_CYCLES", "SQ_ACTIVE_INST_VALU", "SQ_LDS_BANK_CONFLICT",
+               "SQ_LDS_IDX_ACTIVE", "SQ_WAIT_INST_ANY", "SQ_BUSY_CU_CYCLES", "GRBM_GUI_ACTIVE"]
+
+
+def cmd_counters(ns) -> int:
+    # --all-ops: the whole bench line of the workload instead of the step alone, so that the ops the step does not
+    # launch (fused attention, the movers of the reference's sequence) are counted too; a kernel name then mixes
+    # the forms that share it
+    scope = ["--no-extra"] if ns.all_ops else ["--form", ns.form, "--step-only"]
+    bench_args = ["--workload", ns.workload] + scope + ["--no-cpu", "--steps", str(ns.steps), "--warmup", str(ns.warmup)]
+    decode = ns.workload == "c5"
+    d, line, shown = run_profiler(f"sq_{ns.workload}", ["--pmc"] + SQ_COUNTERS, bench_args, ns.timeout)
+    path = find_csv(d, "counter_collection.csv")
+    per = {c: counter_rows(path, c) for c in SQ_COUNTERS}
+    keys = collections.defaultdict(lambda: collections.defaultdict(float))
+    names = collections.defaultdict(set)
+    for c, rows in per.items():
+        for name, vals in rows.items():
+            key = key_of(name, decode)
+            if key is None or key == "copy":
+                continue
+            keys[key][c] += sum(vals)
+            keys[key]["n_" + c] += len(vals)
+            names[key].add(name[:70])
+    print(f"# SQ counters of the kernels of `bench.py --workload {ns.workload} {' '.join(scope)}`\n")
+    print("Command (MI355X box, repo root; the summary below is this command's stdout):\n")
+    print(f"```\npython3 bench_profiles.py counters --workload {ns.workload}"
+          f"{' --all-ops' if ns.all_ops else ' --form ' + ns.form}\n  -> {shown}\n```\n")
+    print("All columns are sums over the launches of an op divided as stated.  `GRBM_GUI_ACTIVE` is summed over the 8 "
+          "XCDs, so SIMD cycles of a launch = GRBM_GUI_ACTIVE / 8 x 1024 SIMDs.  `SQ_WAVE_CYCLES`, "
+          "`SQ_ACTIVE_INST_VALU` and `SQ_WAIT_INST_ANY` count in units of four cycles.\n")
+    print("| op (key in the bench line) | kernels | MFMA busy, share of SIMD cycles | VALU issue, share of SIMD cycles | "
+          "resident waves per SIMD | waves waiting at s_waitcnt, share of wave time | CUs with a wave, of 256 | "
+          "LDS bank conflict cycles / LDS active cycles |\n|---|---|---|---|---|---|---|---|")
+    for key, v in keys.items():
+        simd = v["GRBM_GUI_ACTIVE"] / 8 * 1024
+        if simd <= 0:
+            continue
+        lds = v["SQ_LDS_IDX_ACTIVE"]
+        print(f"| `{key}` | {'; '.join(sorted(names[key]))} | {v['SQ_VALU_MFMA_BUSY_CYCLES'] / simd:.3f} | "
+              f"{4 * v['SQ_ACTIVE_INST_VALU'] / simd:.3f} | {4 * v['SQ_WAVE_CYCLES'] / simd:.2f} | "
+              f"{v['SQ_WAIT_INST_ANY'] / max(v['SQ_WAVE_CYCLES'], 1):.3f} | "
+              f"{v['SQ_BUSY_CU_CYCLES'] / (v['GRBM_GUI_ACTIVE'] / 8):.0f} | "
+              f"{'' if lds <= 0 else format(v['SQ_LDS_BANK_CONFLICT'] / lds, '.3f')} |")
+    return 0
+
+
 def main(argv=None) -> int:
     ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
     sub = ap.add_subparsers(dest="cmd", required=True)
-    for name, fn in (("trace", cmd_trace), ("traffic", cmd_traffic)):
+    for name, fn in (("trace", cmd_trace), ("traffic", cmd_traffic), ("counters", cmd_counters)):
         p = sub.add_parser(name)
         p.add_argument("--workload", default="c3", choices=["c1", "c2", "c3", "c4", "c5"])
+        p.add_argument("--form", default="default", choices=["default", "three_kernel"],
+                       help="which form of the step bench.py times (its --form)")
         p.add_argument("--steps", type=int, default=20)
         p.add_argument("--warmup", type=int, default=5)
         p.add_argument("--timeout", type=int, default=300, help="seconds allowed for each rocprofv3 run")
+        if name == "counters":
+            p.add_argument("--all-ops", action="store_true", help="every op of the bench line, not the step alone")
         p.set_defaults(fn=fn)
     ns = ap.parse_args(argv)
     return ns.fn(ns)

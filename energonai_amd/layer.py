@@ -28,12 +28,22 @@ from .seqinfo import SeqInfo, seq_info
 SOFTMAX_TAIL_ROWS = 1
 
 
-def default_attention_form(causal: bool, dtype: torch.dtype, max_seq_len: int) -> str:
-    """The form ``padding_removal_layer`` runs when the caller names none: the three kernels on packed operands,
-    with the scores in the packed causal layout where that layout exists and is smaller than ``[B,H,S,S]``."""
+def three_kernel_form(causal: bool, dtype: torch.dtype, max_seq_len: int) -> str:
+    """QK^T, softmax and PV as three kernels on packed operands: with the scores in the packed causal layout where
+    that layout exists and is smaller than ``[B,H,S,S]``."""
     if causal and dtype in (torch.float16, torch.bfloat16) and max_seq_len >= 256:
         return "varlen_packed"
     return "varlen"
+
+
+def default_attention_form(causal: bool, dtype: torch.dtype, max_seq_len: int, size_per_head: int,
+                           scale: float = 1.0) -> str:
+    """The form ``padding_removal_layer`` runs when the caller names none: the fused kernel on the packed
+    projections wherever it applies (16-bit storage, heads of at most 128 channels in multiples of 8, a positive
+    scale) -- the score tensor then never exists and the step is two launches -- else the three kernels."""
+    if dtype in (torch.float16, torch.bfloat16) and size_per_head <= 128 and size_per_head % 8 == 0 and scale > 0:
+        return "packed"
+    return three_kernel_form(causal, dtype, max_seq_len)
 
 
 def padding_removal_layer(hidden_padded: torch.Tensor, qkv_packed: torch.Tensor, seq_lens, head_num: int,
@@ -55,11 +65,12 @@ def padding_removal_layer(hidden_padded: torch.Tensor, qkv_packed: torch.Tensor,
     ``True``             QK^T / softmax / PV in the single fused kernel on the padded buffer (16-bit dtypes
                          only); the score tensor is then never written;
     ``"packed"``         the fused kernel on the packed projections;
-    ``None`` (default)   ``"varlen_packed"`` under a causal mask with a 16-bit dtype and rows of at least 256
-                         keys, else ``"varlen"``; with ``keep`` the reference's sequence, whose intermediates
-                         are the ones a caller can name.  (The packed layout halves the score tensor and keeps
-                         every row on whole 128-byte groups: the three kernels together take 415 -> 349 us on
-                         2048-key rows, 461 -> 457 us on 1024-key rows; short rows would only grow.)
+    ``None`` (default)   ``"packed"`` wherever the fused kernel applies (16-bit dtypes, heads of at most 128
+                         channels), else the three kernels: ``"varlen_packed"`` under a causal mask with rows of
+                         at least 256 keys, ``"varlen"`` otherwise; with ``keep`` the reference's sequence, whose
+                         intermediates are the ones a caller can name.  (The packed score layout halves the score
+                         tensor and keeps every row on whole 128-byte groups: the three kernels together take
+                         415 -> 349 us on 2048-key rows, 461 -> 457 us on 1024-key rows; short rows would only grow.)
 
     ``fold_depad`` drops the depad launch: the LayerNorm takes its residual rows straight from
     ``hidden_padded`` (default: on, unless ``keep`` asks for the packed residual).  ``ctx_out``
@@ -74,7 +85,7 @@ def padding_removal_layer(hidden_padded: torch.Tensor, qkv_packed: torch.Tensor,
     T = info.total if sum_seq is None else int(sum_seq)
     scale = float(D) ** -0.5 if scale is None else scale
     if fused_attention is None:
-        fused_attention = False if keep else default_attention_form(causal, hidden_padded.dtype, S)
+        fused_attention = False if keep else default_attention_form(causal, hidden_padded.dtype, S, D, scale)
     if fold_depad is None:
         fold_depad = not keep
     if not keep:

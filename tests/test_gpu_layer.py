@@ -168,14 +168,17 @@ def test_layer_large_fp16_properties(name, total):
 
 @pytest.mark.parametrize("name,total", [("c3", 9244), ("c4", 20142)])
 def test_layer_large_fp16_one_call_path_against_the_oracle(name, total):
-    """The form the benchmark times (one call into the library: padding rows of the padded tensor not written, no
-    softmax tail, depad paired with transpose_pad on small batches) at full size: context and output of the
+    """The forms the benchmark times, through the one-call entry point at full size: the default form (fused
+    attention on the packed projections, depad folded into the LayerNorm) and the three-kernel forms (scores in the
+    packed causal layout or in [B,H,S,S]; padding rows never written, no softmax tail).  Context and output of the
     longest, the median and the shortest sequence against the oracle run on that sequence alone (attention and
-    LayerNorm are independent per sequence), and bit-equality with the op-by-op sequence of public calls.
+    LayerNorm are independent per sequence), and bit-equality of the three-kernel forms with the op-by-op
+    sequence of public calls and with the reference's own sequence of ops.
 
-    Bounds: 2e-3 on top of half an fp16 ulp of the stored value, against the float32 oracle that rounds scores
-    and probabilities to fp16 where the API stores them (the reference materialises the same fp16 tensors,
-    examples/gpt/gpt.py:108-125)."""
+    Bounds: 2e-3 on top of half an fp16 ulp of the stored value.  The three-kernel forms are held against the
+    float32 oracle that rounds scores and probabilities to fp16 where the API stores them (the reference
+    materialises the same fp16 tensors, examples/gpt/gpt.py:108-125); the fused kernel never stores them and is
+    held against the oracle that rounds nothing in between."""
     layer, wl = _mods()
     w = wl.BY_NAME[name]
     announce("layer one-call", name)
@@ -186,10 +189,15 @@ def test_layer_large_fp16_one_call_path_against_the_oracle(name, total):
     dense = None if inp["dense_out"] is None else inp["dense_out"].cuda()
     args = (inp["hidden_padded"].cuda(), inp["qkv_packed"].cuda(), inp["lens"].cuda(), H, D, inp["gamma"].cuda(),
             inp["beta"].cuda(), 1e-5, w.scale, w.causal, w.left_padded)
+    # the default form: fused attention on the packed projections, depad folded into the LayerNorm
+    assert layer.default_attention_form(w.causal, w.dtype, w.seq, D, w.scale) == "packed"
     ctx = torch.full((1, T, H, D), float("nan"), dtype=w.dtype, device="cuda")
     y = layer.padding_removal_layer(*args, dense_out=dense, sum_seq=T, ctx_out=ctx)
-    assert layer.default_attention_form(w.causal, w.dtype, w.seq) == "varlen_packed"
-    # the three kernels on packed operands with [B,H,S,S] scores, in one call and op by op through the public functions
+    # the three kernels on packed operands, scores in the packed causal layout
+    assert layer.three_kernel_form(w.causal, w.dtype, w.seq) == "varlen_packed"
+    ctx_p = torch.full((1, T, H, D), float("nan"), dtype=w.dtype, device="cuda")
+    y_p = layer.padding_removal_layer(*args, dense_out=dense, sum_seq=T, ctx_out=ctx_p, fused_attention="varlen_packed")
+    # the same with [B,H,S,S] scores, in one call and op by op through the public functions
     ctx_v = torch.full((1, T, H, D), float("nan"), dtype=w.dtype, device="cuda")
     y_v = layer.padding_removal_layer(*args, dense_out=dense, sum_seq=T, ctx_out=ctx_v, fused_attention="varlen")
     steps = layer.padding_removal_layer(*args, dense_out=dense, sum_seq=T, keep=True, fused_attention="varlen")
@@ -197,12 +205,13 @@ def test_layer_large_fp16_one_call_path_against_the_oracle(name, total):
     # the reference's sequence of ops (transpose_pad ... transpose_depad on padded tensors): the same bits
     ref = layer.padding_removal_layer(*args, dense_out=dense, sum_seq=T, keep=True, fused_attention=False)
     assert torch.equal(y_v, ref["y"]) and torch.equal(ctx_v, ref["ctx_packed"])
-    # the default form keeps the scores in the packed causal layout: the same bits while the softmax gives a row
-    # the same lanes in both layouts
+    # packed causal scores: the same bits while the softmax gives a row the same lanes in both layouts
     if w.seq <= 1024:
-        assert torch.equal(y, y_v) and torch.equal(ctx, ctx_v)
-    routes = [("one call, default form", y.cpu(), ctx.cpu()), ("one call, [B,H,S,S] scores", y_v.cpu(), ctx_v.cpu())]
-    del steps, ref, y_v, ctx_v
+        assert torch.equal(y_p, y_v) and torch.equal(ctx_p, ctx_v)
+    routes = [("default form (fused attention)", y.cpu(), ctx.cpu(), None),
+              ("three kernels, packed scores", y_p.cpu(), ctx_p.cpu(), torch.float16),
+              ("three kernels, [B,H,S,S] scores", y_v.cpu(), ctx_v.cpu(), torch.float16)]
+    del steps, ref, y_v, ctx_v, y_p, ctx_p
     order = sorted(range(B), key=lambda b: lens_l[b])
     cu = [0]
     for n in lens_l:
@@ -212,12 +221,15 @@ def test_layer_large_fp16_one_call_path_against_the_oracle(name, total):
         announce("  sequence", b, "length", n)
         sl = slice(cu[b], cu[b] + n)
         sub_dense = None if inp["dense_out"] is None else inp["dense_out"][:, sl]
-        want = eager.layer_unpadded(inp["hidden_padded"][b:b + 1], inp["qkv_packed"][:, sl], [n], H, D, inp["gamma"],
-                                    inp["beta"], 1e-5, w.scale, w.causal, w.left_padded, dense_out=sub_dense,
-                                    acc_dtype=torch.float32, storage_dtype=torch.float16)
-        # the LayerNorm passes the error of its input on, scaled by gamma * invvar, and rounds once more
-        amp = max(1.0, float(want["invvar"].max()) * float(inp["gamma"].float().abs().max())) if dense is None else 0.0
-        for route, y_r, ctx_r in routes:
+        # the fused kernel keeps scores and probabilities in fp32 registers: its oracle rounds nothing in between
+        wants = {st: eager.layer_unpadded(inp["hidden_padded"][b:b + 1], inp["qkv_packed"][:, sl], [n], H, D,
+                                          inp["gamma"], inp["beta"], 1e-5, w.scale, w.causal, w.left_padded,
+                                          dense_out=sub_dense, acc_dtype=torch.float32, storage_dtype=st)
+                 for st in (None, torch.float16)}
+        for route, y_r, ctx_r, st in routes:
+            want = wants[st]
+            # the LayerNorm passes the error of its input on, scaled by gamma * invvar, and rounds once more
+            amp = max(1.0, float(want["invvar"].max()) * float(inp["gamma"].float().abs().max())) if dense is None else 0.0
             assert_stored_close(ctx_r[0, sl].reshape(n, H * D), want["ctx_packed"].reshape(n, H * D), w.dtype,
                                 what=f"context, {route}")
             assert_stored_close(y_r[0, sl], want["y"][0], w.dtype, base=BASE[w.dtype] * max(amp, 1.0),
@@ -273,7 +285,7 @@ def test_layer_c2_fused_attention(mode):
 
 
 @pytest.mark.parametrize("name,form", [("c1", False), ("c1", "varlen"), ("c2", False), ("c2", True), ("c2", "packed"),
-                                       ("c2", "varlen"), ("c2", "varlen_packed"), ("c2", None)])
+                                       ("c2", "varlen"), ("c2", "varlen_packed")])
 def test_layer_single_call_equals_the_op_by_op_sequence(name, form):
     """padding_removal_layer without keep= goes through the one-call entry point of the library; it must give
     bit for bit what the same ops give when called one by one."""
@@ -290,10 +302,28 @@ def test_layer_single_call_equals_the_op_by_op_sequence(name, form):
     assert torch.equal(once, steps["y"])
     twice = layer.padding_removal_layer(*args, dense_out=dense, fused_attention=form, sum_seq=int(inp["lens"].sum()))
     assert torch.equal(twice, once)
-    if form in ("varlen", "varlen_packed", None):
+    if form in ("varlen", "varlen_packed"):
         # the contractions on packed tokens compute what the reference's sequence of ops computes, bit for bit
         ref = layer.padding_removal_layer(*args, dense_out=dense, keep=True, fused_attention=False)
         assert torch.equal(once, ref["y"]) and torch.equal(steps["ctx_packed"], ref["ctx_packed"])
+
+
+@pytest.mark.parametrize("name,want_form", [("c1", "varlen"), ("c2", "packed")])
+def test_layer_default_form(name, want_form):
+    """With no form named the step runs the fused kernel on the packed projections where it applies (16-bit
+    storage), else the three kernels on packed operands; depad is folded into the LayerNorm either way."""
+    layer, wl = _mods()
+    w = wl.BY_NAME[name]
+    announce("layer default form", name)
+    assert layer.default_attention_form(w.causal, w.dtype, w.seq, w.head_dim, w.scale) == want_form
+    inp = wl.make_inputs(w)
+    args = (inp["hidden_padded"].cuda(), inp["qkv_packed"].cuda(), inp["lens"].cuda(), w.heads, w.head_dim,
+            inp["gamma"].cuda(), inp["beta"].cuda(), 1e-5, w.scale, w.causal, w.left_padded)
+    dense = inp.get("dense_out")
+    dense = None if dense is None else dense.cuda()
+    default = layer.padding_removal_layer(*args, dense_out=dense)
+    named = layer.padding_removal_layer(*args, dense_out=dense, fused_attention=want_form, fold_depad=True)
+    assert torch.equal(default, named)
 
 
 @pytest.mark.parametrize("name,form", [("c1", False), ("c2", False), ("c2", "packed"), ("c2", "varlen_packed")])

@@ -245,7 +245,10 @@ def test_layer_random_shapes(seed):
     for form, fold in forms:
         y = layer.padding_removal_layer(*args, dense_out=dense_g, fused_attention=form, fold_depad=fold)
         assert y.shape == (1, T, hid)
-        three_kernels = form in (False, None, "varlen", "varlen_packed")
+        if form is None:        # the default: the fused kernel wherever it applies, else the three kernels
+            three_kernels = layer.default_attention_form(causal, dtype, S, D, scale) != "packed"
+        else:
+            three_kernels = form in (False, "varlen", "varlen_packed")
         assert_stored_close(y.cpu(), (want_r if three_kernels else want)["y"], dtype, base=base_y, what=f"y {form} {fold}")
         if three_kernels:
             assert torch.equal(y, kept["y"]), (form, fold)      # the one-call step gives the op-by-op bits
