@@ -16,14 +16,20 @@
 //                    per-lane reductions plus one exchange between the two
 //                    lane groups.
 //   online softmax   running max / sum per lane; exp2 with the scale folded in.
-//   O^T += V^T P^T   A = V^T rows from LDS (V is staged transposed), B = the
-//                    probabilities straight out of the S^T accumulators,
-//                    rounded to the storage type: a lane's registers
-//                    (j, i) hold keys 8j + 4g + i, and the A operand simply
-//                    reads V^T at those same keys, so P never touches LDS.
+//   O^T += V^T P^T   A = V^T, read out of the row-major V tile with the LDS
+//                    transposing read (four keys of one channel per lane and
+//                    instruction), B = the probabilities straight out of the
+//                    S^T accumulators, rounded to the storage type: a lane's
+//                    registers (j, i) hold keys 8j + 4g + i, and the A operand
+//                    simply reads V at those same keys, so P never touches LDS.
 //
-// K/V tiles are fetched with bounds-checked 128-bit buffer loads ahead of use
-// and the barriers order LDS only, as in the unfused kernels.
+// K/V tiles travel from memory straight into LDS (bounds-checked loads that
+// write LDS): no registers hold a tile in flight and no instruction copies
+// one.  Rows keep their 16-byte chunks in XOR-swizzled slots so that both kinds
+// of fragment read are free of bank conflicts.  K has two buffers and is a tile
+// ahead; V has one buffer, is sent for at the top of its own tile and arrives
+// behind the score and softmax work: 48 KB of LDS per workgroup, so that three
+// workgroups fit a CU.  The barriers order LDS only, as in the unfused kernels.
 #include "attn_common.hip.h"
 
 namespace en {
@@ -46,7 +52,7 @@ __device__ __forceinline__ void halves_of(float x, float &lo, float &hi) {
 }
 
 template <int DT, int DP>
-__global__ __launch_bounds__(kBlock, 2) void attn_fused_kernel(FusedArgs fa) {
+__global__ __launch_bounds__(kBlock, 3) void attn_fused_kernel(FusedArgs fa) {
   static_assert(DT != EN_F32, "the fused kernel is built for 16-bit storage");
   typedef Elem<DT> E;
   typedef typename E::T T;
@@ -57,18 +63,14 @@ __global__ __launch_bounds__(kBlock, 2) void attn_fused_kernel(FusedArgs fa) {
   constexpr int KB = BK / 32;                    // 32-key MFMA blocks per tile
   constexpr int NVS = DP / 16;                   // MFMA steps over the head dim
   constexpr int DMT = DP / 32;                   // 32-channel MFMA tiles of the output
-  constexpr int KPITCH = DP + EPV;               // LDS pitch of a K row
-  constexpr int VPITCH = BK + 4;                 // LDS pitch of a V^T row: 34 dwords, so the 32 rows a 64-bit
-                                                 // fragment read touches fall into 32 distinct bank pairs
-  constexpr int KVEC_ROW = DP / EPV;
-  constexpr int KLOADS = BK * KVEC_ROW / kBlock;
-  constexpr int NQUAD = BK / 4, NCHUNK = DP / EPV;
-  constexpr int VUNITS = NQUAD * NCHUNK;         // (four keys, eight channels) units of a V tile
-  constexpr int VLOADS = (VUNITS + kBlock - 1) / kBlock;
+  constexpr int ROW = DP;                        // LDS pitch of a K or V row: tiles are written by direct loads, unpadded
+  constexpr int KVEC_ROW = DP / EPV;             // 16-byte slots per row
+  constexpr int KLOADS = BK * KVEC_ROW / kBlock; // direct-load instructions per wave and tile, for each of K and V
   constexpr float kLog2e = 1.4426950408889634f;
-  static_assert(BK * KVEC_ROW % kBlock == 0, "K tile must divide over the block");
-  __shared__ __attribute__((aligned(16))) T lds_k[2][BK * KPITCH];
-  __shared__ __attribute__((aligned(16))) T lds_v[2][DP * VPITCH];
+  static_assert(DP == 64 || DP == 128, "swizzles are written for 8 or 16 slots per row");
+  static_assert(BK * KVEC_ROW % kBlock == 0, "tiles must divide over the block");
+  __shared__ __attribute__((aligned(16))) T lds_k[2][BK * ROW];
+  __shared__ __attribute__((aligned(16))) T lds_v[BK * ROW];
 
   int unit, qi;
   if (!map_block(a, unit, qi)) return;
@@ -112,48 +114,51 @@ __global__ __launch_bounds__(kBlock, 2) void attn_fused_kernel(FusedArgs fa) {
     }
   }
 
-  // K / V tiles: the resources end with the last valid key, so rows past it (and whole tiles
-  // past the last one) read as zeros with no traffic and no branches.  Each lane keeps one
-  // byte offset per operand and advances it by a tile per iteration; lanes whose channel
-  // chunk lies past the head size sit at an offset that stays out of range.
+  // K / V tiles: the descriptors end with the last valid key, so rows past it (and whole tiles past the last
+  // one) arrive as zeros with no traffic and no branches.  One direct load of a wave fills 1 KB of LDS, lane i
+  // the 16 bytes at 16 i: that is slot i % KVEC_ROW of tile row (64 / KVEC_ROW) * (4 n + wave) + i / KVEC_ROW
+  // for the wave's n-th load.  Which 16-byte chunk of the row a slot holds is the lane's choice of offset:
+  //   K: slot c of row r holds chunk c ^ kswz(r), kswz = r & 15 (16 slots) or (r >> 1) & 7 (8 slots): the
+  //      128-bit fragment reads of 16 consecutive rows at one chunk then cover all 64 banks once;
+  //   V: slot c of key k holds chunk c ^ vswz(k), vswz = 4 (k & 3) (16 slots) or 4 ((k >> 1) & 1) (8 slots):
+  //      a transposing read takes 64 bytes from each of four consecutive keys, which the swizzle spreads over
+  //      the four quarters of the banks.
+  // Both swizzles depend on the row only through bits the lane's position fixes, so each lane keeps one byte
+  // offset per operand and advances it by a tile per load; lanes whose chunk lies past the head size sit at an
+  // offset that stays out of range.
   const uint32_t k_bytes = kl > 0 ? (uint32_t)(((int64_t)(kl - 1) * a.k_ss + a.D) * E::kSize) : 0u;
   const uint32_t v_bytes = kl > 0 ? (uint32_t)(((int64_t)(kl - 1) * fa.v_ss + a.D) * E::kSize) : 0u;
-  const rsrc_t k_rsrc = make_rsrc(kbase, k_bytes);
-  const rsrc_t v_rsrc = make_rsrc(vbase, v_bytes);
+  const desc_t k_desc = make_desc(kbase, k_bytes);
+  const desc_t v_desc = make_desc(vbase, v_bytes);
   const uint32_t k_row_bytes = (uint32_t)(a.k_ss * E::kSize), v_row_bytes = (uint32_t)(fa.v_ss * E::kSize);
-  const int k_row = tid / KVEC_ROW, k_c = tid % KVEC_ROW;                  // vector i sits kBlock / KVEC_ROW rows lower
-  const int v_c = (tid % 4) + 4 * (tid / (4 * NQUAD)), v_kq = (tid / 4) % NQUAD;
-  uint32_t k_off = (k_c * EPV < a.D) ? k_row * k_row_bytes + k_c * EPV * E::kSize : kOutOfRange;
-  uint32_t v_off = (tid < VUNITS && v_c * EPV < a.D) ? v_kq * 4 * v_row_bytes + v_c * EPV * E::kSize : kOutOfRange;
-  static_assert(VUNITS <= kBlock, "one V unit per lane");
-  uint4 kreg[KLOADS];
-  uint4 vreg[4];
-  auto fetch = [&]() {
+  constexpr int RPL = kWave / KVEC_ROW;          // rows one direct load of a wave covers
+  const int ld_row = wave * RPL + lane / KVEC_ROW, ld_slot = lane % KVEC_ROW;
+  const int k_c = ld_slot ^ (DP == 128 ? (ld_row & 15) : ((ld_row >> 1) & 7));
+  const int v_c = ld_slot ^ (DP == 128 ? 4 * (ld_row & 3) : 4 * ((ld_row >> 1) & 1));
+  uint32_t k_off = (k_c * EPV < a.D) ? ld_row * k_row_bytes + k_c * EPV * E::kSize : kOutOfRange;
+  uint32_t v_off = (v_c * EPV < a.D) ? ld_row * v_row_bytes + v_c * EPV * E::kSize : kOutOfRange;
+  auto fetch_k = [&](T *kdst) {
+    const uint32_t k_lds = lds_address(kdst) + wave * kWave * 16;
 #pragma unroll
-    for (int i = 0; i < KLOADS; ++i) kreg[i] = buffer_load16(k_rsrc, k_off + i * (kBlock / KVEC_ROW) * k_row_bytes);
-#pragma unroll
-    for (int x = 0; x < 4; ++x) vreg[x] = buffer_load16(v_rsrc, v_off + x * v_row_bytes);
+    for (int i = 0; i < KLOADS; ++i) buffer_load16_to_lds(k_desc, k_lds + i * kBlock * 16, k_off + i * (kBlock / KVEC_ROW) * k_row_bytes);
     k_off += BK * k_row_bytes;
+  };
+  auto fetch_v = [&]() {
+    const uint32_t v_lds = lds_address(lds_v) + wave * kWave * 16;
+#pragma unroll
+    for (int i = 0; i < KLOADS; ++i) buffer_load16_to_lds(v_desc, v_lds + i * kBlock * 16, v_off + i * (kBlock / KVEC_ROW) * v_row_bytes);
     v_off += BK * v_row_bytes;
   };
-  // registers -> LDS: K as is, V transposed (four keys of one channel per 64-bit store)
-  auto stage = [&](T *kdst, T *vdst) {
+  // fragment addresses.  K: row 32 kb + r, chunk 2 vs + g.  V (transposing read): lane j of a 16-lane group
+  // points at key j / 4 of the group's four keys and at channels 4 (j % 4) .. + 3 of the group's sixteen; the
+  // read hands lane i of the group channel i of those sixteen at the four keys.
+  const int ksw = DP == 128 ? (r & 15) : ((r >> 1) & 7);
+  const int tj = lane & 15, tg = (lane >> 4) & 1;     // position in the 16-lane group; which half of a 32-channel tile
+  const int vsw = DP == 128 ? (tj >> 2) : ((tj >> 3) & 1);
+  uint32_t v_frag[DMT];                                // byte offset of this lane's read for channel tile mt, keys 4g + 0..3
 #pragma unroll
-    for (int i = 0; i < KLOADS; ++i)
-      *reinterpret_cast<uint4 *>(&kdst[(k_row + i * (kBlock / KVEC_ROW)) * KPITCH + k_c * EPV]) = kreg[i];
-    if (VUNITS == kBlock || tid < VUNITS) {
-      Pack<T, EPV> rows[4];
-#pragma unroll
-      for (int x = 0; x < 4; ++x) rows[x] = __builtin_bit_cast(Pack<T, EPV>, vreg[x]);
-#pragma unroll
-      for (int e = 0; e < EPV; ++e) {
-        Pack<T, 4> col;
-#pragma unroll
-        for (int x = 0; x < 4; ++x) col.v[x] = rows[x].v[e];
-        store_pack<T, 4>(&vdst[(v_c * EPV + e) * VPITCH + v_kq * 4], col);
-      }
-    }
-  };
+  for (int mt = 0; mt < DMT; ++mt)
+    v_frag[mt] = (uint32_t)((4 * g + (tj >> 2)) * ROW * E::kSize + (4 * (mt ^ vsw) + 2 * tg + ((tj >> 1) & 1)) * 16 + (tj & 1) * 8);
 
   floatx16 o[DMT];
 #pragma unroll
@@ -168,61 +173,45 @@ __global__ __launch_bounds__(kBlock, 2) void attn_fused_kernel(FusedArgs fa) {
   // range, and the final division by the row sum cancels the common factor.
   const float lazy_gap = 8.0f / c_exp;
 
-  // Tile kt is computed out of LDS buffer kt & 1 while tile kt + 1 travels HBM -> registers ->
-  // the other buffer; one barrier per tile.
-  fetch();
-  stage(lds_k[0], lds_v[0]);
+  // K tile kt is read out of buffer kt & 1 while K tile kt + 1 travels into the other one; V tile kt is sent for
+  // at the top of iteration kt (its buffer was in use until the barrier that ended iteration kt - 1) and waited
+  // for between the softmax and the second contraction.  Two barriers per tile.
+  fetch_k(lds_k[0]);
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   lds_barrier();
 
   for (int kt = 0; kt < nkt; ++kt) {
     const int k0 = kt * BK;
-    const T *ksrc = lds_k[kt & 1], *vsrc = lds_v[kt & 1];
-    fetch();
+    const T *ksrc = lds_k[kt & 1];
+    fetch_v();                                   // V tile kt
+    fetch_k(lds_k[(kt + 1) & 1]);                // K tile kt + 1 (past the end: out of range, zeros, no traffic)
+    uint4 pf[KB * 2];                            // B operands of the second MFMA: the probabilities of this tile
+    const bool live = k0 < vis_max;              // wave-uniform: later tiles are masked for all of this wave's queries
 
-    if (k0 < vis_max) {  // wave-uniform: later tiles are masked for all of this wave's queries
-      // ---- S^T = K Q^T; the K fragments are read from LDS two steps ahead of the MFMAs
+    if (live) {
+      // ---- S^T = K Q^T; the K fragments are read from LDS a step ahead of the MFMAs
       floatx16 s[KB];
 #pragma unroll
       for (int kb = 0; kb < KB; ++kb)
 #pragma unroll
         for (int x = 0; x < 16; ++x) s[kb][x] = 0.f;
       {
-        constexpr int NST = NVS / 2;                 // stages of two steps each
-        uint4 kf[2][2][KB];
-        auto load_stage = [&](int st, uint4 (&dst)[2][KB]) {
+        uint4 kf[2][KB];                             // fragments of the step after the one the MFMAs work on
+        auto load_step = [&](int vs, uint4 (&dst)[KB]) {
 #pragma unroll
-          for (int u = 0; u < 2; ++u)
-#pragma unroll
-            for (int kb = 0; kb < KB; ++kb)
-              dst[u][kb] = *reinterpret_cast<const uint4 *>(&ksrc[(kb * 32 + r) * KPITCH + M::k_of(2 * st + u, g, NVS)]);
+          for (int kb = 0; kb < KB; ++kb)
+            dst[kb] = *reinterpret_cast<const uint4 *>(&ksrc[(kb * 32 + r) * ROW + (((2 * vs + g) ^ ksw) * EPV)]);
         };
-        load_stage(0, kf[0]);
+        load_step(0, kf[0]);
 #pragma unroll
-        for (int st = 0; st < NST; ++st) {
-          if (st + 1 < NST) load_stage(st + 1, kf[(st + 1) & 1]);
-          __builtin_amdgcn_sched_barrier(0);         // keep the reads of the next stage ahead of these MFMAs
+        for (int vs = 0; vs < NVS; ++vs) {
+          if (vs + 1 < NVS) load_step(vs + 1, kf[(vs + 1) & 1]);
+          __builtin_amdgcn_sched_barrier(0);         // keep the reads of the next step ahead of these MFMAs
 #pragma unroll
-          for (int u = 0; u < 2; ++u)
-#pragma unroll
-            for (int kb = 0; kb < KB; ++kb) M::step(kf[st & 1][u][kb], qf[2 * st + u], s[kb]);
+          for (int kb = 0; kb < KB; ++kb) M::step(kf[vs & 1][kb], qf[vs], s[kb]);
           __builtin_amdgcn_sched_barrier(0);
         }
       }
-
-      // first V^T fragments are requested before the softmax arithmetic
-      constexpr int NG = KB * 2;                      // groups of 16 keys
-      uint4 va[2][DMT];
-      auto load_group = [&](int gi, uint4 (&dst)[DMT]) {
-        const int kk = gi * 16 + 4 * g;
-#pragma unroll
-        for (int mt = 0; mt < DMT; ++mt) {
-          const T *vrow = &vsrc[(mt * 32 + r) * VPITCH + kk];
-          const uint2 lo = *reinterpret_cast<const uint2 *>(vrow);
-          const uint2 hi = *reinterpret_cast<const uint2 *>(vrow + 8);
-          dst[mt] = make_uint4(lo.x, lo.y, hi.x, hi.y);
-        }
-      };
-      load_group(0, va[0]);
 
       // ---- mask + online softmax; register 4j+i of block kb holds key k0 + 32kb + 8j + 4g + i
       float m_tile = -INFINITY;
@@ -259,7 +248,6 @@ __global__ __launch_bounds__(kBlock, 2) void attn_fused_kernel(FusedArgs fa) {
       }
       const float moff = (m_run == -INFINITY) ? 0.f : -m_run * c_exp;
       float l_tile = 0.f;
-      uint4 pf[NG];                                              // B operands of the second MFMA
 #pragma unroll
       for (int kb = 0; kb < KB; ++kb) {
         Pack<T, EPV> pk[2];
@@ -280,8 +268,28 @@ __global__ __launch_bounds__(kBlock, 2) void attn_fused_kernel(FusedArgs fa) {
       }
       l_run += l_tile;
 
-      // ---- O^T += V^T P^T; the A operand reads V^T at the keys the B registers hold:
+    }
+
+    // V tile kt was sent for before K tile kt + 1 and the loads complete in order: it has landed once only the
+    // K loads are outstanding; the barrier publishes every wave's share
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(KLOADS) : "memory");
+    lds_barrier();
+
+    if (live) {
+      // ---- O^T += V^T P^T; the A operand reads V at the keys the B registers hold:
       //      elements 0..3 <-> keys 16gi + 4g + 0..3, elements 4..7 <-> keys 16gi + 8 + 4g + 0..3
+      constexpr int NG = KB * 2;                      // groups of 16 keys
+      uint4 va[2][DMT];
+      auto load_group = [&](int gi, uint4 (&dst)[DMT]) {
+        const char *vt = reinterpret_cast<const char *>(lds_v) + gi * 16 * ROW * E::kSize;
+#pragma unroll
+        for (int mt = 0; mt < DMT; ++mt) {
+          const uint2 lo = lds_read_tr16(vt + v_frag[mt]);                          // keys 16 gi + 4 g + 0..3
+          const uint2 hi = lds_read_tr16(vt + v_frag[mt] + 8 * ROW * E::kSize);     // keys 16 gi + 8 + 4 g + 0..3
+          dst[mt] = make_uint4(lo.x, lo.y, hi.x, hi.y);
+        }
+      };
+      load_group(0, va[0]);
 #pragma unroll
       for (int gi = 0; gi < NG; ++gi) {
         if (gi + 1 < NG) load_group(gi + 1, va[(gi + 1) & 1]);
@@ -292,9 +300,9 @@ __global__ __launch_bounds__(kBlock, 2) void attn_fused_kernel(FusedArgs fa) {
       }
     }
 
-    // the tile fetched during this iteration goes to the other buffer, which everyone left
-    // before the barrier that ended the previous iteration
-    stage(lds_k[(kt + 1) & 1], lds_v[(kt + 1) & 1]);
+    // K tile kt + 1 has landed once none of this wave's loads is outstanding; the barrier publishes it and
+    // frees the V buffer and the other K buffer
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     lds_barrier();
   }
 
