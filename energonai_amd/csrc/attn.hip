@@ -730,6 +730,47 @@ __global__ __launch_bounds__(kBlock, 3) void attn_pv_strip_kernel(AttnArgs a) {
     }
 }
 
+// ===========================================================================
+// workgroup order for a batch: real query tiles only, longest sequence first
+// ===========================================================================
+// table[w] for workgroup w of a launch of ceil(B H / 8) * 8 * ntq workgroups.  Workgroups go to the XCDs round-robin,
+// so entries w = 8 j + x are XCD x's sequence: the (batch, head) units are dealt to the XCDs in the order of
+// decreasing sequence length (units of one sequence on consecutive XCDs), each unit's query tiles follow one another
+// from the last (longest under a causal mask) to the first, and tiles past a sequence's end get no entry.  What is
+// left of the table is -1.  One workgroup; the sort is a rank count (batch <= 1024), larger batches keep their order.
+__global__ __launch_bounds__(1024) void attn_tile_table_kernel(const int32_t *__restrict__ lens, int batch, int heads,
+                                                               int seq_len, int ntq, int32_t *__restrict__ table,
+                                                               int capacity) {
+  __shared__ int32_t s_len[1024];
+  __shared__ int32_t s_order[1024];
+  const int tid = threadIdx.x;
+  for (int i = tid; i < capacity; i += 1024) table[i] = -1;
+  const bool sorted = batch <= 1024;
+  if (sorted) {
+    if (tid < batch) s_len[tid] = min(max(lens[tid], 0), seq_len);
+    __syncthreads();
+    if (tid < batch) {
+      const int n = s_len[tid];
+      int rank = 0;
+      for (int j = 0; j < batch; ++j) rank += (s_len[j] > n || (s_len[j] == n && j < tid)) ? 1 : 0;
+      s_order[rank] = tid;
+    }
+  }
+  __syncthreads();   // also orders the -1 fill before the entries written below
+  if (tid < kXcds) {
+    const int units = batch * heads;
+    int j = 0;
+    for (int u = tid; u < units; u += kXcds) {      // u-th unit in sorted order
+      const int p = u / heads, h = u - p * heads;
+      const int b = sorted ? s_order[p] : p;
+      const int n = sorted ? s_len[b] : min(max(lens[b], 0), seq_len);
+      const int nt = (n + kQTile - 1) / kQTile;
+      const int unit = b * heads + h;
+      for (int qi = nt - 1; qi >= 0; --qi, ++j) table[j * kXcds + tid] = unit * ntq + qi;
+    }
+  }
+}
+
 // ---------------------------------------------------------------------------
 // host side
 // ---------------------------------------------------------------------------
@@ -832,16 +873,36 @@ static int check_common(const void *x, const void *y, const void *z, const int32
 
 extern "C" {
 
+int64_t en_attn_tile_table_elems(int batch, int head_num, int q_seq_len) {
+  using namespace en;
+  if (batch < 1 || head_num < 1 || q_seq_len < 1) return 0;
+  return ceil_div((int64_t)batch * head_num, (int64_t)kXcds) * kXcds * ceil_div(q_seq_len, kQTile);
+}
+
+int en_attn_tile_table(const int32_t *seq_lens, int batch, int head_num, int q_seq_len, int32_t *table,
+                       en_stream_t stream) {
+  using namespace en;
+  if (!seq_lens || !table) return EN_ERR_NULL;
+  if (batch < 1 || head_num < 1 || q_seq_len < 1) return EN_ERR_SHAPE;
+  const int64_t cap = en_attn_tile_table_elems(batch, head_num, q_seq_len);
+  if (cap > INT32_MAX || (int64_t)batch * head_num > INT32_MAX / 64) return EN_ERR_SHAPE;
+  attn_tile_table_kernel<<<1, 1024, 0, (hipStream_t)stream>>>(seq_lens, batch, head_num, q_seq_len,
+                                                               (int)ceil_div(q_seq_len, kQTile), table, (int)cap);
+  EN_RETURN_IF_LAUNCH_FAILED();
+  return EN_OK;
+}
+
 int en_attn_qk(const void *q, const void *k, void *scores, const int32_t *k_lens, const int32_t *q_lens, int batch,
                int head_num, int q_seq_len, int k_seq_len, int size_per_head, int64_t q_stride_b,
                int64_t q_stride_h, int64_t q_stride_s, int64_t k_stride_b, int64_t k_stride_h, int64_t k_stride_s,
                float alpha, int causal, int dtype, const int32_t *q_row_offsets, const int32_t *k_row_offsets,
-               int packed_scores, en_stream_t stream) {
+               int packed_scores, const int32_t *tile_table, en_stream_t stream) {
   using namespace en;
   int rc = check_common(q, k, scores, k_lens, batch, head_num, q_seq_len, k_seq_len, size_per_head, dtype);
   if (rc) return rc;
   // the packed score layout is that of causal self-attention: row q holds q + 1 scores
   if (packed_scores && (!causal || q_lens || q_seq_len != k_seq_len)) return EN_ERR_UNSUPPORTED;
+  if (tile_table && q_lens) return EN_ERR_UNSUPPORTED;      // the table lists the query tiles of min(k_lens, q_seq_len) rows
   const int es = dtype_size(dtype), epv = 16 / es;
   if (!aligned_to(q, 16) || !aligned_to(k, 16) || !aligned_to(scores, es)) return EN_ERR_ALIGN;
   if (!strides_vec_ok(q_stride_b, q_stride_h, q_stride_s, epv) ||
@@ -856,6 +917,7 @@ int en_attn_qk(const void *q, const void *k, void *scores, const int32_t *k_lens
   a.k_sb = k_stride_b; a.k_sh = k_stride_h; a.k_ss = k_stride_s;
   a.alpha = alpha; a.causal = causal ? 1 : 0; a.zero_padding = 0;
   a.q_row0 = q_row_offsets; a.k_row0 = k_row_offsets; a.packed_scores = packed_scores ? 1 : 0;
+  a.tile_table = tile_table;
   a.vec_out = ((packed_scores || (k_seq_len % epv) == 0) && aligned_to(scores, 16)) ? 1 : 0;
   a.ntq = (int)ceil_div(q_seq_len, kQTile);
   a.units = batch * head_num;
@@ -871,11 +933,12 @@ int en_attn_pv(const void *p, const void *v, void *ctx, const int32_t *k_lens, c
                int head_num, int q_seq_len, int k_seq_len, int size_per_head, int64_t v_stride_b,
                int64_t v_stride_h, int64_t v_stride_s, int64_t c_stride_b, int64_t c_stride_h, int64_t c_stride_s,
                int causal, int zero_padding, int dtype, const int32_t *c_row_offsets, const int32_t *v_row_offsets,
-               int packed_scores, en_stream_t stream) {
+               int packed_scores, const int32_t *tile_table, en_stream_t stream) {
   using namespace en;
   int rc = check_common(p, v, ctx, k_lens, batch, head_num, q_seq_len, k_seq_len, size_per_head, dtype);
   if (rc) return rc;
   if (packed_scores && (!causal || q_lens || q_seq_len != k_seq_len)) return EN_ERR_UNSUPPORTED;
+  if (tile_table && q_lens) return EN_ERR_UNSUPPORTED;      // the table lists the query tiles of min(k_lens, q_seq_len) rows
   // a packed context has no padding rows: what follows a sequence's last row is the next sequence
   if (c_row_offsets && zero_padding) return EN_ERR_UNSUPPORTED;
   const int es = dtype_size(dtype), epv = 16 / es;
@@ -892,6 +955,7 @@ int en_attn_pv(const void *p, const void *v, void *ctx, const int32_t *k_lens, c
   a.k_sb = v_stride_b; a.k_sh = v_stride_h; a.k_ss = v_stride_s;
   a.alpha = 1.f; a.causal = causal ? 1 : 0; a.zero_padding = zero_padding ? 1 : 0;
   a.q_row0 = c_row_offsets; a.k_row0 = v_row_offsets; a.packed_scores = packed_scores ? 1 : 0;
+  a.tile_table = zero_padding ? nullptr : tile_table;      // the tiles a table leaves out are the ones to fill with zeros
   a.vec_out = ((packed_scores || (k_seq_len % epv) == 0) && aligned_to(p, 16)) ? 1 : 0;
   a.ntq = (int)ceil_div(q_seq_len, kQTile);
   a.units = batch * head_num;

@@ -71,6 +71,7 @@ struct AttnArgs {
   const int32_t *q_row0;
   const int32_t *k_row0;
   int packed_scores;   // scores / probabilities are the packed causal prefixes (common.hip.h), not [B,H,Sq,Sk]
+  const int32_t *tile_table;   // workgroup id -> unit * ntq + query tile, -1 = nothing (en_attn_tile_table); null: computed
 };
 
 // first element of (batch b, head h) in q / ctx and in k / v
@@ -90,9 +91,19 @@ __device__ __forceinline__ int64_t score_row_offset(const AttnArgs &a, int q) {
   return a.packed_scores ? packed_row_start<EPV * kPackedRowVectors>(q) : (int64_t)q * a.Sk;
 }
 
-// workgroup id -> (unit, query tile): see the header comment.
+// workgroup id -> (unit, query tile): see the header comment.  With a tile table (built once per batch by
+// en_attn_tile_table) the workgroups of the sequences' real query tiles come first, longest sequence first, and the
+// rest of the grid finds -1 and leaves; without one every (unit, tile) pair of the padded shape has a workgroup and
+// those past a sequence's end leave after reading its length.
 __device__ __forceinline__ bool map_block(const AttnArgs &a, int &unit, int &qi) {
   const int bid = blockIdx.x;
+  if (a.tile_table) {
+    const int code = a.tile_table[bid];
+    if (code < 0) return false;
+    unit = code / a.ntq;
+    qi = code - unit * a.ntq;
+    return true;
+  }
   const int xcd = bid % kXcds;
   const int slot = bid / kXcds;
   unit = (slot / a.ntq) * kXcds + xcd;

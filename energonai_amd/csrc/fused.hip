@@ -340,7 +340,8 @@ extern "C" int en_attn_fused(const void *q, const void *k, const void *v, void *
                              const int32_t *q_lens, int batch, int head_num, int q_seq_len, int k_seq_len,
                              int size_per_head, const int64_t *q_strides, const int64_t *k_strides,
                              const int64_t *v_strides, const int64_t *c_strides, const int32_t *q_row_offsets,
-                             const int32_t *k_row_offsets, float scale, int causal, int dtype, en_stream_t stream) {
+                             const int32_t *k_row_offsets, float scale, int causal, int dtype,
+                             const int32_t *tile_table, en_stream_t stream) {
   using namespace en;
   if (!q || !k || !v || !ctx || !k_lens || !q_strides || !k_strides || !v_strides || !c_strides) return EN_ERR_NULL;
   if (batch < 1 || head_num < 1 || q_seq_len < 1 || k_seq_len < 1 || size_per_head < 1) return EN_ERR_SHAPE;
@@ -370,6 +371,8 @@ extern "C" int en_attn_fused(const void *q, const void *k, const void *v, void *
   fa.v_sb = v_strides[0]; fa.v_sh = v_strides[1]; fa.v_ss = v_strides[2];
   fa.c_sb = c_strides[0]; fa.c_sh = c_strides[1]; fa.c_ss = c_strides[2];
   fa.q_row0 = q_row_offsets; fa.k_row0 = k_row_offsets;
+  if (tile_table && q_lens) return EN_ERR_UNSUPPORTED;      // the table lists the query tiles of min(k_lens, q_seq_len) rows
+  a.tile_table = tile_table;
   fa.scale = scale;
   hipStream_t s = (hipStream_t)stream;
   return dtype == EN_F16 ? launch_fused<EN_F16>(fa, s) : launch_fused<EN_BF16>(fa, s);

@@ -60,7 +60,7 @@ extern "C" int en_padding_removal_layer(const void *hidden_padded, const void *q
                                         int max_seq_len, int head_num, int size_per_head, int64_t hidden,
                                         int64_t total_tokens, float scale, float eps, int causal, int left_padded,
                                         int attention_form, const int32_t *fold_depad_offsets, int dtype,
-                                        en_stream_t stream) {
+                                        const int32_t *tile_table, en_stream_t stream) {
   using namespace en;
   if (!hidden_padded || !qkv_packed || !gamma || !beta || !ctx_packed || !y || !cu_seqlens || !seq_lens)
     return EN_ERR_NULL;
@@ -89,7 +89,7 @@ extern "C" int en_padding_removal_layer(const void *hidden_padded, const void *q
     const int64_t out_strides[3] = {0, D, (int64_t)H * D};
     rc = en_attn_fused(pk, pk + (int64_t)D * es, pk + (int64_t)2 * D * es, ctx_packed, seq_lens, nullptr, B, H, S, S, D,
                        in_strides, in_strides, in_strides, out_strides, cu_seqlens, cu_seqlens, scale, causal, dtype,
-                       stream);
+                       tile_table, stream);
     if (rc) return rc;
   } else if (attention_form >= 3) {
     // The three kernels on the packed projections: q, k, v are read where the projection left them (batch b at
@@ -100,13 +100,13 @@ extern "C" int en_padding_removal_layer(const void *hidden_padded, const void *q
     const int64_t th = 3 * D, ts = (int64_t)3 * H * D;
     const int packed_scores = attention_form == 4;
     rc = en_attn_qk(q, k, scores, seq_lens, nullptr, B, H, S, S, D, 0, th, ts, 0, th, ts, 1.0f, causal, dtype, cu_seqlens,
-                    cu_seqlens, packed_scores, stream);
+                    cu_seqlens, packed_scores, tile_table, stream);
     if (rc) return rc;
     if (packed_scores) rc = en_scale_mask_softmax_packed(scores, seq_lens, B, H, S, scale, dtype, stream);
     else rc = en_scale_mask_softmax(scores, seq_lens, nullptr, B, H, S, S, scale, causal, 1, dtype, stream);
     if (rc) return rc;
     rc = en_attn_pv(scores, v, ctx_packed, seq_lens, nullptr, B, H, S, S, D, 0, th, ts, 0, D, (int64_t)H * D, causal, 0,
-                    dtype, cu_seqlens, cu_seqlens, packed_scores, stream);
+                    dtype, cu_seqlens, cu_seqlens, packed_scores, tile_table, stream);
     if (rc) return rc;
   } else {
     // the attention entry points never read a row at or past a sequence's length: no zero fill of the padding
@@ -124,17 +124,17 @@ extern "C" int en_padding_removal_layer(const void *hidden_padded, const void *q
       const int64_t in_strides[3] = {sb, sh, ss};
       const int64_t out_strides[3] = {cb, ch, cs};
       rc = en_attn_fused(q, k, v, ctx, seq_lens, nullptr, B, H, S, S, D, in_strides, in_strides, in_strides,
-                         out_strides, nullptr, nullptr, scale, causal, dtype, stream);
+                         out_strides, nullptr, nullptr, scale, causal, dtype, tile_table, stream);
       if (rc) return rc;
     } else {
       rc = en_attn_qk(q, k, scores, seq_lens, nullptr, B, H, S, S, D, sb, sh, ss, sb, sh, ss, 1.0f, causal, dtype,
-                      nullptr, nullptr, 0, stream);
+                      nullptr, nullptr, 0, tile_table, stream);
       if (rc) return rc;
       // the PV kernel reads a probability row only as far as its own query sees: no tail is written
       rc = en_scale_mask_softmax(scores, seq_lens, nullptr, B, H, S, S, scale, causal, 1, dtype, stream);
       if (rc) return rc;
       rc = en_attn_pv(scores, v, ctx, seq_lens, nullptr, B, H, S, S, D, sb, sh, ss, cb, ch, cs, causal, 0, dtype, nullptr,
-                      nullptr, 0, stream);
+                      nullptr, 0, tile_table, stream);
       if (rc) return rc;
     }
     rc = en_transpose_depad(ctx, ctx_packed, cu_seqlens, B, S, H, D, es, stream);
@@ -189,5 +189,5 @@ extern "C" int en_padding_removal_layer_noalloc(const void *hidden_padded, const
   return en_padding_removal_layer(hidden_padded, qkv_packed, dense_out, gamma, beta, at(o_x), at(o_qkv), at(o_scores),
                                   at(o_ctx), at(o_ctxp), y, cu, lens32, batch, max_seq_len, head_num,
                                   size_per_head, hidden, total_tokens, scale, eps, causal, left_padded, attention_form,
-                                  offs, dtype, stream);
+                                  offs, dtype, nullptr, stream);
 }

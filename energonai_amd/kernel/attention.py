@@ -37,6 +37,11 @@ def _lens_ptrs(seq_len_list, q_len_list, batch_size, device):
     return k_info, q_info, (0 if q_info is None else q_info.lens.data_ptr())
 
 
+def _tile_table_ptr(k_info, q_ptr, head_num: int, q_seq_len: int):
+    """Workgroup order for the batch (cached in its SeqInfo) when the query lengths are the key lengths."""
+    return None if q_ptr is not None else k_info.tile_table(head_num, q_seq_len).data_ptr()
+
+
 def attn_qk(q, k, seq_len_list, *, alpha: float = 1.0, causal: bool = True, q_len_list=None,
             out: Optional[torch.Tensor] = None):
     """scores[b,h,i,j] = alpha * <q[b,h,i,:], k[b,h,j,:]> as a new ``[B,H,Sq,Sk]`` tensor.
@@ -61,7 +66,8 @@ def attn_qk(q, k, seq_len_list, *, alpha: float = 1.0, causal: bool = True, q_le
     with _lib.device_guard(q):
         _lib.check(_lib.fn.en_attn_qk(q.data_ptr(), k.data_ptr(), out.data_ptr(), k_info.lens.data_ptr(), q_ptr,
                                           B, H, Sq, Sk, D, *qs, *ks, float(alpha), int(bool(causal)),
-                                          _lib.dtype_tag(q, "attn_qk"), None, None, 0, _lib.stream_of(q)), "attn_qk")
+                                          _lib.dtype_tag(q, "attn_qk"), None, None, 0,
+                                          _tile_table_ptr(k_info, q_ptr, H, Sq), _lib.stream_of(q)), "attn_qk")
     return out
 
 
@@ -90,7 +96,8 @@ def attn_pv(p, v, seq_len_list, *, causal: bool = True, q_len_list=None, zero_pa
     with _lib.device_guard(p):
         _lib.check(_lib.fn.en_attn_pv(p.data_ptr(), v.data_ptr(), out.data_ptr(), k_info.lens.data_ptr(), q_ptr,
                                           B, H, Sq, Sk, D, *vs, *cs, int(bool(causal)), int(bool(zero_padding)),
-                                          _lib.dtype_tag(p, "attn_pv"), None, None, 0, _lib.stream_of(p)), "attn_pv")
+                                          _lib.dtype_tag(p, "attn_pv"), None, None, 0,
+                                          _tile_table_ptr(k_info, q_ptr, H, Sq), _lib.stream_of(p)), "attn_pv")
     return out
 
 
@@ -125,7 +132,8 @@ def attn_fused(q, k, v, seq_len_list, *, scale: Optional[float] = None, causal: 
         _lib.check(_lib.fn.en_attn_fused(q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(),
                                          k_info.lens.data_ptr(), q_ptr, B, H, Sq, Sk, D, arr(*qs), arr(*ks), arr(*vs),
                                          arr(*cs), None, None, scale, int(bool(causal)),
-                                         _lib.dtype_tag(q, "attn_fused"), _lib.stream_of(q)), "attn_fused")
+                                         _lib.dtype_tag(q, "attn_fused"), _tile_table_ptr(k_info, q_ptr, H, Sq),
+                                         _lib.stream_of(q)), "attn_fused")
     return out
 
 
@@ -161,6 +169,7 @@ def attn_fused_varlen(q, k, v, batch_size: int, max_seq_len: int, seq_len_list, 
                                          info.lens.data_ptr(), None, batch_size, H, int(max_seq_len),
                                          int(max_seq_len), D, arr(*qs), arr(*ks), arr(*vs), arr(0, D, H * D), cu, cu,
                                          scale, int(bool(causal)), _lib.dtype_tag(q, "attn_fused_varlen"),
+                                         info.tile_table(H, int(max_seq_len)).data_ptr(),
                                          _lib.stream_of(q)), "attn_fused_varlen")
     return out
 
@@ -195,7 +204,8 @@ def attn_qk_varlen(q, k, batch_size: int, max_seq_len: int, seq_len_list, *, alp
     with _lib.device_guard(q):
         _lib.check(_lib.fn.en_attn_qk(q.data_ptr(), k.data_ptr(), out.data_ptr(), info.lens.data_ptr(), None, B, H, S, S, D,
                                       *qs, *ks, float(alpha), int(bool(causal)), _lib.dtype_tag(q, "attn_qk_varlen"), cu, cu,
-                                      int(bool(packed_scores)), _lib.stream_of(q)), "attn_qk_varlen")
+                                      int(bool(packed_scores)), info.tile_table(H, S).data_ptr(),
+                                      _lib.stream_of(q)), "attn_qk_varlen")
     return out
 
 
@@ -233,7 +243,8 @@ def attn_pv_varlen(p, v, batch_size: int, max_seq_len: int, seq_len_list, *, cau
     with _lib.device_guard(v):
         _lib.check(_lib.fn.en_attn_pv(p.data_ptr(), v.data_ptr(), out.data_ptr(), info.lens.data_ptr(), None, B, H, S, S, D,
                                       *vs, 0, D, H * D, int(bool(causal)), 0, _lib.dtype_tag(v, "attn_pv_varlen"), cu, cu,
-                                      int(bool(packed_scores)), _lib.stream_of(v)), "attn_pv_varlen")
+                                      int(bool(packed_scores)), info.tile_table(H, S).data_ptr(),
+                                      _lib.stream_of(v)), "attn_pv_varlen")
     return out
 
 

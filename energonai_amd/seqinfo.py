@@ -22,7 +22,8 @@ _CACHE_SIZE = 16
 class SeqInfo:
     """Device-resident int32 lengths and exclusive prefix for one batch."""
 
-    __slots__ = ("lens", "cu_seqlens", "batch_size", "_total", "_source", "_row_offsets", "_ready", "_ordered")
+    __slots__ = ("lens", "cu_seqlens", "batch_size", "_total", "_source", "_row_offsets", "_tile_tables", "_ready",
+                 "_ordered")
 
     def __init__(self, lens: torch.Tensor, cu_seqlens: torch.Tensor, batch_size: int, total: Optional[int], source):
         self.lens = lens                # int32 [B] on the device
@@ -31,6 +32,7 @@ class SeqInfo:
         self._total = total
         self._source = source           # keeps the caller's tensor alive while cached
         self._row_offsets = {}          # (max_seq_len, left_padded) -> int32 [T]
+        self._tile_tables = {}          # (head_num, q_seq_len) -> int32 workgroup order of the attention kernels
         self._ready = []                # events recorded behind the kernels that produced the arrays above
         self._ordered = set()           # raw streams already ordered behind every event of _ready
 
@@ -86,6 +88,24 @@ class SeqInfo:
                 self.produced_on_current_stream()
             self._row_offsets[key] = off
         return off
+
+
+    def tile_table(self, head_num: int, q_seq_len: int) -> torch.Tensor:
+        """Workgroup order of the attention kernels for this batch (``en_attn_tile_table``): the query tiles the
+        sequences really have, longest sequence first.  Computed once per batch, head count and bucket by one
+        small kernel and reused by every layer."""
+        key = (int(head_num), int(q_seq_len))
+        tab = self._tile_tables.get(key)
+        self.order_current_stream()
+        if tab is None:
+            n = int(_lib.fn.en_attn_tile_table_elems(self.batch_size, key[0], key[1]))
+            tab = torch.empty(max(n, 1), dtype=torch.int32, device=self.lens.device)
+            with _lib.device_guard(self.lens):
+                _lib.check(_lib.fn.en_attn_tile_table(self.lens.data_ptr(), self.batch_size, key[0], key[1],
+                                                      tab.data_ptr(), _lib.stream_of(self.lens)), "attn_tile_table")
+                self.produced_on_current_stream()
+            self._tile_tables[key] = tab
+        return tab
 
 
 _cache: "OrderedDict[tuple, SeqInfo]" = OrderedDict()

@@ -199,12 +199,14 @@ int en_layernorm_fwd(void *out, float *mean, float *invvar, void *sum_out, const
  * back to back (the [1,T,H,3D] projection output of examples/bert/bert.py:100) and batch b starts at that row
  * (give stride_b = 0, stride_s = the token pitch): the contraction then needs no transpose_pad before it.
  * packed_scores != 0 (causal self-attention only: q_lens NULL, q_seq_len == k_seq_len; 16-bit dtypes): scores
- * are written in the packed layout of en_packed_scores_elems instead of [B,H,Sq,Sk]. */
+ * are written in the packed layout of en_packed_scores_elems instead of [B,H,Sq,Sk].
+ * tile_table (device, from en_attn_tile_table for the same k_lens, batch, head_num and q_seq_len, or NULL; q_lens
+ * must be NULL with it): the order of the workgroups of the launch; same results, a shorter end of the launch. */
 int en_attn_qk(const void *q, const void *k, void *scores, const int32_t *k_lens, const int32_t *q_lens, int batch,
                int head_num, int q_seq_len, int k_seq_len, int size_per_head, int64_t q_stride_b,
                int64_t q_stride_h, int64_t q_stride_s, int64_t k_stride_b, int64_t k_stride_h, int64_t k_stride_s,
                float alpha, int causal, int dtype, const int32_t *q_row_offsets, const int32_t *k_row_offsets,
-               int packed_scores, en_stream_t stream);
+               int packed_scores, const int32_t *tile_table, en_stream_t stream);
 
 /* ctx[b,h,i,:] = sum_j p[b,h,i,j] * v[b,h,j,:]  (examples/bert/bert.py:119,
  * examples/gpt/gpt.py:125) over j < visible(i) only; p contiguous [B,H,Sq,Sk]
@@ -214,12 +216,13 @@ int en_attn_qk(const void *q, const void *k, void *scores, const int32_t *k_lens
  * zero_padding != 0 and left untouched otherwise.
  * c_row_offsets / v_row_offsets as q_row_offsets / k_row_offsets of en_attn_qk: with c_row_offsets the context is
  * written as packed [T,H,D] rows (strides 0, D, H*D), which is what transpose_depad would produce
- * (zero_padding must then be 0: a packed tensor has no padding rows).  packed_scores as in en_attn_qk. */
+ * (zero_padding must then be 0: a packed tensor has no padding rows).  packed_scores and tile_table as in
+ * en_attn_qk (the table is not used when zero_padding != 0). */
 int en_attn_pv(const void *p, const void *v, void *ctx, const int32_t *k_lens, const int32_t *q_lens, int batch,
                int head_num, int q_seq_len, int k_seq_len, int size_per_head, int64_t v_stride_b,
                int64_t v_stride_h, int64_t v_stride_s, int64_t c_stride_b, int64_t c_stride_h, int64_t c_stride_s,
                int causal, int zero_padding, int dtype, const int32_t *c_row_offsets, const int32_t *v_row_offsets,
-               int packed_scores, en_stream_t stream);
+               int packed_scores, const int32_t *tile_table, en_stream_t stream);
 
 /* Single-query forms of the two contractions for cached decode (one new token
  * per sequence against a ragged cache; the reference recomputes the whole
@@ -259,12 +262,22 @@ int en_kv_append(const void *k_new, const void *v_new, void *k_cache, void *v_ca
  * lengths; batch b then starts at row offsets[b] (give stride[0] = 0), so neither
  * transpose_pad before nor transpose_depad after is needed; q_seq_len / k_seq_len
  * are then upper bounds of the lengths.  Null offsets select the padded layout.
- * scale must be positive.  Rows i >= q_lens[b] of ctx are left untouched.  fp16 / bf16, fp32 accumulation and statistics; D a multiple of 8, D <= 128. */
+ * scale must be positive.  Rows i >= q_lens[b] of ctx are left untouched.  fp16 / bf16, fp32 accumulation and statistics; D a multiple of 8, D <= 128.
+ * tile_table as in en_attn_qk. */
 int en_attn_fused(const void *q, const void *k, const void *v, void *ctx, const int32_t *k_lens,
                   const int32_t *q_lens, int batch, int head_num, int q_seq_len, int k_seq_len, int size_per_head,
                   const int64_t *q_strides, const int64_t *k_strides, const int64_t *v_strides,
                   const int64_t *c_strides, const int32_t *q_row_offsets, const int32_t *k_row_offsets, float scale,
-                  int causal, int dtype, en_stream_t stream);
+                  int causal, int dtype, const int32_t *tile_table, en_stream_t stream);
+
+/* Workgroup order for en_attn_qk, en_attn_pv and en_attn_fused on one batch of sequences (no counterpart in the
+ * reference, whose callers run torch.matmul): table gets en_attn_tile_table_elems(batch, head_num, q_seq_len) int32
+ * entries that list the 128-row query tiles the sequences really have (min(seq_lens[b], q_seq_len) rows each), the
+ * longest sequence first, so that the launch wastes no workgroup slots on tiles past a sequence's end and its long
+ * workgroups start first.  Built once per batch and reused by every layer; one small kernel on `stream`. */
+int64_t en_attn_tile_table_elems(int batch, int head_num, int q_seq_len);
+int en_attn_tile_table(const int32_t *seq_lens, int batch, int head_num, int q_seq_len, int32_t *table,
+                       en_stream_t stream);
 
 /* ---- measurement helper ------------------------------------------------- */
 
@@ -283,14 +296,16 @@ int en_attn_fused(const void *q, const void *k, const void *v, void *ctx, const 
  * qkv_padded and ctx unused), 4 = form 3 with the scores in the packed causal layout
  * (causal, 16-bit dtypes; scores needs en_packed_scores_elems elements).  fold_depad_offsets (en_padding_offsets of this
  * batch, or NULL): if given, depad is not run and x_packed may be NULL; the LayerNorm takes
- * its residual rows straight from hidden_padded.  gamma/beta in the activation dtype. */
+ * its residual rows straight from hidden_padded.  gamma/beta in the activation dtype.  tile_table
+ * (en_attn_tile_table for seq_lens, batch, head_num, max_seq_len, or NULL) is handed to the attention kernels of
+ * forms 1 to 4. */
 int en_padding_removal_layer(const void *hidden_padded, const void *qkv_packed, const void *dense_out,
                              const void *gamma, const void *beta, void *x_packed, void *qkv_padded, void *scores,
                              void *ctx, void *ctx_packed, void *y, const int32_t *cu_seqlens,
                              const int32_t *seq_lens, int batch, int max_seq_len, int head_num, int size_per_head,
                              int64_t hidden, int64_t total_tokens, float scale, float eps, int causal,
                              int left_padded, int attention_form, const int32_t *fold_depad_offsets, int dtype,
-                             en_stream_t stream);
+                             const int32_t *tile_table, en_stream_t stream);
 
 /* en_padding_removal_layer for callers that cannot allocate device memory: code under HIP graph capture,
  * tight serving loops, harnesses that forbid hipMalloc.  It has no counterpart in the reference.  Every

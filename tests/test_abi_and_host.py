@@ -76,11 +76,16 @@ def test_entry_points_validate_before_launch():
     assert lib.en_layernorm_fwd(16, None, None, None, 32, None, 80, 48, 64, 1, 8, 1e-5, 1, 1, None) == -1   # offsets, no residual
     assert lib.en_padding_offsets(16, 0, 8, 0, 32, None) == -2           # batch 0
     assert lib.en_attn_qk(16, 32, 48, 64, None, 1, 1, 8, 8, 200, 0, 0, 200, 0, 0, 200, 1.0, 1, 1, None, None, 0,
-                          None) == -5                                    # D > 128
+                          None, None) == -5                              # D > 128
     assert lib.en_attn_qk(16, 32, 48, 64, None, 1, 1, 8, 8, 64, 0, 0, 64, 0, 0, 64, 1.0, 0, 1, None, None, 1,
-                          None) == -5                                    # packed scores are those of a causal mask
+                          None, None) == -5                              # packed scores are those of a causal mask
+    assert lib.en_attn_qk(16, 32, 48, 64, 80, 1, 1, 8, 8, 64, 0, 0, 64, 0, 0, 64, 1.0, 1, 1, None, None, 0,
+                          96, None) == -5                                # a tile table is built from the key lengths alone
     assert lib.en_attn_pv(16, 32, 48, 64, None, 1, 1, 8, 8, 64, 0, 0, 64, 0, 0, 64, 1, 1, 1, 80, None, 0,
-                          None) == -5                                    # a packed context has no padding rows to zero
+                          None, None) == -5                              # a packed context has no padding rows to zero
+    assert lib.en_attn_tile_table_elems(16, 56, 1024) == 16 * 56 * 8 and lib.en_attn_tile_table_elems(3, 3, 130) == 16 * 2
+    assert lib.en_attn_tile_table(None, 1, 1, 8, 16, None) == -1
+    assert lib.en_attn_tile_table(16, 0, 1, 8, 32, None) == -2
     assert lib.en_packed_scores_elems(2, 3, 16, 1) == 2 * 3 * 16 * 64 and lib.en_packed_scores_elems(1, 1, 130, 1) == 64 * (64 * 3 + 2 * 3) and lib.en_packed_scores_elems(0, 3, 16, 1) == 0
     assert lib.en_scale_mask_softmax_packed(16, 32, 1, 1, 4096, 1.0, 1, None) == -5     # rows of more than 256 vectors
     assert lib.en_copy_bytes(16, 32, 24, None) == -2                     # not a multiple of 16
@@ -92,17 +97,17 @@ def test_entry_points_validate_before_launch():
     assert lib.en_kv_append(16, 32, 48, 64, None, 1, 1, 1, 8, 8, 8, 8, 8, 8, 2, None) == -1
     assert lib.en_kv_append(16, 32, 48, 64, 80, 1, 1, 1, 8, 8, 8, 8, 8, 8, 3, None) == -3   # element size 3
     assert lib.en_attn_fused(16, 32, 48, 64, 80, None, 1, 1, 8, 8, 64, i64x3, i64x3, i64x3, i64x3, None, None, 1.0, 1, 0,
-                             None) == -3                                 # fp32 is not a fused-attention dtype
+                             None, None) == -3                           # fp32 is not a fused-attention dtype
     assert lib.en_attn_fused(16, 32, 48, 64, 80, None, 1, 1, 8, 8, 64, i64x3, i64x3, i64x3, i64x3, None, None, 0.0, 1, 1,
-                             None) == -5                                 # scale must be positive
+                             None, None) == -5                           # scale must be positive
     assert lib.en_attn_fused(16, 32, 48, 64, 80, None, 1, 1, 8, 8, 200, i64x3, i64x3, i64x3, i64x3, None, None, 1.0, 1, 1,
-                             None) == -5                                 # head size above 128
+                             None, None) == -5                           # head size above 128
     assert lib.en_padding_removal_layer(16, 32, None, 48, 64, 80, 96, 112, 128, 144, 160, 176, 192, 1, 8, 2, 8, 16, 4,
-                                        1.0, 1e-5, 1, 0, 5, None, 1, None) == -5   # unknown attention form
+                                        1.0, 1e-5, 1, 0, 5, None, 1, None, None) == -5   # unknown attention form
     assert lib.en_padding_removal_layer(16, 32, None, 48, 64, 80, 96, 112, 128, 144, 160, 176, 192, 1, 8, 2, 8, 32, 4,
-                                        1.0, 1e-5, 1, 0, 0, None, 1, None) == -2   # LayerNorm width 32 != 2 heads x 8, no dense_out
+                                        1.0, 1e-5, 1, 0, 0, None, 1, None, None) == -2   # LayerNorm width 32 != 2 heads x 8, no dense_out
     assert lib.en_padding_removal_layer(16, 32, None, 48, 64, 80, None, 112, 128, 144, 160, 176, 192, 1, 8, 2, 8, 16, 4,
-                                        1.0, 1e-5, 1, 0, 0, None, 1, None) == -1   # unfused form without the padded buffer
+                                        1.0, 1e-5, 1, 0, 0, None, 1, None, None) == -1   # unfused form without the padded buffer
 
 
 def test_python_api_keeps_reference_names_and_signatures():

@@ -510,3 +510,75 @@ def test_contractions_on_packed_tokens_match_the_padded_route(dtype, causal, B, 
     elif dtype == torch.float32 or not causal:
         with pytest.raises(RuntimeError):
             k.attn_qk_varlen(q, kk, B, S, lens_t, causal=causal, packed_scores=True)
+
+
+@pytest.mark.parametrize("B,H,S,lens", [(16, 7, 1000, None), (3, 12, 130, [130, 0, 77]), (9, 1, 2048, None),
+                                        (1, 1, 8, [5])])
+def test_attn_tile_table_lists_every_real_query_tile_once_longest_sequence_first(B, H, S, lens):
+    """en_attn_tile_table: workgroup w of a launch finds unit * ntq + query tile or -1.  Every 128-row query tile a
+    sequence really has appears exactly once, tiles past a sequence's end never; a unit stays on one XCD (w % 8);
+    its tiles run from the last to the first; sequences come in the order of decreasing length."""
+    from energonai_amd import _lib
+    from energonai_amd.seqinfo import build_seq_info
+    if lens is None:
+        g = torch.Generator().manual_seed(B * 31 + S)
+        lens = torch.randint(0, S + 40, (B,), generator=g).tolist()      # some longer than the bucket
+    announce("tile table", B, H, S, lens)
+    info = build_seq_info(torch.tensor(lens, dtype=torch.int32), B)
+    tab = info.tile_table(H, S).cpu().tolist()
+    ntq = -(-S // 128)
+    assert len(tab) == _lib.fn.en_attn_tile_table_elems(B, H, S) == -(-B * H // 8) * 8 * ntq
+    want = {(b * H + h) * ntq + qi for b in range(B) for h in range(H) for qi in range(-(-min(lens[b], S) // 128))}
+    got = [c for c in tab if c >= 0]
+    assert len(got) == len(set(got)) and set(got) == want
+    assert all(c >= -1 for c in tab)
+    where = {}
+    for w, c in enumerate(tab):
+        if c >= 0:
+            where.setdefault(c // ntq, []).append((w, c % ntq))
+    first = {}
+    for unit, entries in where.items():
+        assert len({w % 8 for w, _ in entries}) == 1                     # one XCD per unit
+        assert [qi for _, qi in entries] == sorted((qi for _, qi in entries), reverse=True)
+        first[unit] = entries[0][0]
+    # of two units on the same XCD the one of the longer sequence starts earlier
+    units = sorted(first, key=lambda u: first[u])
+    for x in range(8):
+        seq = [min(lens[u // H], S) for u in units if first[u] % 8 == x]
+        assert seq == sorted(seq, reverse=True)
+
+
+@pytest.mark.parametrize("causal", [True, False])
+def test_attention_kernels_give_the_same_bits_with_and_without_a_tile_table(causal):
+    """The table only reorders the workgroups of a launch."""
+    import ctypes
+    from energonai_amd import _lib
+    from energonai_amd.seqinfo import build_seq_info
+    B, H, S, D = 5, 3, 520, 128
+    lens = [520, 3, 0, 257, 128]
+    announce("tile table on/off", causal)
+    dtype = torch.float16
+    g = torch.Generator().manual_seed(77)
+    q, kk, v = (torch.randn(B, H, S, D, generator=g).to(dtype).cuda() for _ in range(3))
+    info = build_seq_info(torch.tensor(lens, dtype=torch.int32), B)
+    tab = info.tile_table(H, S)
+    strides = (H * S * D, S * D, D)
+    arr = (ctypes.c_int64 * 3)(*strides)
+    stream = _lib.stream_of(q)
+    outs = []
+    for t in (None, tab.data_ptr()):
+        scores = torch.zeros(B, H, S, S, dtype=dtype, device="cuda")
+        ctx = torch.zeros(B, H, S, D, dtype=dtype, device="cuda")
+        fused = torch.zeros(B, H, S, D, dtype=dtype, device="cuda")
+        _lib.check(_lib.fn.en_attn_qk(q.data_ptr(), kk.data_ptr(), scores.data_ptr(), info.lens.data_ptr(), None, B, H, S,
+                                      S, D, *strides, *strides, 1.0, int(causal), 1, None, None, 0, t, stream), "qk")
+        probs = _kernel().scale_mask_softmax(B, S, H, scores, info, scale=D ** -0.5, causal=causal, tail_rows=1)
+        _lib.check(_lib.fn.en_attn_pv(probs.data_ptr(), v.data_ptr(), ctx.data_ptr(), info.lens.data_ptr(), None, B, H, S,
+                                      S, D, *strides, *strides, int(causal), 0, 1, None, None, 0, t, stream), "pv")
+        _lib.check(_lib.fn.en_attn_fused(q.data_ptr(), kk.data_ptr(), v.data_ptr(), fused.data_ptr(), info.lens.data_ptr(),
+                                         None, B, H, S, S, D, arr, arr, arr, arr, None, None, D ** -0.5, int(causal), 1,
+                                         t, stream), "fused")
+        outs.append((probs.clone(), ctx, fused))
+    for a, b in zip(*outs):
+        assert torch.equal(a, b)
+    assert bool(outs[0][2].any())
