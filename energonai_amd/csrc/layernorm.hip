@@ -48,8 +48,17 @@ __global__ __launch_bounds__(TPR < kBlock ? kBlock : TPR) void layernorm_rows_ke
 
   const int nvec = a.n2 / EPV;
   const TI *in = reinterpret_cast<const TI *>(a.in) + row * a.n2;
-  const TI *res = a.residual ? reinterpret_cast<const TI *>(a.residual) + (row + (a.res_off ? a.res_off[row] : 0)) * a.n2 : nullptr;
   TI *sum_out = a.sum_out ? reinterpret_cast<TI *>(a.sum_out) + row * a.n2 : nullptr;
+
+  // The row's own loads go out first: where the residual row is found through res_off, its address hangs on a
+  // load of its own, and loads issue in order -- placed first it would hold the others back for its whole latency.
+  uint4 raw[VPL];
+#pragma unroll
+  for (int j = 0; j < VPL; ++j) {
+    const int v = t + TPR * j;
+    raw[j] = (v < nvec) ? load16<STREAM_LD>(in + v * EPV) : make_uint4(0u, 0u, 0u, 0u);
+  }
+  const TI *res = a.residual ? reinterpret_cast<const TI *>(a.residual) + (row + (a.res_off ? a.res_off[row] : 0)) * a.n2 : nullptr;
 
   float x[VPL][EPV];
   float s = 0.f;
@@ -57,7 +66,7 @@ __global__ __launch_bounds__(TPR < kBlock ? kBlock : TPR) void layernorm_rows_ke
   for (int j = 0; j < VPL; ++j) {
     const int v = t + TPR * j;
     if (v < nvec) {
-      const Pack<TI, EPV> pk = __builtin_bit_cast(Pack<TI, EPV>, load16<STREAM_LD>(in + v * EPV));
+      const Pack<TI, EPV> pk = __builtin_bit_cast(Pack<TI, EPV>, raw[j]);
 #pragma unroll
       for (int e = 0; e < EPV; ++e) x[j][e] = EI::to_float(pk.v[e]);
       if (res) {
