@@ -6,7 +6,8 @@
     python3 bench_profiles.py counters --workload c3     # one --pmc run of SQ counters: MFMA and VALU busy, LDS, waits
 
 Each sub-command starts rocprofv3 as a child process with `python3 bench.py ...` after `--`, reads the CSV files it
-leaves under gpurun_out/prof/, and prints a markdown summary (redirect it into profiles/bench_<workload>_*.md).
+leaves in a scratch directory (--raw-dir, default: a fresh temporary one), and prints a markdown summary (redirect it
+into profiles/bench_<workload>_*.md).
 `--step-only` makes bench.py launch nothing but the step and the kernels of the step, each op the same number of
 times, so every kernel name in a trace is one op of one workload.
 
@@ -23,9 +24,10 @@ import json
 import os
 import subprocess
 import sys
+import tempfile
 
 ROOT = os.path.dirname(os.path.abspath(__file__))
-OUT = os.path.join(ROOT, "gpurun_out", "prof")
+OUT = None      # where rocprofv3 leaves its raw files: --raw-dir, or a temporary directory made on first use
 
 # kernel name (substring) -> the op's key in the bench line; first match wins
 KERNEL_KEYS = [
@@ -51,7 +53,10 @@ def key_of(kernel: str, decode: bool):
 
 
 def run_profiler(tag: str, prof_args, bench_args, timeout_s: int):
-    """rocprofv3 <prof_args> -d gpurun_out/prof/<tag> -- python3 bench.py <bench_args>; returns (dir, bench line)."""
+    """rocprofv3 <prof_args> -d <raw dir>/<tag> -- python3 bench.py <bench_args>; returns (dir, bench line, command)."""
+    global OUT
+    if OUT is None:
+        OUT = tempfile.mkdtemp(prefix="energon_prof_")
     d = os.path.join(OUT, tag)
     subprocess.run(["rm", "-rf", d], check=True)
     os.makedirs(d, exist_ok=True)
@@ -235,10 +240,13 @@ def main(argv=None) -> int:
         p.add_argument("--steps", type=int, default=20)
         p.add_argument("--warmup", type=int, default=5)
         p.add_argument("--timeout", type=int, default=300, help="seconds allowed for each rocprofv3 run")
+        p.add_argument("--raw-dir", default=None, help="directory for rocprofv3's raw output (default: a temporary one)")
         if name == "counters":
             p.add_argument("--all-ops", action="store_true", help="every op of the bench line, not the step alone")
         p.set_defaults(fn=fn)
     ns = ap.parse_args(argv)
+    global OUT
+    OUT = ns.raw_dir
     return ns.fn(ns)
 
 
