@@ -35,6 +35,14 @@ ATTN_CASES = [
     (2, 2, 384, 32, [300, 1]),           # head dim below the tile's 64
     (1, 2, 520, 80, [515]),              # OPT-2.7B head dim: padded to 128 inside the kernel
     (9, 1, 130, 128, [130, 5, 64, 65, 127, 128, 129, 1, 33]),   # more units than XCDs, odd split
+    # head sizes between the two tile widths: the 16-byte chunks past the head must arrive as zeros, for every
+    # remainder and in each of the swizzled slot positions
+    (2, 1, 200, 72, [200, 131]),
+    (1, 3, 136, 96, [133]),
+    (2, 2, 264, 104, [264, 9]),
+    (1, 1, 328, 120, [321]),
+    (2, 2, 136, 40, [136, 70]),
+    (1, 2, 72, 8, [65]),
 ]
 
 
@@ -582,3 +590,27 @@ def test_attention_kernels_give_the_same_bits_with_and_without_a_tile_table(caus
     for a, b in zip(*outs):
         assert torch.equal(a, b)
     assert bool(outs[0][2].any())
+
+
+def test_attn_tile_table_of_a_batch_beyond_the_sort_limit_keeps_the_batch_order():
+    """More than 1024 sequences: the table still lists every real tile once (in batch order)."""
+    from energonai_amd.seqinfo import build_seq_info
+    B, H, S = 1100, 1, 200
+    g = torch.Generator().manual_seed(5)
+    lens = torch.randint(0, S + 1, (B,), generator=g).tolist()
+    announce("tile table, large batch", B)
+    info = build_seq_info(torch.tensor(lens, dtype=torch.int32), B)
+    tab = info.tile_table(H, S).cpu().tolist()
+    ntq = 2
+    want = {b * ntq + qi for b in range(B) for qi in range(-(-lens[b] // 128))}
+    got = [c for c in tab if c >= 0]
+    assert len(got) == len(set(got)) and set(got) == want
+    # and the kernels run with it
+    D = 32
+    q, kk, v = (torch.randn(B, H, S, D, generator=g).half().cuda() for _ in range(3))
+    ctx = _kernel().attn_fused(q, kk, v, info, causal=True).cpu().float()
+    b = max(range(B), key=lambda i: lens[i])
+    n = lens[b]
+    ref = torch.nn.functional.scaled_dot_product_attention(q[b:b + 1, :, :n].float().cpu(), kk[b:b + 1, :, :n].float().cpu(),
+                                                           v[b:b + 1, :, :n].float().cpu(), is_causal=True)
+    assert max_abs(ctx[b:b + 1, :, :n], ref) <= 2e-3 * max(1.0, float(ref.abs().max()))
