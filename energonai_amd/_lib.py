@@ -47,7 +47,7 @@ SIGNATURES = {
     "en_attn_pv": (c_int, [c_void_p] * 5 + [c_int] * 5 + [c_int64] * 6 + [c_int, c_int, c_int, c_void_p, c_void_p,
                            c_int, c_void_p, c_void_p]),
     "en_attn_tile_table_elems": (c_int64, [c_int] * 3),
-    "en_attn_tile_table": (c_int, [c_void_p, c_int, c_int, c_int, c_void_p, c_void_p]),
+    "en_attn_tile_table": (c_int, [c_void_p, c_int, c_int, c_int, c_int, c_void_p, c_void_p]),
     "en_packed_scores_elems": (c_int64, [c_int] * 4),
     "en_scale_mask_softmax_packed": (c_int, [c_void_p, c_void_p, c_int, c_int, c_int, c_float, c_int, c_void_p]),
     "en_decode_qk": (c_int, [c_void_p] * 4 + [c_int] * 4 + [c_int64] * 3 + [c_float, c_int, c_void_p]),

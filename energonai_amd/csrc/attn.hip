@@ -735,12 +735,17 @@ __global__ __launch_bounds__(kBlock, 3) void attn_pv_strip_kernel(AttnArgs a) {
 // ===========================================================================
 // table[w] for workgroup w of a launch of ceil(B H / 8) * 8 * ntq workgroups.  Workgroups go to the XCDs round-robin,
 // so entries w = 8 j + x are XCD x's sequence: the (batch, head) units are dealt to the XCDs in the order of
-// decreasing sequence length (units of one sequence on consecutive XCDs), each unit's query tiles follow one another
-// from the last (longest under a causal mask) to the first, and tiles past a sequence's end get no entry.  What is
-// left of the table is -1.  One workgroup; the sort is a rank count (batch <= 1024), larger batches keep their order.
+// decreasing sequence length (units of one sequence on consecutive XCDs), and tiles past a sequence's end get no
+// entry; what is left of the table is -1.  Within an XCD either
+//   unit by unit, each unit's query tiles from the last (longest under a causal mask) to the first
+//     (tiles_first == 0): the tiles of a unit run together and share its K and V in the XCD's L2; or
+//   tile index by tile index from the last to the first, every unit that has the tile (tiles_first == 1): the
+//     long workgroups of all units start first -- the better schedule when a unit's K and V are small enough
+//     to be re-read cheaply (512-key, 64-channel units: 21.3 -> 19.6 us; 1024 x 128: 213 -> 225 us).
+// One workgroup; the sort is a rank count (batch <= 1024), larger batches keep their order.
 __global__ __launch_bounds__(1024) void attn_tile_table_kernel(const int32_t *__restrict__ lens, int batch, int heads,
                                                                int seq_len, int ntq, int32_t *__restrict__ table,
-                                                               int capacity) {
+                                                               int capacity, int tiles_first) {
   __shared__ int32_t s_len[1024];
   __shared__ int32_t s_order[1024];
   const int tid = threadIdx.x;
@@ -759,14 +764,23 @@ __global__ __launch_bounds__(1024) void attn_tile_table_kernel(const int32_t *__
   __syncthreads();   // also orders the -1 fill before the entries written below
   if (tid < kXcds) {
     const int units = batch * heads;
-    int j = 0;
-    for (int u = tid; u < units; u += kXcds) {      // u-th unit in sorted order
+    auto tiles_of = [&](int u, int &unit) {          // u-th unit in sorted order -> its index and tile count
       const int p = u / heads, h = u - p * heads;
       const int b = sorted ? s_order[p] : p;
       const int n = sorted ? s_len[b] : min(max(lens[b], 0), seq_len);
-      const int nt = (n + kQTile - 1) / kQTile;
-      const int unit = b * heads + h;
-      for (int qi = nt - 1; qi >= 0; --qi, ++j) table[j * kXcds + tid] = unit * ntq + qi;
+      unit = b * heads + h;
+      return (n + kQTile - 1) / kQTile;
+    };
+    int j = 0, unit;
+    if (tiles_first) {
+      for (int qi = ntq - 1; qi >= 0; --qi)
+        for (int u = tid; u < units; u += kXcds)
+          if (qi < tiles_of(u, unit)) table[j++ * kXcds + tid] = unit * ntq + qi;
+    } else {
+      for (int u = tid; u < units; u += kXcds) {
+        const int nt = tiles_of(u, unit);
+        for (int qi = nt - 1; qi >= 0; --qi) table[j++ * kXcds + tid] = unit * ntq + qi;
+      }
     }
   }
 }
@@ -879,15 +893,15 @@ int64_t en_attn_tile_table_elems(int batch, int head_num, int q_seq_len) {
   return ceil_div((int64_t)batch * head_num, (int64_t)kXcds) * kXcds * ceil_div(q_seq_len, kQTile);
 }
 
-int en_attn_tile_table(const int32_t *seq_lens, int batch, int head_num, int q_seq_len, int32_t *table,
-                       en_stream_t stream) {
+int en_attn_tile_table(const int32_t *seq_lens, int batch, int head_num, int q_seq_len, int tiles_first,
+                       int32_t *table, en_stream_t stream) {
   using namespace en;
   if (!seq_lens || !table) return EN_ERR_NULL;
   if (batch < 1 || head_num < 1 || q_seq_len < 1) return EN_ERR_SHAPE;
   const int64_t cap = en_attn_tile_table_elems(batch, head_num, q_seq_len);
   if (cap > INT32_MAX || (int64_t)batch * head_num > INT32_MAX / 64) return EN_ERR_SHAPE;
   attn_tile_table_kernel<<<1, 1024, 0, (hipStream_t)stream>>>(seq_lens, batch, head_num, q_seq_len,
-                                                               (int)ceil_div(q_seq_len, kQTile), table, (int)cap);
+                                                               (int)ceil_div(q_seq_len, kQTile), table, (int)cap, tiles_first ? 1 : 0);
   EN_RETURN_IF_LAUNCH_FAILED();
   return EN_OK;
 }

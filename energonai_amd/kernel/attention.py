@@ -37,9 +37,14 @@ def _lens_ptrs(seq_len_list, q_len_list, batch_size, device):
     return k_info, q_info, (0 if q_info is None else q_info.lens.data_ptr())
 
 
-def _tile_table_ptr(k_info, q_ptr, head_num: int, q_seq_len: int):
+def _unit_kv_bytes(k_seq_len: int, size_per_head: int, t: torch.Tensor) -> int:
+    """Bytes of one (batch, head) unit's K and V at full length: picks the workgroup order (SeqInfo.tile_table)."""
+    return 2 * int(k_seq_len) * int(size_per_head) * t.element_size()
+
+
+def _tile_table_ptr(k_info, q_ptr, head_num: int, q_seq_len: int, unit_kv_bytes: int):
     """Workgroup order for the batch (cached in its SeqInfo) when the query lengths are the key lengths."""
-    return None if q_ptr is not None else k_info.tile_table(head_num, q_seq_len).data_ptr()
+    return None if q_ptr is not None else k_info.tile_table(head_num, q_seq_len, unit_kv_bytes).data_ptr()
 
 
 def attn_qk(q, k, seq_len_list, *, alpha: float = 1.0, causal: bool = True, q_len_list=None,
@@ -67,7 +72,7 @@ def attn_qk(q, k, seq_len_list, *, alpha: float = 1.0, causal: bool = True, q_le
         _lib.check(_lib.fn.en_attn_qk(q.data_ptr(), k.data_ptr(), out.data_ptr(), k_info.lens.data_ptr(), q_ptr,
                                           B, H, Sq, Sk, D, *qs, *ks, float(alpha), int(bool(causal)),
                                           _lib.dtype_tag(q, "attn_qk"), None, None, 0,
-                                          _tile_table_ptr(k_info, q_ptr, H, Sq), _lib.stream_of(q)), "attn_qk")
+                                          _tile_table_ptr(k_info, q_ptr, H, Sq, _unit_kv_bytes(Sk, D, q)), _lib.stream_of(q)), "attn_qk")
     return out
 
 
@@ -97,7 +102,7 @@ def attn_pv(p, v, seq_len_list, *, causal: bool = True, q_len_list=None, zero_pa
         _lib.check(_lib.fn.en_attn_pv(p.data_ptr(), v.data_ptr(), out.data_ptr(), k_info.lens.data_ptr(), q_ptr,
                                           B, H, Sq, Sk, D, *vs, *cs, int(bool(causal)), int(bool(zero_padding)),
                                           _lib.dtype_tag(p, "attn_pv"), None, None, 0,
-                                          _tile_table_ptr(k_info, q_ptr, H, Sq), _lib.stream_of(p)), "attn_pv")
+                                          _tile_table_ptr(k_info, q_ptr, H, Sq, _unit_kv_bytes(Sk, D, p)), _lib.stream_of(p)), "attn_pv")
     return out
 
 
@@ -132,7 +137,7 @@ def attn_fused(q, k, v, seq_len_list, *, scale: Optional[float] = None, causal: 
         _lib.check(_lib.fn.en_attn_fused(q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(),
                                          k_info.lens.data_ptr(), q_ptr, B, H, Sq, Sk, D, arr(*qs), arr(*ks), arr(*vs),
                                          arr(*cs), None, None, scale, int(bool(causal)),
-                                         _lib.dtype_tag(q, "attn_fused"), _tile_table_ptr(k_info, q_ptr, H, Sq),
+                                         _lib.dtype_tag(q, "attn_fused"), _tile_table_ptr(k_info, q_ptr, H, Sq, _unit_kv_bytes(Sk, D, q)),
                                          _lib.stream_of(q)), "attn_fused")
     return out
 
@@ -169,7 +174,7 @@ def attn_fused_varlen(q, k, v, batch_size: int, max_seq_len: int, seq_len_list, 
                                          info.lens.data_ptr(), None, batch_size, H, int(max_seq_len),
                                          int(max_seq_len), D, arr(*qs), arr(*ks), arr(*vs), arr(0, D, H * D), cu, cu,
                                          scale, int(bool(causal)), _lib.dtype_tag(q, "attn_fused_varlen"),
-                                         info.tile_table(H, int(max_seq_len)).data_ptr(),
+                                         info.tile_table(H, int(max_seq_len), _unit_kv_bytes(max_seq_len, D, q)).data_ptr(),
                                          _lib.stream_of(q)), "attn_fused_varlen")
     return out
 
@@ -204,7 +209,7 @@ def attn_qk_varlen(q, k, batch_size: int, max_seq_len: int, seq_len_list, *, alp
     with _lib.device_guard(q):
         _lib.check(_lib.fn.en_attn_qk(q.data_ptr(), k.data_ptr(), out.data_ptr(), info.lens.data_ptr(), None, B, H, S, S, D,
                                       *qs, *ks, float(alpha), int(bool(causal)), _lib.dtype_tag(q, "attn_qk_varlen"), cu, cu,
-                                      int(bool(packed_scores)), info.tile_table(H, S).data_ptr(),
+                                      int(bool(packed_scores)), info.tile_table(H, S, _unit_kv_bytes(S, D, q)).data_ptr(),
                                       _lib.stream_of(q)), "attn_qk_varlen")
     return out
 
@@ -243,7 +248,7 @@ def attn_pv_varlen(p, v, batch_size: int, max_seq_len: int, seq_len_list, *, cau
     with _lib.device_guard(v):
         _lib.check(_lib.fn.en_attn_pv(p.data_ptr(), v.data_ptr(), out.data_ptr(), info.lens.data_ptr(), None, B, H, S, S, D,
                                       *vs, 0, D, H * D, int(bool(causal)), 0, _lib.dtype_tag(v, "attn_pv_varlen"), cu, cu,
-                                      int(bool(packed_scores)), info.tile_table(H, S).data_ptr(),
+                                      int(bool(packed_scores)), info.tile_table(H, S, _unit_kv_bytes(S, D, v)).data_ptr(),
                                       _lib.stream_of(v)), "attn_pv_varlen")
     return out
 

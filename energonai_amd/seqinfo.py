@@ -17,6 +17,7 @@ import torch
 from . import _lib
 
 _CACHE_SIZE = 16
+TILES_FIRST_MAX_KV_BYTES = 256 << 10     # see SeqInfo.tile_table
 
 
 class SeqInfo:
@@ -90,18 +91,20 @@ class SeqInfo:
         return off
 
 
-    def tile_table(self, head_num: int, q_seq_len: int) -> torch.Tensor:
+    def tile_table(self, head_num: int, q_seq_len: int, unit_kv_bytes: int = 1 << 30) -> torch.Tensor:
         """Workgroup order of the attention kernels for this batch (``en_attn_tile_table``): the query tiles the
-        sequences really have, longest sequence first.  Computed once per batch, head count and bucket by one
-        small kernel and reused by every layer."""
-        key = (int(head_num), int(q_seq_len))
+        sequences really have, longest sequence first.  ``unit_kv_bytes`` is what one (batch, head) unit's K and V
+        hold at full length: up to 256 KB the last tiles of all units run first, above that a unit's tiles stay
+        together.  Computed once per batch, head count, bucket and order by one small kernel and reused by every
+        layer."""
+        key = (int(head_num), int(q_seq_len), int(unit_kv_bytes) <= TILES_FIRST_MAX_KV_BYTES)
         tab = self._tile_tables.get(key)
         self.order_current_stream()
         if tab is None:
             n = int(_lib.fn.en_attn_tile_table_elems(self.batch_size, key[0], key[1]))
             tab = torch.empty(max(n, 1), dtype=torch.int32, device=self.lens.device)
             with _lib.device_guard(self.lens):
-                _lib.check(_lib.fn.en_attn_tile_table(self.lens.data_ptr(), self.batch_size, key[0], key[1],
+                _lib.check(_lib.fn.en_attn_tile_table(self.lens.data_ptr(), self.batch_size, key[0], key[1], int(key[2]),
                                                       tab.data_ptr(), _lib.stream_of(self.lens)), "attn_tile_table")
                 self.produced_on_current_stream()
             self._tile_tables[key] = tab

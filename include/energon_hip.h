@@ -274,10 +274,13 @@ int en_attn_fused(const void *q, const void *k, const void *v, void *ctx, const 
  * reference, whose callers run torch.matmul): table gets en_attn_tile_table_elems(batch, head_num, q_seq_len) int32
  * entries that list the 128-row query tiles the sequences really have (min(seq_lens[b], q_seq_len) rows each), the
  * longest sequence first, so that the launch wastes no workgroup slots on tiles past a sequence's end and its long
- * workgroups start first.  Built once per batch and reused by every layer; one small kernel on `stream`. */
+ * workgroups start first.  tiles_first == 0 keeps the query tiles of a (batch, head) unit together (they share its
+ * K and V in L2); tiles_first != 0 runs the last tiles of all units first, then the second-to-last ... (the better
+ * order when a unit's K and V are small: about 256 KB or less).  Built once per batch and reused by every layer;
+ * one small kernel on `stream`. */
 int64_t en_attn_tile_table_elems(int batch, int head_num, int q_seq_len);
-int en_attn_tile_table(const int32_t *seq_lens, int batch, int head_num, int q_seq_len, int32_t *table,
-                       en_stream_t stream);
+int en_attn_tile_table(const int32_t *seq_lens, int batch, int head_num, int q_seq_len, int tiles_first,
+                       int32_t *table, en_stream_t stream);
 
 /* ---- measurement helper ------------------------------------------------- */
 

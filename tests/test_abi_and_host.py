@@ -84,8 +84,8 @@ def test_entry_points_validate_before_launch():
     assert lib.en_attn_pv(16, 32, 48, 64, None, 1, 1, 8, 8, 64, 0, 0, 64, 0, 0, 64, 1, 1, 1, 80, None, 0,
                           None, None) == -5                              # a packed context has no padding rows to zero
     assert lib.en_attn_tile_table_elems(16, 56, 1024) == 16 * 56 * 8 and lib.en_attn_tile_table_elems(3, 3, 130) == 16 * 2
-    assert lib.en_attn_tile_table(None, 1, 1, 8, 16, None) == -1
-    assert lib.en_attn_tile_table(16, 0, 1, 8, 32, None) == -2
+    assert lib.en_attn_tile_table(None, 1, 1, 8, 0, 16, None) == -1
+    assert lib.en_attn_tile_table(16, 0, 1, 8, 1, 32, None) == -2
     assert lib.en_packed_scores_elems(2, 3, 16, 1) == 2 * 3 * 16 * 64 and lib.en_packed_scores_elems(1, 1, 130, 1) == 64 * (64 * 3 + 2 * 3) and lib.en_packed_scores_elems(0, 3, 16, 1) == 0
     assert lib.en_scale_mask_softmax_packed(16, 32, 1, 1, 4096, 1.0, 1, None) == -5     # rows of more than 256 vectors
     assert lib.en_copy_bytes(16, 32, 24, None) == -2                     # not a multiple of 16

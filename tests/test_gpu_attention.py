@@ -520,12 +520,15 @@ def test_contractions_on_packed_tokens_match_the_padded_route(dtype, causal, B, 
             k.attn_qk_varlen(q, kk, B, S, lens_t, causal=causal, packed_scores=True)
 
 
+@pytest.mark.parametrize("tiles_first", [False, True])
 @pytest.mark.parametrize("B,H,S,lens", [(16, 7, 1000, None), (3, 12, 130, [130, 0, 77]), (9, 1, 2048, None),
                                         (1, 1, 8, [5])])
-def test_attn_tile_table_lists_every_real_query_tile_once_longest_sequence_first(B, H, S, lens):
+def test_attn_tile_table_lists_every_real_query_tile_once_longest_sequence_first(B, H, S, lens, tiles_first):
     """en_attn_tile_table: workgroup w of a launch finds unit * ntq + query tile or -1.  Every 128-row query tile a
     sequence really has appears exactly once, tiles past a sequence's end never; a unit stays on one XCD (w % 8);
-    its tiles run from the last to the first; sequences come in the order of decreasing length."""
+    its tiles run from the last to the first; sequences come in the order of decreasing length.  In the
+    tiles-first order (units with little K and V) an XCD runs the last tiles of all its units, then the
+    second-to-last ..., the longer sequence first within a tile index."""
     from energonai_amd import _lib
     from energonai_amd.seqinfo import build_seq_info
     if lens is None:
@@ -533,7 +536,7 @@ def test_attn_tile_table_lists_every_real_query_tile_once_longest_sequence_first
         lens = torch.randint(0, S + 40, (B,), generator=g).tolist()      # some longer than the bucket
     announce("tile table", B, H, S, lens)
     info = build_seq_info(torch.tensor(lens, dtype=torch.int32), B)
-    tab = info.tile_table(H, S).cpu().tolist()
+    tab = info.tile_table(H, S, (64 << 10) if tiles_first else (1 << 20)).cpu().tolist()
     ntq = -(-S // 128)
     assert len(tab) == _lib.fn.en_attn_tile_table_elems(B, H, S) == -(-B * H // 8) * 8 * ntq
     want = {(b * H + h) * ntq + qi for b in range(B) for h in range(H) for qi in range(-(-min(lens[b], S) // 128))}
@@ -549,11 +552,20 @@ def test_attn_tile_table_lists_every_real_query_tile_once_longest_sequence_first
         assert len({w % 8 for w, _ in entries}) == 1                     # one XCD per unit
         assert [qi for _, qi in entries] == sorted((qi for _, qi in entries), reverse=True)
         first[unit] = entries[0][0]
-    # of two units on the same XCD the one of the longer sequence starts earlier
-    units = sorted(first, key=lambda u: first[u])
-    for x in range(8):
-        seq = [min(lens[u // H], S) for u in units if first[u] % 8 == x]
-        assert seq == sorted(seq, reverse=True)
+    if tiles_first:
+        # on an XCD the tile indices never grow along the launch, and within one index the longer sequence is first
+        for x in range(8):
+            seq = [(c % ntq, min(lens[(c // ntq) // H], S)) for w, c in enumerate(tab) if c >= 0 and w % 8 == x]
+            assert seq == sorted(seq, key=lambda t: (-t[0], -t[1]))
+    else:
+        # of two units on the same XCD the one of the longer sequence starts earlier, and a unit's tiles are adjacent
+        units = sorted(first, key=lambda u: first[u])
+        for x in range(8):
+            seq = [min(lens[u // H], S) for u in units if first[u] % 8 == x]
+            assert seq == sorted(seq, reverse=True)
+        for unit, entries in where.items():
+            ws = [w for w, _ in entries]
+            assert ws == list(range(ws[0], ws[0] + 8 * len(ws), 8))
 
 
 @pytest.mark.parametrize("causal", [True, False])
