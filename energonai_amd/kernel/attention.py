@@ -44,7 +44,7 @@ def _unit_kv_bytes(k_seq_len: int, size_per_head: int, t: torch.Tensor) -> int:
 
 def _tile_table_ptr(k_info, q_ptr, head_num: int, q_seq_len: int, unit_kv_bytes: int):
     """Workgroup order for the batch (cached in its SeqInfo) when the query lengths are the key lengths."""
-    return None if q_ptr is not None else k_info.tile_table(head_num, q_seq_len, unit_kv_bytes).data_ptr()
+    return None if q_ptr else k_info.tile_table(head_num, q_seq_len, unit_kv_bytes).data_ptr()
 
 
 def attn_qk(q, k, seq_len_list, *, alpha: float = 1.0, causal: bool = True, q_len_list=None,

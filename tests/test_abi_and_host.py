@@ -166,6 +166,29 @@ def test_host_side_argument_errors_without_gpu():
         kernel.depad(torch.zeros(2, 4, 8), 2, lens)
 
 
+def test_public_attention_calls_pass_the_tile_table_when_there_are_no_query_lengths():
+    """attn_qk / attn_pv / attn_fused get the raw pointer of the query lengths as 0 when the caller gives none; the
+    workgroup order of the batch must then be handed to the kernels (it once was not: 0 is not None)."""
+    from energonai_amd.kernel import attention
+
+    class Table:
+        def data_ptr(self):
+            return 4096
+
+    class Info:
+        def __init__(self):
+            self.asked = []
+
+        def tile_table(self, head_num, q_seq_len, unit_kv_bytes):
+            self.asked.append((head_num, q_seq_len, unit_kv_bytes))
+            return Table()
+
+    info = Info()
+    assert attention._tile_table_ptr(info, 0, 12, 512, 1 << 17) == 4096 and info.asked == [(12, 512, 1 << 17)]
+    assert attention._tile_table_ptr(info, None, 12, 512, 1 << 17) == 4096
+    assert attention._tile_table_ptr(info, 0x7f0000001000, 12, 512, 1 << 17) is None and len(info.asked) == 2
+
+
 def test_missing_library_fails_loudly(tmp_path, monkeypatch):
     """No CPU fallback: without the shared object the product refuses to load."""
     from energonai_amd import _lib
