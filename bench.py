@@ -736,12 +736,22 @@ def main(argv=None) -> int:
     dom = max(kt, key=lambda n: kt[n]["us"])
     row = kt[dom]
     if "mfma_frac" in row and dom.startswith("attn_fused"):
-        # fused attention moves 4 T H D bytes and is bound by the matrix and vector pipes, not by HBM
-        roofline = {"kernel": dom, "bound": "mfma", "achieved": row["TFLOPs"], "peak": MFMA_PEAK_TFLOPS[head["dtype"]],
-                    "unit": "TFLOP/s", "frac": row["mfma_frac"],
-                    "traffic": measured_traffic(w.name, ns.form).get(dom), "us_per_launch": row["us"],
-                    "alg_flops_per_launch": row["TFLOPs"] * 1e12 * row["us"] * 1e-6,
-                    "alg_bytes_per_launch": row["alg_MB"] * 1e6, "hbm_frac": row["hbm_frac"]}
+        # fused attention reads q, k, v and writes ctx (4 T H D e bytes) and does 4 D FLOPs per visible score: which roof
+        # bounds it follows from its FLOPs per byte against the machine's (peak FLOP/s over peak bytes/s); c3 (short
+        # sequences, 170 FLOP/B against 312) sits under the HBM roof, c4 (355 FLOP/B) under the matrix roof.  Both
+        # fractions are in the line whichever one `frac` is.
+        peak_tf = MFMA_PEAK_TFLOPS[head["dtype"]]
+        flops = row["TFLOPs"] * 1e12 * row["us"] * 1e-6
+        intensity = flops / (row["alg_MB"] * 1e6)
+        balance = peak_tf * 1e12 / (HBM_PEAK_GBS * 1e9)
+        roofline = {"kernel": dom, "traffic": measured_traffic(w.name, ns.form).get(dom), "us_per_launch": row["us"],
+                    "alg_flops_per_launch": flops, "alg_bytes_per_launch": row["alg_MB"] * 1e6,
+                    "flops_per_byte": intensity, "machine_flops_per_byte": balance,
+                    "hbm_frac": row["hbm_frac"], "mfma_frac": row["mfma_frac"]}
+        if intensity < balance:
+            roofline.update({"bound": "hbm", "achieved": row["GBps"], "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": row["hbm_frac"]})
+        else:
+            roofline.update({"bound": "mfma", "achieved": row["TFLOPs"], "peak": peak_tf, "unit": "TFLOP/s", "frac": row["mfma_frac"]})
     else:
         roofline = {"kernel": dom, "bound": "hbm", "achieved": row["GBps"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
                     "frac": row["GBps"] / HBM_PEAK_GBS,
