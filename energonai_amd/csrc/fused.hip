@@ -34,6 +34,14 @@
 
 namespace en {
 
+// The lane's number in its wave, counted afresh (two VALU instructions) where a value derived from it is needed only
+// now and then, instead of keeping that value in a register through the key loop: the kernel has none to spare.
+__device__ __forceinline__ int lane_now() {
+  int l;
+  asm volatile("v_mbcnt_lo_u32_b32 %0, -1, 0\n\tv_mbcnt_hi_u32_b32 %0, -1, %0" : "=v"(l));
+  return l;
+}
+
 struct FusedArgs {
   AttnArgs base;             // a_ptr = q, b_ptr = k, out = ctx; q_s* = q strides, k_s* = k strides
   const void *v;
@@ -42,6 +50,7 @@ struct FusedArgs {
   const int32_t *q_row0;     // packed layout: first row of batch b in q / ctx (else null)
   const int32_t *k_row0;     // packed layout: first row of batch b in k / v (else null)
   float scale;
+  int c_vec16;               // ctx rows may be written with 128-bit stores (16-byte aligned base and strides)
 };
 
 // Both halves of the wave get (x of lanes 0..31, x of lanes 32..63): one VALU swap, no LDS round trip.
@@ -87,8 +96,6 @@ __global__ __launch_bounds__(kBlock, 3) void attn_fused_kernel(FusedArgs fa) {
   const int r = lane & 31, g = lane >> 5;
   const int q = q0 + wave * 32 + r;              // this lane's query row
   const bool q_valid = q < ql;
-  // keys this query may see: k < vis
-  const int vis = q_valid ? (a.causal ? min(kl, q + (kl - ql) + 1) : kl) : 0;
   // smallest and largest extent among the wave's 32 queries (wave-uniform): tiles below the
   // smallest need no masking, tiles from the largest on hold nothing for this wave
   const int q_first = q0 + wave * 32;
@@ -221,7 +228,10 @@ __global__ __launch_bounds__(kBlock, 3) void attn_fused_kernel(FusedArgs fa) {
 #pragma unroll
           for (int x = 0; x < 16; ++x) m_tile = fmaxf(m_tile, s[kb][x]);
       } else {
-        const int lim = vis - k0 - 4 * g;      // register (kb, x) is visible iff 32kb + 8(x/4) + x%4 < lim
+        // this lane's query and the keys it may see (k < vis_l), counted afresh: only the tiles on the diagonal come here
+        const int l = lane_now(), ql_ = q0 + wave * 32 + (l & 31);
+        const int vis_l = (ql_ < ql) ? (a.causal ? min(kl, ql_ + (kl - ql) + 1) : kl) : 0;
+        const int lim = vis_l - k0 - 4 * (l >> 5);   // register (kb, x) is visible iff 32kb + 8(x/4) + x%4 < lim
 #pragma unroll
         for (int kb = 0; kb < KB; ++kb)
 #pragma unroll
@@ -236,7 +246,7 @@ __global__ __launch_bounds__(kBlock, 3) void attn_fused_kernel(FusedArgs fa) {
         halves_of(m_tile, lo, hi);
         m_tile = fmaxf(lo, hi);
       }
-      if (__builtin_amdgcn_ballot_w64(m_tile > m_run + lazy_gap) != 0) {   // -inf + gap stays -inf: the first tile moves it
+      if (__builtin_amdgcn_ballot_w64(m_tile - lazy_gap > m_run) != 0) {   // -inf + gap stays -inf: the first tile moves it
         const float m_new = fmaxf(m_run, m_tile);
         const float alpha = (m_run == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f((m_run - m_new) * c_exp);
         l_run *= alpha;
@@ -307,14 +317,43 @@ __global__ __launch_bounds__(kBlock, 3) void attn_fused_kernel(FusedArgs fa) {
   }
 
   // ---- normalise and store: register 4j+i of tile mt holds channel 32mt + 8j + 4g + i of this lane's query
-  if (!q_valid) return;
   const float inv = l_run > 0.f ? 1.0f / l_run : 0.f;
-  T *crow = cbase + (int64_t)q * fa.c_ss;
+  const int lane_e = lane_now(), r_e = lane_e & 31, g_e = lane_e >> 5;
+  if (fa.c_vec16) {
+    // A lane holds 8-byte pieces of its own row, 32 rows per store instruction; through LDS (the K buffers are free
+    // behind the loop's last barrier, each wave takes the 32 rows' worth that is its own, so no barrier is needed)
+    // the wave's tile leaves as whole rows: 16 bytes per lane, 64 / KVEC_ROW rows per instruction.  Chunk c of row r
+    // sits in slot c ^ (r % KVEC_ROW): writes and reads both spread over all banks.
+    char *stage = reinterpret_cast<char *>(&lds_k[0][0]) + wave * 32 * ROW * E::kSize;
+#pragma unroll
+    for (int mt = 0; mt < DMT; ++mt)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        Pack<T, 4> pk;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) pk.v[i] = E::from_float(o[mt][4 * j + i] * inv);
+        const int c = 4 * mt + j;
+        *reinterpret_cast<Pack<T, 4> *>(stage + r_e * ROW * E::kSize + ((c ^ (r_e & (KVEC_ROW - 1))) * 16) + g_e * 8) = pk;
+      }
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // the wave's own writes, before its lanes read each other's
+    constexpr int RPI = kWave / KVEC_ROW;              // rows per store instruction
+#pragma unroll
+    for (int i = 0; i < 32 / RPI; ++i) {
+      const int row = i * RPI + lane_e / KVEC_ROW, c = lane_e % KVEC_ROW;
+      const uint4 v = *reinterpret_cast<const uint4 *>(stage + row * ROW * E::kSize + ((c ^ (row & (KVEC_ROW - 1))) * 16));
+      const int qrow = q0 + wave * 32 + row;
+      if (qrow < ql && c * EPV < a.D) *reinterpret_cast<uint4 *>(cbase + (int64_t)qrow * fa.c_ss + c * EPV) = v;
+    }
+    return;
+  }
+  const int q_e = q0 + wave * 32 + r_e;
+  if (q_e >= ql) return;
+  T *crow = cbase + (int64_t)q_e * fa.c_ss;
 #pragma unroll
   for (int mt = 0; mt < DMT; ++mt)
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
-      const int d = mt * 32 + 8 * j + 4 * g;
+      const int d = mt * 32 + 8 * j + 4 * g_e;
       if (d < a.D) {
         Pack<T, 4> pk;
 #pragma unroll
@@ -371,6 +410,7 @@ extern "C" int en_attn_fused(const void *q, const void *k, const void *v, void *
   fa.v_sb = v_strides[0]; fa.v_sh = v_strides[1]; fa.v_ss = v_strides[2];
   fa.c_sb = c_strides[0]; fa.c_sh = c_strides[1]; fa.c_ss = c_strides[2];
   fa.q_row0 = q_row_offsets; fa.k_row0 = k_row_offsets;
+  fa.c_vec16 = aligned_to(ctx, 16) && (c_strides[0] % 8) == 0 && (c_strides[1] % 8) == 0 && (c_strides[2] % 8) == 0;
   if (tile_table && q_lens) return EN_ERR_UNSUPPORTED;      // the table lists the query tiles of min(k_lens, q_seq_len) rows
   a.tile_table = tile_table;
   fa.scale = scale;
