@@ -94,8 +94,6 @@ __global__ __launch_bounds__(kBlock, 3) void attn_fused_kernel(FusedArgs fa) {
   const int tid = threadIdx.x;
   const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int r = lane & 31, g = lane >> 5;
-  const int q = q0 + wave * 32 + r;              // this lane's query row
-  const bool q_valid = q < ql;
   // smallest and largest extent among the wave's 32 queries (wave-uniform): tiles below the
   // smallest need no masking, tiles from the largest on hold nothing for this wave
   const int q_first = q0 + wave * 32;
@@ -109,15 +107,24 @@ __global__ __launch_bounds__(kBlock, 3) void attn_fused_kernel(FusedArgs fa) {
   const T *vbase = reinterpret_cast<const T *>(fa.v) + (int64_t)b * fa.v_sb + kr * fa.v_ss + (int64_t)h * fa.v_sh;
   T *cbase = reinterpret_cast<T *>(a.out) + (int64_t)b * fa.c_sb + qr * fa.c_ss + (int64_t)h * fa.c_sh;
 
-  // Q fragments (B operand of S^T = K Q^T): this lane's query row, 8 channels per step
+  // Q fragments (B operand of S^T = K Q^T): this lane's query row, 8 channels per step.  The wave's 32 rows come in
+  // as whole rows, memory straight into LDS (the second K buffer and the V buffer are idle until the key loop starts;
+  // waves 0 and 1 take the one, waves 2 and 3 the other, 32 rows each), chunks in the K tile's swizzled slots, and
+  // each lane then reads its own row's chunks: sixteen-byte pieces fetched by every lane from a row of its own
+  // kept the address unit busy with 32 rows per instruction.
   uint4 qf[NVS];
+  T *q_stage = (wave < 2 ? lds_k[1] : lds_v) + (wave & 1) * 32 * ROW;
   {
-    const rsrc_t q_rsrc = make_rsrc(qbase, (uint32_t)(((int64_t)(ql - 1) * a.q_ss + a.D) * E::kSize));
+    const desc_t q_desc = make_desc(qbase, (uint32_t)(((int64_t)(ql - 1) * a.q_ss + a.D) * E::kSize));
+    constexpr int RPLQ = kWave / KVEC_ROW;         // rows one direct load of a wave covers
+    const int row = lane / KVEC_ROW, slot = lane % KVEC_ROW;
 #pragma unroll
-    for (int vs = 0; vs < NVS; ++vs) {
-      const int d = M::k_of(vs, g, NVS);
-      const uint32_t off = (uint32_t)(((int64_t)q * a.q_ss + d) * E::kSize);
-      qf[vs] = buffer_load16(q_rsrc, (q_valid && d < a.D) ? off : kOutOfRange);
+    for (int n = 0; n < 32 / RPLQ; ++n) {
+      const int rr = n * RPLQ + row;               // row of the wave's 32
+      const int c = slot ^ (DP == 128 ? (rr & 15) : ((rr >> 1) & 7));
+      const int qq = q0 + wave * 32 + rr;
+      const uint32_t off = (uint32_t)(((int64_t)qq * a.q_ss + c * EPV) * E::kSize);
+      buffer_load16_to_lds(q_desc, lds_address(q_stage) + n * kWave * 16, (qq < ql && c * EPV < a.D) ? off : kOutOfRange);
     }
   }
 
@@ -185,6 +192,12 @@ __global__ __launch_bounds__(kBlock, 3) void attn_fused_kernel(FusedArgs fa) {
   // for between the softmax and the second contraction.  Two barriers per tile.
   fetch_k(lds_k[0]);
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  {  // the wave's own rows have landed; the barrier below also keeps the tiles of the key loop off them until all have read
+    const int qsw = DP == 128 ? (r & 15) : ((r >> 1) & 7);
+#pragma unroll
+    for (int vs = 0; vs < NVS; ++vs)
+      qf[vs] = *reinterpret_cast<const uint4 *>(&q_stage[r * ROW + (((2 * vs + g) ^ qsw) * EPV)]);
+  }
   lds_barrier();
 
   for (int kt = 0; kt < nkt; ++kt) {
