@@ -236,9 +236,25 @@ __global__ __launch_bounds__(kBlock, 3) void attn_qk_strip_kernel(AttnArgs a) {
   const T *kbase = reinterpret_cast<const T *>(a.b_ptr) + k_unit_offset(a, b, h);
   T *sbase = reinterpret_cast<T *>(a.out) + score_unit_offset<EPV>(a, unit);
 
-  // Q fragments (B operand): this lane's query row, 8 channels per step; rows >= ql read as zero
+  // Q fragments (B operand): this lane's query row, 8 channels per step; rows >= ql read as zero.  With direct loads
+  // the wave's 32 rows come in as whole rows, memory straight into LDS (the second K buffer for waves 0 and 1, the
+  // score strips, idle until the first tile's scores exist, for waves 2 and 3; 8 KB each), chunks in the K tile's
+  // swizzled slots, and each lane then reads its own row's chunks from there: sixteen-byte pieces fetched by every
+  // lane from a row of its own kept the address unit busy with 32 rows per instruction.
   uint4 qf[NVS];
-  {
+  static_assert(!DMA || sizeof(lds_c) >= 2 * 32 * DP * sizeof(T), "two waves stage their Q rows in the score strips");
+  T *q_stage = (wave < 2 ? lds_k[1] : &lds_c[0][0]) + (wave & 1) * 32 * DP;
+  if constexpr (DMA) {
+    const desc_t q_desc = make_desc(qbase, (uint32_t)(((int64_t)(ql - 1) * a.q_ss + a.D) * E::kSize));
+    constexpr int RPLQ = kWave / KVEC_ROW;         // rows one direct load of a wave covers
+#pragma unroll
+    for (int n = 0; n < 32 / RPLQ; ++n) {
+      const int rr = n * RPLQ + lane / KVEC_ROW;   // row of the wave's 32
+      const int c = (lane % KVEC_ROW) ^ (rr & (KVEC_ROW - 1));
+      const uint32_t off = (uint32_t)(((int64_t)(qw + rr) * a.q_ss + c * EPV) * E::kSize);
+      buffer_load16_to_lds(q_desc, lds_address(q_stage) + n * kWave * 16, (qw + rr < ql && c * EPV < a.D) ? off : kOutOfRange);
+    }
+  } else {
     const rsrc_t q_rsrc = make_rsrc(qbase, (uint32_t)(((int64_t)(ql - 1) * a.q_ss + a.D) * E::kSize));
 #pragma unroll
     for (int vs = 0; vs < NVS; ++vs) {
@@ -293,6 +309,11 @@ __global__ __launch_bounds__(kBlock, 3) void attn_qk_strip_kernel(AttnArgs a) {
   if constexpr (DMA) {
     dma_k(lds_k[0]);
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    // the wave's own Q rows have landed; the barrier below keeps the tiles and strips of the loop off them until
+    // every wave has read its own
+#pragma unroll
+    for (int vs = 0; vs < NVS; ++vs)
+      qf[vs] = *reinterpret_cast<const uint4 *>(&q_stage[r * DP + (((2 * vs + g) ^ (r & (KVEC_ROW - 1))) * EPV)]);
   } else {
     fetch_k();
     stage_k(lds_k[0]);
@@ -712,6 +733,33 @@ __global__ __launch_bounds__(kBlock, 3) void attn_pv_strip_kernel(AttnArgs a) {
   }
 
   // register 4j+i of tile mt holds channel 32mt + 8j + 4g + i of this lane's query
+  if (a.ctx_vec16) {
+    // A lane holds 8-byte pieces of its own row, 32 rows per store instruction; through LDS (the V buffers are free
+    // behind the loop's last barrier, each wave takes the 32 rows' worth that is its own, so no barrier is needed)
+    // the wave's tile leaves as whole rows: 16 bytes per lane, 64 / VVEC_ROW rows per instruction.  Chunk c of row r
+    // sits in slot c ^ (r % VVEC_ROW): writes and reads both spread over all banks.
+    char *stage = reinterpret_cast<char *>(&lds_v[0][0]) + wave * 32 * VROW_BYTES;
+    const bool valid = q < ql;
+#pragma unroll
+    for (int mt = 0; mt < DMT; ++mt)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        Pack<T, 4> pk;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) pk.v[i] = E::from_float(valid ? o[mt][4 * j + i] : 0.f);
+        const int c = 4 * mt + j;
+        *reinterpret_cast<Pack<T, 4> *>(stage + r * VROW_BYTES + ((c ^ (r & (VVEC_ROW - 1))) * 16) + g * 8) = pk;
+      }
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // the wave's own writes, before its lanes read each other's
+#pragma unroll
+    for (int i = 0; i < 32 / RPL; ++i) {
+      const int row = i * RPL + lane / VVEC_ROW, c = lane % VVEC_ROW;
+      const uint4 v = *reinterpret_cast<const uint4 *>(stage + row * VROW_BYTES + ((c ^ (row & (VVEC_ROW - 1))) * 16));
+      const int qrow = q0 + wave * 32 + row;
+      if (qrow < (a.zero_padding ? a.Sq : ql) && c * EPV < a.D) *reinterpret_cast<uint4 *>(cbase + (int64_t)qrow * a.q_ss + c * EPV) = v;
+    }
+    return;
+  }
   if (q >= a.Sq) return;
   const bool valid = q < ql;
   if (!valid && !a.zero_padding) return;
@@ -971,6 +1019,7 @@ int en_attn_pv(const void *p, const void *v, void *ctx, const int32_t *k_lens, c
   a.q_row0 = c_row_offsets; a.k_row0 = v_row_offsets; a.packed_scores = packed_scores ? 1 : 0;
   a.tile_table = zero_padding ? nullptr : tile_table;      // the tiles a table leaves out are the ones to fill with zeros
   a.vec_out = ((packed_scores || (k_seq_len % epv) == 0) && aligned_to(p, 16)) ? 1 : 0;
+  a.ctx_vec16 = (aligned_to(ctx, 16) && strides_vec_ok(c_stride_b, c_stride_h, c_stride_s, epv)) ? 1 : 0;
   a.ntq = (int)ceil_div(q_seq_len, kQTile);
   a.units = batch * head_num;
   hipStream_t s = (hipStream_t)stream;

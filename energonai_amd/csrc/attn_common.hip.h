@@ -64,6 +64,7 @@ struct AttnArgs {
   int causal;
   int zero_padding;
   int vec_out;   // output rows may be written with 128-bit stores
+  int ctx_vec16; // PV: ctx rows may be written with 128-bit stores (16-byte aligned base and strides)
   int ntq;       // query tiles per unit
   int units;     // B * H
   // Packed operands: batch b's rows start at row q_row0[b] (q in QK, ctx in PV) / k_row0[b] (k in QK, v in PV)
