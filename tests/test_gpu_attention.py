@@ -228,6 +228,38 @@ def test_attn_fused(dtype, causal, B, H, S, D, lens):
     assert bool((ctx[rows_pad] == sentinel).all())
 
 
+@pytest.mark.parametrize("D", [64, 128, 40])
+def test_attn_fused_and_pv_write_an_output_that_is_not_16_byte_aligned(D):
+    """The whole-row output path needs 16-byte aligned rows; an output that is only 8-byte aligned (a view four
+    elements into a wider tensor) takes the piecewise stores.  Both give the bits of the aligned call, and neither
+    touches the columns beside the view or the rows of the padding."""
+    k = _kernel()
+    B, H, S = 3, 2, 200
+    lens = [200, 77, 1]
+    announce("unaligned ctx", D, lens)
+    g = torch.Generator().manual_seed(31 + D)
+    q, kk, v = (torch.randn(B, H, S, D, generator=g).half().cuda() for _ in range(3))
+    lens_t = torch.tensor(lens, dtype=torch.int32).cuda()
+    aligned = k.attn_fused(q, kk, v, lens_t, causal=True)
+    wide = torch.full((B, H, S, D + 8), 5.0, dtype=torch.float16, device="cuda")
+    view = wide[..., 4:4 + D]
+    assert view.data_ptr() % 16 == 8
+    k.attn_fused(q, kk, v, lens_t, causal=True, out=view)
+    for b, n in enumerate(lens):
+        assert torch.equal(view[b, :, :n], aligned[b, :, :n])
+        assert bool((view[b, :, n:] == 5.0).all())
+    assert bool((wide[..., :4] == 5.0).all()) and bool((wide[..., 4 + D:] == 5.0).all())
+    # the same for PV on the probabilities of these scores
+    scores = k.attn_qk(q, kk, lens_t, alpha=D ** -0.5, causal=True)
+    probs = k.scale_mask_softmax(B, S, H, scores, lens_t)
+    ctx_aligned = k.attn_pv(probs, v, lens_t, causal=True)
+    wide.fill_(5.0)
+    k.attn_pv(probs, v, lens_t, causal=True, out=view)
+    for b, n in enumerate(lens):
+        assert torch.equal(view[b, :, :n], ctx_aligned[b, :, :n])
+    assert bool((wide[..., :4] == 5.0).all()) and bool((wide[..., 4 + D:] == 5.0).all())
+
+
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 @pytest.mark.parametrize("causal", [True, False])
 @pytest.mark.parametrize("B,H,S,D,lens", ATTN_CASES)
