@@ -4,6 +4,7 @@
     python3 bench_profiles.py trace   --workload c3      # rocprofv3 --kernel-trace --stats of `bench.py --step-only`
     python3 bench_profiles.py traffic --workload c3      # two --pmc runs (FETCH_SIZE, then WRITE_SIZE) + copy calibration
     python3 bench_profiles.py counters --workload c3     # one --pmc run of SQ counters: MFMA and VALU busy, LDS, waits
+    python3 bench_profiles.py issue --workload c3        # one --pmc run: matrix / vector co-execution, address unit queues
 
 Each sub-command starts rocprofv3 as a child process with `python3 bench.py ...` after `--`, reads the CSV files it
 leaves in a scratch directory (--raw-dir, default: a fresh temporary one), and prints a markdown summary (redirect it
@@ -229,10 +230,54 @@ def cmd_counters(ns) -> int:
     return 0
 
 
+ISSUE_COUNTERS = ["SQ_VALU_MFMA_BUSY_CYCLES", "SQ_VALU_MFMA_COEXEC_CYCLES", "SQ_VMEM_TA_CMD_FIFO_FULL",
+                  "SQ_VMEM_TA_ADDR_FIFO_FULL", "SQ_INSTS_VALU", "SQ_INSTS_MFMA", "SQ_INSTS_LDS", "GRBM_GUI_ACTIVE"]
+
+
+def cmd_issue(ns) -> int:
+    """What the SIMDs issue and what holds the memory instructions back: matrix pipe busy, matrix and vector pipe
+    busy at once, cycles with the address unit's queues full, instruction counts per launch."""
+    scope = ["--no-extra"] if ns.all_ops else ["--form", ns.form, "--step-only"]
+    bench_args = ["--workload", ns.workload] + scope + ["--no-cpu", "--steps", str(ns.steps), "--warmup", str(ns.warmup)]
+    decode = ns.workload == "c5"
+    d, line, shown = run_profiler(f"issue_{ns.workload}", ["--pmc"] + ISSUE_COUNTERS, bench_args, ns.timeout)
+    path = find_csv(d, "counter_collection.csv")
+    per = {c: counter_rows(path, c) for c in ISSUE_COUNTERS}
+    keys = collections.defaultdict(lambda: collections.defaultdict(float))
+    names = collections.defaultdict(set)
+    for c, rows in per.items():
+        for name, vals in rows.items():
+            key = key_of(name, decode)
+            if key is None or key == "copy":
+                continue
+            keys[key][c] += sum(vals)
+            keys[key]["n_" + c] = max(keys[key]["n_" + c], len(vals))
+            names[key].add(name[:70])
+    print(f"# Issue counters of the kernels of `bench.py --workload {ns.workload} {' '.join(scope)}`\n")
+    print("Command (MI355X box, repo root; the summary below is this command's stdout):\n")
+    print(f"```\npython3 bench_profiles.py issue --workload {ns.workload}"
+          f"{' --all-ops' if ns.all_ops else ' --form ' + ns.form}\n  -> {shown}\n```\n")
+    print("Shares are of all SIMD cycles of an op's launches (`GRBM_GUI_ACTIVE` / 8 XCDs x 1024 SIMDs); the queue "
+          "counters are per SIMD as well.  Instruction counts are per launch, summed over all waves.\n")
+    print("| op (key in the bench line) | kernels | matrix pipe busy | matrix and vector pipe busy at once | "
+          "address unit's command queue full | address unit's address queue full | VALU instructions (incl. MFMA), M | "
+          "MFMA instructions, M | LDS instructions, M |\n|---|---|---|---|---|---|---|---|---|")
+    for key, v in keys.items():
+        simd = v["GRBM_GUI_ACTIVE"] / 8 * 1024
+        if simd <= 0:
+            continue
+        n = max(v["n_SQ_INSTS_VALU"], 1)
+        print(f"| `{key}` | {'; '.join(sorted(names[key]))} | {v['SQ_VALU_MFMA_BUSY_CYCLES'] / simd:.3f} | "
+              f"{v['SQ_VALU_MFMA_COEXEC_CYCLES'] / simd:.3f} | {v['SQ_VMEM_TA_CMD_FIFO_FULL'] / simd:.3f} | "
+              f"{v['SQ_VMEM_TA_ADDR_FIFO_FULL'] / simd:.3f} | {v['SQ_INSTS_VALU'] / n / 1e6:.2f} | "
+              f"{v['SQ_INSTS_MFMA'] / n / 1e6:.2f} | {v['SQ_INSTS_LDS'] / n / 1e6:.2f} |")
+    return 0
+
+
 def main(argv=None) -> int:
     ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
     sub = ap.add_subparsers(dest="cmd", required=True)
-    for name, fn in (("trace", cmd_trace), ("traffic", cmd_traffic), ("counters", cmd_counters)):
+    for name, fn in (("trace", cmd_trace), ("traffic", cmd_traffic), ("counters", cmd_counters), ("issue", cmd_issue)):
         p = sub.add_parser(name)
         p.add_argument("--workload", default="c3", choices=["c1", "c2", "c3", "c4", "c5"])
         p.add_argument("--form", default="default", choices=["default", "three_kernel"],
@@ -241,7 +286,7 @@ def main(argv=None) -> int:
         p.add_argument("--warmup", type=int, default=5)
         p.add_argument("--timeout", type=int, default=300, help="seconds allowed for each rocprofv3 run")
         p.add_argument("--raw-dir", default=None, help="directory for rocprofv3's raw output (default: a temporary one)")
-        if name == "counters":
+        if name in ("counters", "issue"):
             p.add_argument("--all-ops", action="store_true", help="every op of the bench line, not the step alone")
         p.set_defaults(fn=fn)
     ns = ap.parse_args(argv)
