@@ -30,6 +30,14 @@
 // ahead; V has one buffer, is sent for at the top of its own tile and arrives
 // behind the score and softmax work: 48 KB of LDS per workgroup, so that three
 // workgroups fit a CU.  The barriers order LDS only, as in the unfused kernels.
+//
+// Everything that crosses the memory interface does so as whole rows: the K and
+// V tiles, the workgroup's Q rows (loaded straight into the buffers that are
+// idle before the key loop, each lane then reads its fragments from LDS) and the
+// output tile (written to the K buffers behind the loop's last barrier, stored
+// 16 bytes per lane).  A lane that fetches or stores pieces of a row of its own
+// makes every instruction touch 32 rows, and the queue of the address unit then
+// stands full and holds back the tile loads of every wave on the CU.
 #include "attn_common.hip.h"
 
 namespace en {
