@@ -5,6 +5,7 @@
     python3 bench_profiles.py traffic --workload c3      # two --pmc runs (FETCH_SIZE, then WRITE_SIZE) + copy calibration
     python3 bench_profiles.py counters --workload c3     # one --pmc run of SQ counters: MFMA and VALU busy, LDS, waits
     python3 bench_profiles.py issue --workload c3        # one --pmc run: matrix / vector co-execution, address unit queues
+    python3 bench_profiles.py memsys --workload c3       # three --pmc runs: L2 hit rate, requests to memory, stalled channels
 
 Each sub-command starts rocprofv3 as a child process with `python3 bench.py ...` after `--`, reads the CSV files it
 leaves in a scratch directory (--raw-dir, default: a fresh temporary one), and prints a markdown summary (redirect it
@@ -274,10 +275,68 @@ def cmd_issue(ns) -> int:
     return 0
 
 
+# three runs of at most four L2 (TCC) counters each, plus the cycle count that turns stalls into shares
+MEMSYS_RUNS = [
+    ["TCC_REQ_sum", "TCC_HIT_sum", "TCC_MISS_sum", "GRBM_GUI_ACTIVE"],
+    ["TCC_EA0_RDREQ_sum", "TCC_EA0_WRREQ_sum", "TCC_EA0_WRREQ_64B_sum", "TCC_EA0_RDREQ_32B_sum", "GRBM_GUI_ACTIVE"],
+    ["TCC_EA0_WRREQ_STALL_sum", "TCC_TOO_MANY_EA_WRREQS_STALL_sum", "TCC_TAG_STALL_sum",
+     "TCC_EA0_RDREQ_DRAM_CREDIT_STALL_sum", "GRBM_GUI_ACTIVE"],
+]
+
+
+def cmd_memsys(ns) -> int:
+    """What the L2 and its memory interface see: hit rate, requests that go on to memory by size, and the cycles a
+    channel could not send (summed over the 16 channels of each of the 8 XCDs, so a share of 1.0 would be every
+    channel blocked all the time)."""
+    scope = ["--no-extra"] if ns.all_ops else ["--form", ns.form, "--step-only"]
+    bench_args = ["--workload", ns.workload] + scope + ["--no-cpu", "--steps", str(ns.steps), "--warmup", str(ns.warmup)]
+    decode = ns.workload == "c5"
+    keys = collections.defaultdict(lambda: collections.defaultdict(float))
+    shown_all = []
+    for i, counters in enumerate(MEMSYS_RUNS):
+        d, line, shown = run_profiler(f"memsys{i}_{ns.workload}", ["--pmc"] + counters, bench_args, ns.timeout)
+        shown_all.append(shown)
+        path = find_csv(d, "counter_collection.csv")
+        for c in counters:
+            for name, vals in counter_rows(path, c).items():
+                key = key_of(name, decode)
+                if key is None or key == "copy":
+                    continue
+                tag = c if c != "GRBM_GUI_ACTIVE" else f"cycles{i}"
+                keys[key][tag] += sum(vals)
+                keys[key]["n_" + tag] = max(keys[key]["n_" + tag], len(vals))
+    print(f"# L2 and memory-interface counters of the kernels of `bench.py --workload {ns.workload} {' '.join(scope)}`\n")
+    print("Command (MI355X box, repo root; the summary below is this command's stdout):\n")
+    print(f"```\npython3 bench_profiles.py memsys --workload {ns.workload}"
+          f"{' --all-ops' if ns.all_ops else ' --form ' + ns.form}")
+    for sh in shown_all:
+        print(f"  -> {sh}")
+    print("```\n")
+    print("Requests are per launch, in millions.  Requests to memory: reads of 32 / 64 bytes (the rest are 128-byte "
+          "reads), writes of 64 bytes (the rest 32).  Stall shares: cycles summed over the L2 channels divided by "
+          "128 channels x the launch's cycles (`GRBM_GUI_ACTIVE` counts the cycles of all 8 XCDs).\n")
+    print("| op (key in the bench line) | L2 requests, M | L2 hit rate | reads to memory, M (32-byte ones) | "
+          "writes to memory, M (64-byte ones) | write requests held back | too many writes outstanding | tag stall | "
+          "read credits to DRAM exhausted |\n|---|---|---|---|---|---|---|---|---|")
+    for key, v in keys.items():
+        n0, n1 = max(v["n_TCC_REQ_sum"], 1), max(v["n_TCC_EA0_RDREQ_sum"], 1)
+        chan_cycles = v["cycles2"] / 8 * 128
+        if chan_cycles <= 0:
+            continue
+        hit = v["TCC_HIT_sum"] / max(v["TCC_HIT_sum"] + v["TCC_MISS_sum"], 1.0)
+        print(f"| `{key}` | {v['TCC_REQ_sum'] / n0 / 1e6:.2f} | {hit:.3f} | {v['TCC_EA0_RDREQ_sum'] / n1 / 1e6:.2f} "
+              f"({v['TCC_EA0_RDREQ_32B_sum'] / n1 / 1e6:.2f}) | {v['TCC_EA0_WRREQ_sum'] / n1 / 1e6:.2f} "
+              f"({v['TCC_EA0_WRREQ_64B_sum'] / n1 / 1e6:.2f}) | {v['TCC_EA0_WRREQ_STALL_sum'] / chan_cycles:.3f} | "
+              f"{v['TCC_TOO_MANY_EA_WRREQS_STALL_sum'] / chan_cycles:.3f} | {v['TCC_TAG_STALL_sum'] / chan_cycles:.3f} | "
+              f"{v['TCC_EA0_RDREQ_DRAM_CREDIT_STALL_sum'] / chan_cycles:.3f} |")
+    return 0
+
+
 def main(argv=None) -> int:
     ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
     sub = ap.add_subparsers(dest="cmd", required=True)
-    for name, fn in (("trace", cmd_trace), ("traffic", cmd_traffic), ("counters", cmd_counters), ("issue", cmd_issue)):
+    for name, fn in (("trace", cmd_trace), ("traffic", cmd_traffic), ("counters", cmd_counters), ("issue", cmd_issue),
+                     ("memsys", cmd_memsys)):
         p = sub.add_parser(name)
         p.add_argument("--workload", default="c3", choices=["c1", "c2", "c3", "c4", "c5"])
         p.add_argument("--form", default="default", choices=["default", "three_kernel"],
@@ -286,7 +345,7 @@ def main(argv=None) -> int:
         p.add_argument("--warmup", type=int, default=5)
         p.add_argument("--timeout", type=int, default=300, help="seconds allowed for each rocprofv3 run")
         p.add_argument("--raw-dir", default=None, help="directory for rocprofv3's raw output (default: a temporary one)")
-        if name in ("counters", "issue"):
+        if name in ("counters", "issue", "memsys"):
             p.add_argument("--all-ops", action="store_true", help="every op of the bench line, not the step alone")
         p.set_defaults(fn=fn)
     ns = ap.parse_args(argv)
