@@ -5,10 +5,13 @@
 
 A step is one pass of
     depad -> transpose_pad -> QK^T -> scale_mask_softmax -> PV -> transpose_depad -> residual + LayerNorm
-over one synthetic batch whose inputs are already resident in HBM.  The timed form issues it as four launches:
-QK^T and PV address the packed projections and the packed context through per-sequence row offsets (so neither
-transpose is a launch of its own), the LayerNorm takes its residual rows straight from the padded activations (so
-depad is not one either); the seven-launch form and the unchanged caller's seven Python calls are timed beside it.  The headline
+over one synthetic batch whose inputs are already resident in HBM.  The timed form is the one
+layer.padding_removal_layer runs when the caller names none (`step_form` in the line): for 16-bit storage two
+launches -- fused attention that addresses the packed projections and the packed context through per-sequence row
+offsets (so neither transpose is a launch of its own and no score tensor exists), then the LayerNorm, which takes
+its residual rows straight from the padded activations (so depad is not a launch either); for fp32 QK^T, softmax
+and PV as three kernels on the same packed operands plus that LayerNorm.  The three-kernel form, the reference's
+seven ops through one call and the unchanged caller's seven Python calls are timed beside it.  The headline
 value is tokens/s of that pass on the workload named by --workload (default c3,
 the OPT-30B-shaped layer: the largest of the five that fits one GPU -- 1.9 GB of
 scores, 45 GFLOP per contraction -- and the one whose kernels are bound by HBM
@@ -40,18 +43,28 @@ MFMA_PEAK_TFLOPS = {"f16": 2500.0, "bf16": 2500.0, "f32": 157.3}
 PROFILES = os.path.join(ROOT, "profiles")
 
 
+def library_source_hash() -> str:
+    """Digest of the sources libenergon_hip.so was compiled from (en_source_hash)."""
+    from energonai_amd import _lib
+    return _lib.load().en_source_hash().decode()
+
+
 def measured_traffic(workload: str, form: str = "default"):
     """HBM bytes per launch of each kernel of the step, from the counter summary kept under profiles/
     (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this file, scaled by what the same counters read for
     en_copy_bytes of known size; written by bench_profiles.py).  Counters cannot be read from inside the
-    benchmark, so the figures of the last profiled tree are reported beside the live timing; {} when the
+    benchmark, so the figures of the last profiled tree are reported beside the live timing.  Returns
+    (bytes by op, digest of the library sources the summary was measured on or None); ({}, None) when the
     summary is not there."""
     tag = "" if form == "default" else f"_{form}"
     path = os.path.join(PROFILES, f"bench_{workload}{tag}_hbm_traffic.md")
-    out = {}
+    out, digest = {}, None
     try:
         with open(path) as f:
             for line in f:
+                if line.startswith("Library sources"):
+                    parts = line.split("`")
+                    digest = parts[-2] if len(parts) >= 3 else None
                 cells = [c.strip() for c in line.strip().strip("|").split("|")]
                 if len(cells) >= 3 and cells[0].startswith("`") and cells[0].endswith("`"):
                     try:
@@ -60,7 +73,7 @@ def measured_traffic(workload: str, form: str = "default"):
                         pass
     except OSError:
         pass
-    return out
+    return out, digest
 
 
 DTYPE_NAME = {"torch.float16": "f16", "torch.bfloat16": "bf16", "torch.float32": "f32"}
@@ -688,6 +701,42 @@ def copy_yardstick(torch, iters):
     return out
 
 
+def roofline_of(res, workload_name, form="default"):
+    """Roofline object of the kernel that takes the largest share of a workload's step, in the form the step
+    launches it: algorithmic bytes (or FLOPs) per launch over the launch-to-launch time measured above.
+    Fused attention reads q, k, v and writes ctx (4 T H D e bytes) and does 4 D FLOPs per visible score: which roof
+    bounds it follows from its FLOPs per byte against the machine's (peak FLOP/s over peak bytes/s); c3 (short
+    sequences, 170 FLOP/B against 312) sits under the HBM roof, c4 (355 FLOP/B) under the matrix roof.  Both
+    fractions are in the object whichever one `frac` is.  `traffic` comes from the counter summary under profiles/
+    (None when there is none for this workload, or when it was measured on other sources than this library's)."""
+    kt = res["step_kernels"]
+    dom = max(kt, key=lambda n: kt[n]["us"])
+    row = kt[dom]
+    by_op, digest = measured_traffic(workload_name, form)
+    traffic = by_op.get(dom)
+    if "mfma_frac" in row and dom.startswith("attn_fused"):
+        peak_tf = MFMA_PEAK_TFLOPS[res["dtype"]]
+        flops = row["TFLOPs"] * 1e12 * row["us"] * 1e-6
+        intensity = flops / (row["alg_MB"] * 1e6)
+        balance = peak_tf * 1e12 / (HBM_PEAK_GBS * 1e9)
+        roofline = {"kernel": dom, "traffic": traffic, "us_per_launch": row["us"],
+                    "alg_flops_per_launch": flops, "alg_bytes_per_launch": row["alg_MB"] * 1e6,
+                    "flops_per_byte": intensity, "machine_flops_per_byte": balance,
+                    "hbm_frac": row["hbm_frac"], "mfma_frac": row["mfma_frac"]}
+        if intensity < balance:
+            roofline.update({"bound": "hbm", "achieved": row["GBps"], "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": row["hbm_frac"]})
+        else:
+            roofline.update({"bound": "mfma", "achieved": row["TFLOPs"], "peak": peak_tf, "unit": "TFLOP/s", "frac": row["mfma_frac"]})
+    else:
+        roofline = {"kernel": dom, "bound": "hbm", "achieved": row["GBps"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                    "frac": row["GBps"] / HBM_PEAK_GBS, "traffic": traffic, "us_per_launch": row["us"],
+                    "alg_bytes_per_launch": row["alg_MB"] * 1e6}
+    # the counter summary speaks for the sources it was measured on: say whether those are this library's
+    roofline["traffic_measured_on_sources"] = digest
+    roofline["traffic_is_of_this_library"] = None if traffic is None else (digest == library_source_hash())
+    return roofline
+
+
 def main(argv=None) -> int:
     ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
     ap.add_argument("--gpus", type=int, default=1)
@@ -731,37 +780,14 @@ def main(argv=None) -> int:
                         step_only=ns.step_only, form=ns.form)
     torch.cuda.synchronize()
 
-    # roofline of the kernel that takes the largest share of the step, in the form the step launches it
     kt = head["step_kernels"]
-    dom = max(kt, key=lambda n: kt[n]["us"])
-    row = kt[dom]
-    if "mfma_frac" in row and dom.startswith("attn_fused"):
-        # fused attention reads q, k, v and writes ctx (4 T H D e bytes) and does 4 D FLOPs per visible score: which roof
-        # bounds it follows from its FLOPs per byte against the machine's (peak FLOP/s over peak bytes/s); c3 (short
-        # sequences, 170 FLOP/B against 312) sits under the HBM roof, c4 (355 FLOP/B) under the matrix roof.  Both
-        # fractions are in the line whichever one `frac` is.
-        peak_tf = MFMA_PEAK_TFLOPS[head["dtype"]]
-        flops = row["TFLOPs"] * 1e12 * row["us"] * 1e-6
-        intensity = flops / (row["alg_MB"] * 1e6)
-        balance = peak_tf * 1e12 / (HBM_PEAK_GBS * 1e9)
-        roofline = {"kernel": dom, "traffic": measured_traffic(w.name, ns.form).get(dom), "us_per_launch": row["us"],
-                    "alg_flops_per_launch": flops, "alg_bytes_per_launch": row["alg_MB"] * 1e6,
-                    "flops_per_byte": intensity, "machine_flops_per_byte": balance,
-                    "hbm_frac": row["hbm_frac"], "mfma_frac": row["mfma_frac"]}
-        if intensity < balance:
-            roofline.update({"bound": "hbm", "achieved": row["GBps"], "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": row["hbm_frac"]})
-        else:
-            roofline.update({"bound": "mfma", "achieved": row["TFLOPs"], "peak": peak_tf, "unit": "TFLOP/s", "frac": row["mfma_frac"]})
-    else:
-        roofline = {"kernel": dom, "bound": "hbm", "achieved": row["GBps"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                    "frac": row["GBps"] / HBM_PEAK_GBS,
-                    "traffic": measured_traffic(w.name, ns.form).get(dom), "us_per_launch": row["us"],
-                    "alg_bytes_per_launch": row["alg_MB"] * 1e6}
+    roofline = roofline_of(head, w.name, ns.form)
 
     out = {
         "metric": "per_layer_tokens_per_s", "value": head["tokens_per_s"], "unit": "tokens/s", "n_gpus": 1,
         "steps": ns.steps, "warmup": ns.warmup, "ms_per_step": head["ms_per_step"], "higher_is_better": True,
         "scaling": "weak", "vs_baseline": None, "dtype": head["dtype"], "data": "synthetic",
+        "library_source_hash": library_source_hash(),
         "config": {"workload": f"{w.name}: {w.title}; batch {w.batch}, bucket {w.seq}, {w.heads}x{w.head_dim} heads, "
                                f"LayerNorm width {w.hidden}, {head['tokens']} valid tokens"},
         "roofline": roofline,
@@ -787,6 +813,7 @@ def main(argv=None) -> int:
                 continue
             try:
                 others[ow.name] = run_workload(torch, ow, max(5, ns.steps // 2), max(2, ns.warmup // 2))
+                others[ow.name]["roofline"] = roofline_of(others[ow.name], ow.name)
             except Exception as exc:
                 others[ow.name] = {"error": str(exc)[:300]}
         out["workloads"] = others

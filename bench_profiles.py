@@ -78,6 +78,16 @@ def run_profiler(tag: str, prof_args, bench_args, timeout_s: int):
     return d, line, " ".join(cmd[:1] + prof_args + ["--", "python3", "bench.py"] + bench_args)
 
 
+def print_sources(line) -> None:
+    """Names the library sources the profiled run was made on (en_source_hash, carried in the bench line):
+    bench.py compares it with the library it runs before it takes a figure from the summary for that library's."""
+    h = (line or {}).get("library_source_hash")
+    if h is None:
+        from energonai_amd import build
+        h = build.source_hash()
+    print(f"Library sources (`en_source_hash`) of the profiled run: `{h}`\n")
+
+
 def find_csv(d: str, suffix: str) -> str:
     hits = glob.glob(os.path.join(d, "**", f"*{suffix}"), recursive=True)
     if not hits:
@@ -112,6 +122,7 @@ def cmd_trace(ns) -> int:
     print(f"# rocprofv3 kernel-trace summary: `bench.py --workload {ns.workload} --form {ns.form} --step-only`\n")
     print("Command (MI355X box, repo root; the summary below is this command's stdout):\n")
     print(f"```\npython3 bench_profiles.py trace --workload {ns.workload} --form {ns.form}\n  -> {shown}\n```\n")
+    print_sources(line)
     if line:
         print(f"Bench line of the profiled run: {line['ms_per_step'] * 1e3:.1f} us per step "
               f"({line['config']['workload']}). Event timings of the same run (`us (events)`) are taken by bench.py "
@@ -166,6 +177,7 @@ def cmd_traffic(ns) -> int:
     for c in shown_cmds:
         print(f"  -> {c}")
     print("```\n")
+    print_sources(line)
     print(f"Calibration: the same counters over `en_copy_bytes` of 1 GiB (reads 1 GiB, writes 1 GiB) give "
           f"{calib['FETCH_SIZE']:.1f} bytes per FETCH_SIZE unit and {calib['WRITE_SIZE']:.1f} bytes per WRITE_SIZE unit; "
           f"the columns below are scaled by that. Each op ran {calls} times; traffic = counter total / {calls}.\n")
@@ -212,6 +224,7 @@ def cmd_counters(ns) -> int:
     print("Command (MI355X box, repo root; the summary below is this command's stdout):\n")
     print(f"```\npython3 bench_profiles.py counters --workload {ns.workload}"
           f"{' --all-ops' if ns.all_ops else ' --form ' + ns.form}\n  -> {shown}\n```\n")
+    print_sources(line)
     print("All columns are sums over the launches of an op divided as stated.  `GRBM_GUI_ACTIVE` is summed over the 8 "
           "XCDs, so SIMD cycles of a launch = GRBM_GUI_ACTIVE / 8 x 1024 SIMDs.  `SQ_WAVE_CYCLES`, "
           "`SQ_ACTIVE_INST_VALU` and `SQ_WAIT_INST_ANY` count in units of four cycles.\n")
@@ -258,6 +271,7 @@ def cmd_issue(ns) -> int:
     print("Command (MI355X box, repo root; the summary below is this command's stdout):\n")
     print(f"```\npython3 bench_profiles.py issue --workload {ns.workload}"
           f"{' --all-ops' if ns.all_ops else ' --form ' + ns.form}\n  -> {shown}\n```\n")
+    print_sources(line)
     print("Shares are of all SIMD cycles of an op's launches (`GRBM_GUI_ACTIVE` / 8 XCDs x 1024 SIMDs); the queue "
           "counters are per SIMD as well.  Instruction counts are per launch, summed over all waves.\n")
     print("| op (key in the bench line) | kernels | matrix pipe busy | matrix and vector pipe busy at once | "
@@ -312,6 +326,7 @@ def cmd_memsys(ns) -> int:
     for sh in shown_all:
         print(f"  -> {sh}")
     print("```\n")
+    print_sources(line)
     print("Requests are per launch, in millions.  Requests to memory: reads of 32 / 64 bytes (the rest are 128-byte "
           "reads), writes of 64 bytes (the rest 32).  Stall shares: cycles summed over the L2 channels divided by "
           "128 channels x the launch's cycles (`GRBM_GUI_ACTIVE` counts the cycles of all 8 XCDs).\n")

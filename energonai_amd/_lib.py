@@ -31,7 +31,7 @@ SIGNATURES = {
     "en_repad": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int64, c_int, c_int, c_void_p]),
     "en_transpose_pad": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p]),
     "en_transpose_pad_heads": (c_int, [c_void_p, c_void_p, c_void_p] + [c_int] * 8 + [c_void_p]),
-    "en_kv_append": (c_int, [c_void_p] * 5 + [c_int] * 4 + [c_int64] * 5 + [c_int, c_void_p]),
+    "en_kv_append": (c_int, [c_void_p] * 5 + [c_int] * 4 + [c_int64] * 5 + [c_int, c_void_p, c_void_p]),
     "en_transpose_depad": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p]),
     "en_ft_build_offsets": (c_int, [c_void_p, c_int, c_int, c_void_p, c_void_p, c_void_p]),
     "en_ft_remove_padding": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int64, c_int, c_void_p]),

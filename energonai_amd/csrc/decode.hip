@@ -180,7 +180,7 @@ static int check_decode(const void *x, const void *kv, const void *out, const in
 namespace en {
 
 // Appends one new K row and one new V row per (batch, head) to the caches at position
-// kv_lens[b]; sequences whose cache is full are left alone.  Bytes are moved as they are.
+// kv_lens[b]; sequences whose cache is full are left alone and counted.  Bytes are moved as they are.
 struct AppendArgs {
   const unsigned char *k_new, *v_new;
   unsigned char *k_cache, *v_cache;
@@ -189,13 +189,17 @@ struct AppendArgs {
   int row_bytes;
   int64_t n_sb, n_sh;           // strides of the new rows, bytes
   int64_t c_sb, c_sh, c_ss;     // strides of the caches, bytes
+  int32_t *overflow;            // counts the sequences that had no room (null: not counted)
 };
 
 template <typename Vec>
 __global__ __launch_bounds__(kWave) void kv_append_kernel(AppendArgs a) {
   const int h = blockIdx.x, b = blockIdx.y;
   const int pos = a.kv_lens[b];
-  if (pos < 0 || pos >= a.Sk) return;
+  if (pos < 0 || pos >= a.Sk) {
+    if (a.overflow && h == 0 && threadIdx.x == 0) atomicAdd(a.overflow, 1);
+    return;
+  }
   const int64_t src = (int64_t)b * a.n_sb + (int64_t)h * a.n_sh;
   const int64_t dst = (int64_t)b * a.c_sb + (int64_t)h * a.c_sh + (int64_t)pos * a.c_ss;
   for (int i = threadIdx.x * (int)sizeof(Vec); i < a.row_bytes; i += kWave * (int)sizeof(Vec)) {
@@ -211,9 +215,10 @@ extern "C" {
 int en_kv_append(const void *k_new, const void *v_new, void *k_cache, void *v_cache, const int32_t *kv_lens,
                  int batch, int head_num, int k_seq_len, int size_per_head, int64_t new_stride_b,
                  int64_t new_stride_h, int64_t cache_stride_b, int64_t cache_stride_h, int64_t cache_stride_s,
-                 int elem_size, en_stream_t stream) {
+                 int elem_size, int32_t *overflow, en_stream_t stream) {
   using namespace en;
   if (!k_new || !v_new || !k_cache || !v_cache || !kv_lens) return EN_ERR_NULL;
+  if (overflow && !aligned_to(overflow, 4)) return EN_ERR_ALIGN;
   if (elem_size != 2 && elem_size != 4) return EN_ERR_DTYPE;
   if (batch < 1 || head_num < 1 || k_seq_len < 1 || size_per_head < 1) return EN_ERR_SHAPE;
   if (batch > 65535) return EN_ERR_SHAPE;
@@ -222,7 +227,7 @@ int en_kv_append(const void *k_new, const void *v_new, void *k_cache, void *v_ca
   AppendArgs a{(const unsigned char *)k_new, (const unsigned char *)v_new, (unsigned char *)k_cache,
                (unsigned char *)v_cache, kv_lens, head_num, k_seq_len, size_per_head * elem_size,
                new_stride_b * elem_size, new_stride_h * elem_size, cache_stride_b * elem_size,
-               cache_stride_h * elem_size, cache_stride_s * elem_size};
+               cache_stride_h * elem_size, cache_stride_s * elem_size, overflow};
   const dim3 grid((unsigned)head_num, (unsigned)batch, 1);
   hipStream_t s = (hipStream_t)stream;
   const bool v16 = (a.row_bytes % 16 == 0) && aligned_to(k_new, 16) && aligned_to(v_new, 16) &&

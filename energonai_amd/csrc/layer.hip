@@ -7,6 +7,7 @@
 // launch of transpose_pad: six launches.
 #include "common.hip.h"
 
+#include <initializer_list>
 #include <mutex>
 
 namespace en {
@@ -40,16 +41,31 @@ static int scratch_for_current_device(unsigned char **out) {
 }
 
 // Lays out 256-byte aligned pieces of the scratch array: take() returns a piece's offset, or -1 for a piece the
-// call does not need; `used` may run past the end (checked by the caller before anything is launched).
+// call does not need.  `used` may run past the end (checked by the caller before anything is launched) but never
+// wraps: a piece that does not fit what is left pins it at one past the array's size, whatever follows.
 struct Layout {
   int64_t used = 0;
   int64_t take(bool wanted, int64_t bytes) {
     if (!wanted) return -1;
     const int64_t at = used;
-    used += (bytes + 255) / 256 * 256;
+    if (bytes < 0 || used > kLayerScratchBytes || bytes > kLayerScratchBytes - used) used = kLayerScratchBytes + 1;
+    else used += (bytes + 255) / 256 * 256;
     return at;
   }
 };
+
+// Product of extents that stops growing at one past the array's size, so that absurd shapes cannot wrap the
+// signed arithmetic of a piece's size into something small.
+static int64_t piece_bytes(std::initializer_list<int64_t> factors) {
+  int64_t p = 1;
+  for (int64_t f : factors) {
+    if (f < 0) return -1;
+    if (f == 0) return 0;
+    if (p > (kLayerScratchBytes + 1) / f) return kLayerScratchBytes + 1;
+    p *= f;
+  }
+  return p;
+}
 
 }  // namespace en
 
@@ -166,11 +182,15 @@ extern "C" int en_padding_removal_layer_noalloc(const void *hidden_padded, const
   Layout l;
   const bool padded = attention_form < 2;
   const int64_t o_cu = l.take(true, (B + 1) * 4), o_lens = l.take(true, B * 4);
-  const int64_t o_offs = l.take(fold_depad != 0, T * 4), o_x = l.take(fold_depad == 0, T * hidden * es);
-  const int64_t score_elems = attention_form == 4 ? en_packed_scores_elems(batch, head_num, max_seq_len, dtype) : B * H * S * S;
-  const int64_t o_qkv = l.take(padded, B * H * S * 3 * D * es);
-  const int64_t o_scores = l.take(attention_form == 0 || attention_form >= 3, score_elems * es);
-  const int64_t o_ctx = l.take(padded, B * H * S * D * es), o_ctxp = l.take(true, T * H * D * es);
+  const int64_t o_offs = l.take(fold_depad != 0, piece_bytes({T, 4})), o_x = l.take(fold_depad == 0, piece_bytes({T, hidden, es}));
+  // packed scores: a unit's slot is below S * (S + 128 bytes' worth) elements, so the product below bounds it
+  const bool scores_fit = piece_bytes({B, H, S, S, es}) <= kLayerScratchBytes;
+  const int64_t score_bytes = attention_form == 4
+      ? (scores_fit ? en_packed_scores_elems(batch, head_num, max_seq_len, dtype) * es : kLayerScratchBytes + 1)
+      : piece_bytes({B, H, S, S, es});
+  const int64_t o_qkv = l.take(padded, piece_bytes({B, H, S, 3 * D, es}));
+  const int64_t o_scores = l.take(attention_form == 0 || attention_form >= 3, score_bytes);
+  const int64_t o_ctx = l.take(padded, piece_bytes({B, H, S, D, es})), o_ctxp = l.take(true, piece_bytes({T, H, D, es}));
   if (l.used > kLayerScratchBytes) return EN_ERR_SCRATCH;
   unsigned char *base = nullptr;   // the array's address on the current device; never the array's name
   int rc = scratch_for_current_device(&base);

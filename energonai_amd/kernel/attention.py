@@ -181,7 +181,10 @@ def attn_fused_varlen(q, k, v, batch_size: int, max_seq_len: int, seq_len_list, 
 
 def packed_scores_elems(batch_size: int, head_num: int, seq_len: int, dtype) -> int:
     """Elements of the packed causal score tensor of a self-attention batch: per (batch, head) unit the visible
-    prefix of every row, rounded up to one 16-byte vector, back to back; each unit owns the slot of a full-length one."""
+    prefix of every row, rounded up to a whole 128-byte group (``V`` = 64 fp16 / bf16 or 32 fp32 entries), back to
+    back: row ``q`` starts ``V * (V*t*(t+1)/2 + (q - V*t) * (t+1))`` elements into its unit, ``t = q // V``, and holds
+    ``V * (t+1)`` elements; each unit owns the slot of a full-length one.  QK^T writes and the softmax zeroes a row
+    only up to the end of the 16-byte vector that holds its last visible entry."""
     n = _lib.fn.en_packed_scores_elems(int(batch_size), int(head_num), int(seq_len), _lib._DTYPE_TAG[dtype])
     if n <= 0:
         raise RuntimeError("packed_scores_elems: bad arguments")
@@ -288,9 +291,11 @@ def kv_cache_fill(src, cache, batch_size: int, seq_len_list, head_first: int = 0
     return cache
 
 
-def kv_cache_append(k_new, v_new, k_cache, v_cache, kv_len_list):
+def kv_cache_append(k_new, v_new, k_cache, v_cache, kv_len_list, overflow: Optional[torch.Tensor] = None):
     """Writes the new token's rows ``k_new`` / ``v_new`` (``[B,H,D]`` views) into the ``[B,H,Smax,D]`` caches at
-    position ``kv_len[b]``.  The caller advances the lengths afterwards."""
+    position ``kv_len[b]``.  The caller advances the lengths afterwards.  A sequence whose cache is full keeps
+    its rows and loses the new one; ``overflow`` (one int32 on the device) is incremented once per such
+    sequence, so that a caller without a host-side bound of the lengths can still notice."""
     for t, n in ((k_new, "k_new"), (v_new, "v_new")):
         _lib.require_gpu(t, n, contiguous=False)
         if t.dim() != 3 or t.stride(2) != 1:
@@ -302,10 +307,15 @@ def kv_cache_append(k_new, v_new, k_cache, v_cache, kv_len_list):
     if k_new.shape != (B, H, D) or v_new.shape != (B, H, D) or k_new.dtype != k_cache.dtype:
         raise RuntimeError("kv_cache_append: new rows must be [B,H,D] of the cache dtype")
     info = seq_info(kv_len_list, B, k_cache.device)
+    if overflow is not None:
+        _lib.require_gpu(overflow, "overflow")
+        if overflow.dtype != torch.int32 or overflow.numel() < 1:
+            raise RuntimeError("kv_cache_append: overflow must be an int32 tensor of at least one element")
     with _lib.device_guard(k_cache):
         _lib.check(_lib.fn.en_kv_append(k_new.data_ptr(), v_new.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(),
                                         info.lens.data_ptr(), B, H, Smax, D, k_new.stride(0), k_new.stride(1), *cs,
-                                        k_cache.element_size(), _lib.stream_of(k_cache)), "kv_cache_append")
+                                        k_cache.element_size(), _lib.ptr(overflow), _lib.stream_of(k_cache)),
+                   "kv_cache_append")
 
 
 def decode_qk(q, k_cache, kv_len_list, *, alpha: float = 1.0, out: Optional[torch.Tensor] = None):

@@ -158,8 +158,8 @@ def _layer_one_call(hidden_padded, qkv_packed, info, B, S, H, D, hid, T, gamma, 
         ctx_packed = torch.empty((1, T, H, D), dtype=dt, device=dev)
     else:
         _lib.require_gpu(ctx_out, "ctx_out")
-        if ctx_out.numel() != T * H * D or ctx_out.dtype != dt:
-            raise RuntimeError("padding_removal_layer: ctx_out must be [1,T,H,D] of the activation dtype")
+        if ctx_out.numel() != T * H * D or ctx_out.dtype != dt or not ctx_out.is_contiguous():
+            raise RuntimeError("padding_removal_layer: ctx_out must be a contiguous [1,T,H,D] tensor of the activation dtype")
         ctx_packed = ctx_out
     qkv = torch.empty((B, H, S, 3 * D), dtype=dt, device=dev) if form < 2 else None
     ctx = torch.empty((B, H, S, D), dtype=dt, device=dev) if form < 2 else None
@@ -201,16 +201,21 @@ def padding_removal_layer_noalloc(hidden_padded: torch.Tensor, qkv_packed: torch
         _lib.require_gpu(t, name)
     if seq_lens.dtype not in (torch.int32, torch.int64) or seq_lens.numel() < B:
         raise RuntimeError("padding_removal_layer_noalloc: seq_lens must hold batch int32 or int64 lengths")
-    if qkv_packed.numel() != T * H * 3 * D or qkv_packed.dtype != dt:
-        raise RuntimeError("padding_removal_layer_noalloc: qkv_packed must be [1,T,H,3D] of the activation dtype")
-    if out.numel() != T * hid or out.dtype != dt:
-        raise RuntimeError("padding_removal_layer_noalloc: out must be [1,T,hidden] of the activation dtype")
+    if qkv_packed.numel() != T * H * 3 * D or qkv_packed.dtype != dt or not qkv_packed.is_contiguous():
+        raise RuntimeError("padding_removal_layer_noalloc: qkv_packed must be a contiguous [1,T,H,3D] tensor of the "
+                           "activation dtype")
+    if out.numel() != T * hid or out.dtype != dt or not out.is_contiguous():
+        raise RuntimeError("padding_removal_layer_noalloc: out must be a contiguous [1,T,hidden] tensor of the "
+                           "activation dtype")
+    if not hidden_padded.is_contiguous() or not seq_lens.is_contiguous():
+        raise RuntimeError("padding_removal_layer_noalloc: hidden_padded and seq_lens must be contiguous")
     if gamma.dtype != dt or beta.dtype != dt or gamma.numel() != hid or beta.numel() != hid:
         raise RuntimeError("padding_removal_layer_noalloc: gamma and beta must be [hidden] of the activation dtype")
     if dense_out is not None:
         _lib.require_gpu(dense_out, "dense_out")
-        if dense_out.numel() != T * hid or dense_out.dtype != dt:
-            raise RuntimeError("padding_removal_layer_noalloc: dense_out must be [1,T,hidden] of the activation dtype")
+        if dense_out.numel() != T * hid or dense_out.dtype != dt or not dense_out.is_contiguous():
+            raise RuntimeError("padding_removal_layer_noalloc: dense_out must be a contiguous [1,T,hidden] tensor of the "
+                               "activation dtype")
     elif hid != H * D:
         raise RuntimeError("padding_removal_layer_noalloc: without dense_out the LayerNorm width must equal "
                            "heads * size_per_head")
@@ -229,7 +234,8 @@ def decode_layer(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, 
                  gamma: torch.Tensor, beta: torch.Tensor, eps: float = 1e-5, scale: Optional[float] = None,
                  dense_out: Optional[torch.Tensor] = None, keep: bool = False):
     """One cached decode step: a single new query per sequence against a ragged
-    cache, then transpose_depad and residual + LayerNorm on the B new tokens.
+    cache, then residual + LayerNorm on the B new tokens (transpose_depad of a
+    one-row sequence is the identity, so the context is passed on as a view).
 
     q [B,H,1,D]; caches [B,H,Smax,D]; residual [1,B,hid].
     """
@@ -243,7 +249,7 @@ def decode_layer(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, 
     scores = decode_qk(q, k_cache, info)
     probs = scale_mask_softmax(B, 1, H, scores, info, scale=scale, causal=True, k_seq_len=Smax, q_len_list=ones)
     ctx = decode_pv(probs, v_cache, info)
-    ctx_packed = transpose_depad(ctx, B, B, 1, ones, H, D)
+    ctx_packed = ctx.view(1, B, H, D)      # [B,H,1,D] with one query per sequence is [1,T=B,H,D] already
     attn_out = ctx_packed.view(1, B, H * D) if dense_out is None else dense_out
     y = layer_norm_forward(attn_out, gamma, beta, (hid,), eps, residual=residual)
     if keep:

@@ -32,8 +32,8 @@ class SeqInfo:
         self.batch_size = batch_size
         self._total = total
         self._source = source           # keeps the caller's tensor alive while cached
-        self._row_offsets = {}          # (max_seq_len, left_padded) -> int32 [T]
-        self._tile_tables = {}          # (head_num, q_seq_len) -> int32 workgroup order of the attention kernels
+        self._row_offsets = {}          # (max_seq_len, left_padded, version of lens) -> int32 [T]
+        self._tile_tables = {}          # (head_num, q_seq_len, order, version of lens) -> int32 workgroup order
         self._ready = []                # events recorded behind the kernels that produced the arrays above
         self._ordered = set()           # raw streams already ordered behind every event of _ready
 
@@ -45,6 +45,7 @@ class SeqInfo:
         ev = torch.cuda.Event()
         ev.record(torch.cuda.current_stream(self.lens.device))
         self._ready.append(ev)
+        del self._ready[:-8]            # lengths that change every step rebuild their tables every step
         self._ordered = {_lib.stream_of(self.lens)}
 
     def order_current_stream(self) -> None:
@@ -74,12 +75,23 @@ class SeqInfo:
         return self._total
 
 
+    def _lens_version(self):
+        """Version counter of the lengths, part of every key under which something derived from them is kept:
+        a caller that owns ``lens`` may change it in place (the K/V cache advances its lengths every step), and
+        what was derived from the old lengths must then not be found again.  Tensors created under
+        ``torch.inference_mode()`` have no counter; ``None`` then means "do not keep"."""
+        try:
+            return self.lens._version
+        except RuntimeError:
+            return None
+
     def row_offsets(self, max_seq_len: int, left_padded: bool) -> torch.Tensor:
         """``off[t]`` = row of token ``t`` in the padded ``[B*S]`` numbering minus ``t``; computed once per
         batch and bucket by one small kernel (the reference's ft offsets, csrc/transpose_pad_fusion_kernel.cu:
         112-131, made aware of left padding)."""
-        key = (int(max_seq_len), bool(left_padded))
-        off = self._row_offsets.get(key)
+        version = self._lens_version()
+        key = (int(max_seq_len), bool(left_padded), version)
+        off = None if version is None and self._mutable() else self._row_offsets.get(key)
         self.order_current_stream()
         if off is None:
             off = torch.empty(max(self.total, 1), dtype=torch.int32, device=self.lens.device)
@@ -87,8 +99,15 @@ class SeqInfo:
                 _lib.check(_lib.fn.en_padding_offsets(self.lens.data_ptr(), self.batch_size, key[0], int(key[1]),
                                                       off.data_ptr(), _lib.stream_of(self.lens)), "padding_offsets")
                 self.produced_on_current_stream()
-            self._row_offsets[key] = off
+            if version is not None or not self._mutable():
+                self._row_offsets = {k: o for k, o in self._row_offsets.items() if k[2] == version}
+                self._row_offsets[key] = off
         return off
+
+    def _mutable(self) -> bool:
+        """True when the lengths belong to a caller that may edit them in place (no prefix was computed from
+        them, or they are the caller's own tensor)."""
+        return self.cu_seqlens is None or self._source is self.lens
 
 
     def tile_table(self, head_num: int, q_seq_len: int, unit_kv_bytes: int = 1 << 30) -> torch.Tensor:
@@ -97,8 +116,9 @@ class SeqInfo:
         hold at full length: up to 256 KB the last tiles of all units run first, above that a unit's tiles stay
         together.  Computed once per batch, head count, bucket and order by one small kernel and reused by every
         layer."""
-        key = (int(head_num), int(q_seq_len), int(unit_kv_bytes) <= TILES_FIRST_MAX_KV_BYTES)
-        tab = self._tile_tables.get(key)
+        version = self._lens_version()
+        key = (int(head_num), int(q_seq_len), int(unit_kv_bytes) <= TILES_FIRST_MAX_KV_BYTES, version)
+        tab = None if version is None and self._mutable() else self._tile_tables.get(key)
         self.order_current_stream()
         if tab is None:
             n = int(_lib.fn.en_attn_tile_table_elems(self.batch_size, key[0], key[1]))
@@ -107,7 +127,10 @@ class SeqInfo:
                 _lib.check(_lib.fn.en_attn_tile_table(self.lens.data_ptr(), self.batch_size, key[0], key[1], int(key[2]),
                                                       tab.data_ptr(), _lib.stream_of(self.lens)), "attn_tile_table")
                 self.produced_on_current_stream()
-            self._tile_tables[key] = tab
+            if version is not None or not self._mutable():
+                # tables of older versions of the lengths can never be found again: drop them
+                self._tile_tables = {k: t for k, t in self._tile_tables.items() if k[3] == version}
+                self._tile_tables[key] = tab
         return tab
 
 

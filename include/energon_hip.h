@@ -155,10 +155,15 @@ int en_scale_mask_softmax(void *src, const int32_t *k_lens, const int32_t *q_len
 /* Packed causal scores.  Under a causal mask of a self-attention batch row q of a (batch, head) unit holds
  * q + 1 visible scores; in [B,H,S,S] those prefixes start a whole row pitch apart and every kernel of the
  * chain QK^T -> softmax -> PV streams short ragged pieces of memory.  The packed layout keeps the prefixes only,
- * each rounded up to one 16-byte vector of V = 16 / element size entries, back to back: row q of a unit starts
- * V * (V * t * (t + 1) / 2 + (q - V * t) * (t + 1)) elements into it, t = q / V, and holds V * (t + 1) elements;
- * every unit owns a slot as large as a full-length one (row_start(seq_len) elements), unit (b, h) the slot
- * b * head_num + h.  en_packed_scores_elems returns the elements of the whole tensor (0 on bad arguments).
+ * each rounded up to a whole group of 128 bytes, back to back.  With V = 128 / element size entries per group
+ * (64 for fp16 / bf16, 32 for fp32) and t = q / V (integer division), row q of a unit starts
+ *   row_start(q) = V * (V * t * (t + 1) / 2 + (q - V * t) * (t + 1))
+ * elements into the unit and holds V * (t + 1) elements; every unit owns a slot as large as a full-length one,
+ * row_start(seq_len) elements (seq_len = 1024, fp16: 557 056), unit (b, h) the slot b * head_num + h.
+ * en_packed_scores_elems returns the elements of the whole tensor, batch * head_num * row_start(seq_len)
+ * (0 on bad arguments).  Of a row's group the kernels write the visible prefix only: QK^T up to the end of the
+ * 16-byte vector that holds the last visible score, the softmax zeros up to that same point; the rest of the
+ * group is never written and never read.
  * An internal format of the step: the reference's [B,H,S,S] tensor (scale_mask_softmax_wrapper.cpp:25-44) stays
  * the format of en_scale_mask_softmax. */
 int64_t en_packed_scores_elems(int batch, int head_num, int seq_len, int dtype);
@@ -244,11 +249,13 @@ int en_decode_pv(const void *p, const void *v_cache, void *ctx, const int32_t *k
  * (energonai/model/attention.py:66-71,89-98).  k_new / v_new are addressed as
  * base + b*new_stride_b + h*new_stride_h + d, the caches as
  * base + b*stride_b + h*stride_h + s*stride_s + d (elements of elem_size bytes).
- * A sequence with kv_lens[b] >= k_seq_len is left alone. */
+ * A sequence with kv_lens[b] >= k_seq_len (or < 0) has no room: its rows are not written.  So that this cannot
+ * go unnoticed, overflow (device, one int32, or NULL) counts such sequences: the kernel adds one to it for each
+ * (the caller zeroes it when it likes and reads it when it likes; the call itself never synchronises). */
 int en_kv_append(const void *k_new, const void *v_new, void *k_cache, void *v_cache, const int32_t *kv_lens,
                  int batch, int head_num, int k_seq_len, int size_per_head, int64_t new_stride_b,
                  int64_t new_stride_h, int64_t cache_stride_b, int64_t cache_stride_h, int64_t cache_stride_s,
-                 int elem_size, en_stream_t stream);
+                 int elem_size, int32_t *overflow, en_stream_t stream);
 
 /* Fused attention (an addition: the reference callers run matmul, softmax, matmul,
  * examples/bert/bert.py:108-119): ctx[b,h,i,:] = sum_j softmax_j(scale * <q_i, k_j>) v[b,h,j,:]

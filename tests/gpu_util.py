@@ -65,3 +65,16 @@ def assert_stored_close(got, want, dtype, base=None, what=""):
     base = BASE[dtype] if base is None else base
     ex = excess(got, want, dtype)
     assert ex <= base, f"{what}: error exceeds half an ulp of the stored value by {ex:.3e} > {base:.3e}"
+
+
+def assert_ctx_close(got, want, dtype, what=""):
+    """The bound for attention outputs.  16-bit storage: BASE[dtype] on top of half an ulp of the stored value,
+    elementwise (assert_stored_close).  fp32: a relative bound, 1e-5 x max(1, largest reference magnitude),
+    because fp32 results carry rounding in proportion to the values they add up."""
+    if got.numel() == 0:
+        return
+    if dtype == torch.float32:
+        err = max_abs(got, want)
+        assert err <= BASE[dtype] * max(1.0, float(want.abs().max())), f"{what}: {err:.3e}"
+    else:
+        assert_stored_close(got, want, dtype, what=what)

@@ -94,8 +94,8 @@ def test_entry_points_validate_before_launch():
     assert lib.en_repad(None, 32, 48, 1, 1, 1, 2, 0, None) == -1
     assert lib.en_repad(16, 32, 48, 1, 0, 1, 2, 0, None) == -2           # max_seq_len 0
     assert lib.en_transpose_pad_heads(16, 32, 48, 1, 1, 4, 8, 6, 4, 1, 2, None) == -2   # heads 4..7 of a 6-row source
-    assert lib.en_kv_append(16, 32, 48, 64, None, 1, 1, 1, 8, 8, 8, 8, 8, 8, 2, None) == -1
-    assert lib.en_kv_append(16, 32, 48, 64, 80, 1, 1, 1, 8, 8, 8, 8, 8, 8, 3, None) == -3   # element size 3
+    assert lib.en_kv_append(16, 32, 48, 64, None, 1, 1, 1, 8, 8, 8, 8, 8, 8, 2, None, None) == -1
+    assert lib.en_kv_append(16, 32, 48, 64, 80, 1, 1, 1, 8, 8, 8, 8, 8, 8, 3, None, None) == -3   # element size 3
     assert lib.en_attn_fused(16, 32, 48, 64, 80, None, 1, 1, 8, 8, 64, i64x3, i64x3, i64x3, i64x3, None, None, 1.0, 1, 0,
                              None, None) == -3                           # fp32 is not a fused-attention dtype
     assert lib.en_attn_fused(16, 32, 48, 64, 80, None, 1, 1, 8, 8, 64, i64x3, i64x3, i64x3, i64x3, None, None, 0.0, 1, 1,
@@ -108,6 +108,16 @@ def test_entry_points_validate_before_launch():
                                         1.0, 1e-5, 1, 0, 0, None, 1, None, None) == -2   # LayerNorm width 32 != 2 heads x 8, no dense_out
     assert lib.en_padding_removal_layer(16, 32, None, 48, 64, 80, None, 112, 128, 144, 160, 176, 192, 1, 8, 2, 8, 16, 4,
                                         1.0, 1e-5, 1, 0, 0, None, 1, None, None) == -1   # unfused form without the padded buffer
+    # the entry point that allocates nothing sizes its pieces without wrapping: absurd extents whose products
+    # overflow 64-bit arithmetic are refused before anything is launched (arguments: ..., y, seq_lens, i64, B, S, H,
+    # D, hidden, T, scale, eps, causal, left, form, fold, dtype, stream)
+    for form in (0, 1, 2, 3, 4):
+        for fold in (0, 1):
+            assert lib.en_padding_removal_layer_noalloc(16, 32, None, 48, 64, 80, 96, 0, 65536, 2 ** 31 - 1, 2 ** 31 - 1,
+                                                        2 ** 31 - 1, 2 ** 62, 65536 * (2 ** 31 - 1), 1.0, 1e-5, 1, 0,
+                                                        form, fold, 1, None) == -7
+    assert lib.en_padding_removal_layer_noalloc(16, 32, None, 48, 64, 80, 96, 0, 4, 2 ** 20, 2 ** 20, 2 ** 20, 2 ** 40,
+                                                4, 1.0, 1e-5, 1, 0, 0, 0, 1, None) == -7
 
 
 def test_python_api_keeps_reference_names_and_signatures():

@@ -104,6 +104,17 @@ def test_kv_cache_fill_and_append_bit_exact(dtype):
     with pytest.raises(RuntimeError, match="max_seq_len"):
         small.append(new_g[:, :H], new_g[:, H:2 * H])
     assert small.lens.cpu().tolist() == [n + 2 for n in lens]
+    # a caller of the C entry point itself (no host-side bound of the lengths) is told through a device counter:
+    # sequence 1 is full now, the other two take the row
+    overflow = torch.zeros(1, dtype=torch.int32, device="cuda")
+    before_k = small.k.clone()
+    K.kv_cache_append(new_g[:, :H], new_g[:, H:2 * H], small.k, small.v, small.info, overflow=overflow)
+    assert overflow.item() == 1
+    assert torch.equal(small.k[1], before_k[1])
+    for b in (0, 2):
+        assert torch.equal(small.k[b, :, lens[b] + 2], new_g[b, :H])
+    K.kv_cache_append(new_g[:, :H], new_g[:, H:2 * H], small.k, small.v, small.info, overflow=overflow)
+    assert overflow.item() == 2
 
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.float32])
