@@ -41,6 +41,7 @@ KERNEL_KEYS = [
     ("softmax", "scale_mask_softmax"),
     ("attn_pv", "attn_pv"),
     ("layernorm", "layernorm_residual"),
+    ("decode_attn", "decode_attn"),
     ("decode_qk", "decode_qk"),
     ("decode_pv", "decode_pv"),
     ("attn_fused", "attn_fused_packed"),

@@ -179,6 +179,190 @@ static int check_decode(const void *x, const void *kv, const void *out, const in
 
 namespace en {
 
+// ---------------------------------------------------------------------------------------------------------------
+// Single-pass decode attention: ctx = softmax(scale * q K^T) V for one query per sequence, K and V each read
+// once, scores and probabilities never written.  One workgroup per (batch, head); LPK lanes cover one cached row
+// (16 bytes each), so the workgroup's NT / LPK lane groups take NT / LPK keys per step.  Two stages of registers:
+// the K and V pieces of the next step are in flight while this step's are worked on, and the kernel stays within
+// 64 registers so that two 1024-lane workgroups share a CU (measured on 72 heads x 64 caches of up to 2048
+// positions, 2.6 GB: 6.7 TB/s; four pieces per lane and stage at one workgroup per CU 5.9, one stage of four
+// pieces as in the two-kernel forms 5.3; a third stage spills).  Each lane group carries its own running maximum, sum and
+// output slice (online softmax, maximum and exponent in the log2 domain with the scale folded in); the groups are
+// combined once, through LDS, at the end.  The sequences are taken longest first (rank computed inside each
+// workgroup from the lengths, batches of up to kRankBatch): the launch then ends on its short units instead of on
+// whatever the last batch index happens to hold.
+// ---------------------------------------------------------------------------------------------------------------
+struct DecodeAttnArgs {
+  const void *q;      // [B,H,D]
+  const void *k, *v;  // caches [B,H,Smax,D], strided
+  void *ctx;          // [B,H,D]
+  const int32_t *kv_lens;
+  int B, H, Sk, D;
+  int64_t k_sb, k_sh, k_ss, v_sb, v_sh, v_ss;
+  float c_exp;        // scale * log2(e)
+};
+
+constexpr int kRankBatch = 256;
+
+template <int DT, int LPK, bool STREAM>
+__global__ __launch_bounds__(STREAM ? kStreamBlock : kBlock, 8) void decode_attn_kernel(DecodeAttnArgs a) {
+  constexpr int NT = STREAM ? kStreamBlock : en::kBlock;
+  typedef Elem<DT> E;
+  typedef typename E::T T;
+  constexpr int EPV = 16 / E::kSize;
+  constexpr int G = NT / LPK;        // lane groups = keys per step
+  constexpr int U = 1;               // keys per lane group and stage
+  constexpr int W = LPK * EPV;       // channels the lanes of a group cover (>= D)
+  __shared__ float s_m[G], s_l[G], s_w[G];
+  __shared__ float s_acc[G][W + 1];
+  __shared__ int s_len[kRankBatch];
+  __shared__ int s_b;
+  const int tid = threadIdx.x;
+  const int h = blockIdx.x;
+  int b = blockIdx.y;
+  if (a.B <= kRankBatch && a.B > 1) {
+    // batch index whose length ranks blockIdx.y-th (longest first, ties by index)
+    if (tid < a.B) s_len[tid] = min(a.kv_lens[tid], a.Sk);
+    __syncthreads();
+    if (tid < a.B) {
+      const int mine = s_len[tid];
+      int rank = 0;
+      for (int j = 0; j < a.B; ++j) {
+        const int lj = s_len[j];
+        rank += (lj > mine || (lj == mine && j < tid)) ? 1 : 0;
+      }
+      if (rank == (int)blockIdx.y) s_b = tid;
+    }
+    __syncthreads();
+    b = s_b;
+  }
+  const int c = tid % LPK, g = tid / LPK;
+  const int kl = max(min(a.kv_lens[b], a.Sk), 0);
+  const T *q = reinterpret_cast<const T *>(a.q) + ((int64_t)b * a.H + h) * a.D;
+  const T *kbase = reinterpret_cast<const T *>(a.k) + (int64_t)b * a.k_sb + (int64_t)h * a.k_sh;
+  const T *vbase = reinterpret_cast<const T *>(a.v) + (int64_t)b * a.v_sb + (int64_t)h * a.v_sh;
+  T *ctx = reinterpret_cast<T *>(a.ctx) + ((int64_t)b * a.H + h) * a.D;
+  const bool cv = c * EPV < a.D;     // lanes past the head size idle (head sizes such as 80 and 96)
+
+  float qv[EPV];
+  {
+    Pack<T, EPV> pk;
+#pragma unroll
+    for (int e = 0; e < EPV; ++e) pk.v[e] = E::from_float(0.f);
+    if (cv) pk = load_pack<T, EPV>(q + c * EPV);
+#pragma unroll
+    for (int e = 0; e < EPV; ++e) qv[e] = E::to_float(pk.v[e]) * a.c_exp;
+  }
+  float m_run = -INFINITY, l_run = 0.f;
+  float acc[EPV];
+#pragma unroll
+  for (int e = 0; e < EPV; ++e) acc[e] = 0.f;
+
+  // Bounds-checked buffer loads: a row at or past the sequence's length (and a lane past the head size) reads
+  // zeros without a branch, so the loads of the next stage can be issued ahead of this stage's arithmetic and the
+  // compiler counts what is outstanding statically.
+  const rsrc_t k_rsrc = make_rsrc(kbase, kl > 0 ? (uint32_t)(((int64_t)(kl - 1) * a.k_ss + a.D) * E::kSize) : 0u);
+  const rsrc_t v_rsrc = make_rsrc(vbase, kl > 0 ? (uint32_t)(((int64_t)(kl - 1) * a.v_ss + a.D) * E::kSize) : 0u);
+  const uint32_t k_row = (uint32_t)(a.k_ss * E::kSize), v_row = (uint32_t)(a.v_ss * E::kSize);
+  const uint32_t col = cv ? (uint32_t)(c * 16) : kOutOfRange;
+  constexpr int AUX = STREAM ? 2 : 0;
+  auto load_stage = [&](uint4 (&kk)[U], uint4 (&vv)[U], int k0) {
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int key = k0 + u * G + g;
+      const uint32_t in = key < kl ? 0u : kOutOfRange;       // past the end: out of range whatever the stride
+      kk[u] = buffer_load16<AUX>(k_rsrc, (uint32_t)key * k_row + col | in);
+      vv[u] = buffer_load16<AUX>(v_rsrc, (uint32_t)key * v_row + col | in);
+    }
+  };
+  auto compute_stage = [&](const uint4 (&kk)[U], const uint4 (&vv)[U], int k0) {
+    float sc[U];
+    float m_new = m_run;
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int key = k0 + u * G + g;
+      const Pack<T, EPV> kp = __builtin_bit_cast(Pack<T, EPV>, kk[u]);
+      float dot = 0.f;
+#pragma unroll
+      for (int e = 0; e < EPV; ++e) dot += qv[e] * E::to_float(kp.v[e]);
+      dot = group_allreduce<OpSum, LPK>(dot);
+      sc[u] = key < kl ? dot : -INFINITY;
+      m_new = fmaxf(m_new, sc[u]);
+    }
+    if (m_new > -INFINITY) {            // this group has seen a key: (-inf) - (-inf) never reaches exp2
+      const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);      // exp2(-inf) = 0 on the first key
+      l_run *= alpha;
+#pragma unroll
+      for (int e = 0; e < EPV; ++e) acc[e] *= alpha;
+      m_run = m_new;
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const Pack<T, EPV> vp = __builtin_bit_cast(Pack<T, EPV>, vv[u]);
+        const float p = __builtin_amdgcn_exp2f(sc[u] - m_new);        // 0 for a key past the end
+        l_run += p;
+#pragma unroll
+        for (int e = 0; e < EPV; ++e) acc[e] += p * E::to_float(vp.v[e]);
+      }
+    }
+  };
+  // NS stages of registers: while one is worked on, the loads of the others are in flight
+  constexpr int STEP = G * U;
+  constexpr int NS = 2;
+  static_assert((2 * NS - 1) * STEP <= 4096, "the host check allows 4096 keys past the end");
+  uint4 kr[NS][U], vr[NS][U];
+#pragma unroll
+  for (int st = 0; st < NS - 1; ++st) load_stage(kr[st], vr[st], st * STEP);
+  for (int k0 = 0; k0 < kl; k0 += NS * STEP) {   // uniform trip count: all lanes reach the reductions
+#pragma unroll
+    for (int st = 0; st < NS; ++st) {
+      load_stage(kr[(st + NS - 1) % NS], vr[(st + NS - 1) % NS], k0 + (st + NS - 1) * STEP);
+      compute_stage(kr[st], vr[st], k0 + st * STEP);
+    }
+  }
+  if (c == 0) { s_m[g] = m_run; s_l[g] = l_run; }
+#pragma unroll
+  for (int e = 0; e < EPV; ++e) s_acc[g][c * EPV + e] = acc[e];
+  __syncthreads();
+  float m_all = -INFINITY;
+  for (int j = 0; j < G; ++j) m_all = fmaxf(m_all, s_m[j]);
+  if (tid < G) s_w[tid] = s_m[tid] > -INFINITY ? __builtin_amdgcn_exp2f(s_m[tid] - m_all) : 0.f;
+  __syncthreads();
+  for (int d = tid; d < a.D; d += NT) {
+    float l = 0.f, o = 0.f;
+#pragma unroll 4
+    for (int j = 0; j < G; ++j) {
+      l += s_l[j] * s_w[j];
+      o += s_acc[j][d] * s_w[j];
+    }
+    ctx[d] = E::from_float(l > 0.f ? o / l : 0.f);
+  }
+}
+
+template <int DT, int LPK> struct AttnLauncher {
+  static void go(const DecodeAttnArgs &a, dim3 grid, bool stream_cache, hipStream_t s) {
+    if (stream_cache) decode_attn_kernel<DT, LPK, true><<<grid, kStreamBlock, 0, s>>>(a);
+    else decode_attn_kernel<DT, LPK, false><<<grid, kBlock, 0, s>>>(a);
+  }
+};
+
+template <int DT>
+static int dispatch_attn(const DecodeAttnArgs &a, bool stream_cache, hipStream_t s) {
+  constexpr int EPV = 16 / Elem<DT>::kSize;
+  int lpk = 4;
+  while (lpk * EPV < a.D) lpk *= 2;
+  dim3 grid((unsigned)a.H, (unsigned)a.B, 1);
+  switch (lpk) {
+    case 4: AttnLauncher<DT, 4>::go(a, grid, stream_cache, s); break;
+    case 8: AttnLauncher<DT, 8>::go(a, grid, stream_cache, s); break;
+    case 16: AttnLauncher<DT, 16>::go(a, grid, stream_cache, s); break;
+    case 32: AttnLauncher<DT, 32>::go(a, grid, stream_cache, s); break;
+    case 64: AttnLauncher<DT, 64>::go(a, grid, stream_cache, s); break;
+    default: return EN_ERR_UNSUPPORTED;
+  }
+  EN_RETURN_IF_LAUNCH_FAILED();
+  return EN_OK;
+}
+
 // Appends one new K row and one new V row per (batch, head) to the caches at position
 // kv_lens[b]; sequences whose cache is full are left alone and counted.  Bytes are moved as they are.
 struct AppendArgs {
@@ -246,6 +430,35 @@ int en_kv_append(const void *k_new, const void *v_new, void *k_cache, void *v_ca
   }
   EN_RETURN_IF_LAUNCH_FAILED();
   return EN_OK;
+}
+
+int en_decode_attn(const void *q, const void *k_cache, const void *v_cache, void *ctx, const int32_t *kv_lens, int batch,
+                   int head_num, int k_seq_len, int size_per_head, const int64_t *k_strides, const int64_t *v_strides,
+                   float scale, int dtype, en_stream_t stream) {
+  using namespace en;
+  if (!k_strides || !v_strides || !v_cache) return EN_ERR_NULL;
+  int rc = check_decode(q, k_cache, ctx, kv_lens, batch, head_num, k_seq_len, size_per_head, k_strides[0], k_strides[1],
+                        k_strides[2], dtype);
+  if (rc) return rc;
+  const int es = dtype_size(dtype), epv = 16 / es;
+  if (!aligned_to(v_cache, 16) || (v_strides[0] % epv) || (v_strides[1] % epv) || (v_strides[2] % epv)) return EN_ERR_ALIGN;
+  if (!aligned_to(q, 16) || !aligned_to(ctx, es)) return EN_ERR_ALIGN;
+  if (size_per_head > 64 * epv) return EN_ERR_UNSUPPORTED;
+  // 32-bit byte offsets inside a (batch, head) unit, two stages of keys past the end included
+  if (((int64_t)k_seq_len + 4096) * k_strides[2] * es >= (1ll << 31) || ((int64_t)k_seq_len + 4096) * v_strides[2] * es >= (1ll << 31))
+    return EN_ERR_UNSUPPORTED;
+  if (!(scale > 0.f)) return EN_ERR_UNSUPPORTED;     // the running maximum is kept in units of scale * log2(e)
+  for (int i = 0; i < 3; ++i)
+    if (k_strides[i] < 0 || v_strides[i] < 0) return EN_ERR_UNSUPPORTED;
+  DecodeAttnArgs a{q, k_cache, v_cache, ctx, kv_lens, batch, head_num, k_seq_len, size_per_head, k_strides[0], k_strides[1],
+                   k_strides[2], v_strides[0], v_strides[1], v_strides[2], scale * 1.4426950408889634f};
+  const bool stream_cache = 2 * cache_bytes(batch, head_num, k_seq_len, size_per_head, dtype) >= kStreamCacheBytes;
+  hipStream_t s = (hipStream_t)stream;
+  switch (dtype) {
+    case EN_F32: return dispatch_attn<EN_F32>(a, stream_cache, s);
+    case EN_F16: return dispatch_attn<EN_F16>(a, stream_cache, s);
+    default: return dispatch_attn<EN_BF16>(a, stream_cache, s);
+  }
 }
 
 int en_decode_qk(const void *q, const void *k_cache, void *scores, const int32_t *kv_lens, int batch, int head_num,

@@ -4,7 +4,8 @@ Same names, same positional signatures; every function runs hand-written
 gfx950 kernels through the C ABI of libenergon_hip.so.  ``attn_qk`` /
 ``attn_pv`` / ``decode_qk`` / ``decode_pv`` are additions: the reference
 callers use ``torch.matmul`` for the two contractions.  ``attn_fused`` and
-``attn_fused_packed`` run the contractions and the softmax in one kernel;
+``attn_fused_packed`` run the contractions and the softmax in one kernel, ``decode_attn``
+does the same for the single-query step of cached decode;
 ``attn_qk_varlen`` / ``attn_pv_varlen`` are the two contractions on packed tokens
 (no ``transpose_pad`` / ``transpose_depad`` around them), optionally with the scores in
 the packed causal layout that ``scale_mask_softmax_packed`` works on.
@@ -14,7 +15,7 @@ from .cuda_native import (ft_build_padding_offsets, ft_remove_padding, ft_rebuil
                           ft_transpose_remove_padding, ft_transpose_rebuild_padding)
 from .cuda_native import linear, find_algo
 from .cuda_native import LayerNorm, layer_norm_forward
-from .attention import (attn_qk, attn_pv, attn_fused, attn_fused_packed, attn_fused_varlen, decode_qk, decode_pv,
+from .attention import (attn_qk, attn_pv, attn_fused, attn_fused_packed, attn_fused_varlen, decode_qk, decode_pv, decode_attn,
                         kv_cache_fill, kv_cache_append, attn_qk_varlen, attn_pv_varlen, scale_mask_softmax_packed,
                         packed_scores_elems)
 
@@ -22,6 +23,6 @@ __all__ = [
     "transpose_pad", "transpose_depad", "depad", "scale_mask_softmax", "ft_build_padding_offsets",
     "ft_remove_padding", "ft_rebuild_padding", "ft_transpose_remove_padding", "ft_transpose_rebuild_padding",
     "linear", "find_algo", "LayerNorm", "layer_norm_forward", "attn_qk", "attn_pv", "attn_fused",
-    "attn_fused_packed", "attn_fused_varlen", "decode_qk", "decode_pv", "kv_cache_fill", "kv_cache_append", "repad",
+    "attn_fused_packed", "attn_fused_varlen", "decode_qk", "decode_pv", "decode_attn", "kv_cache_fill", "kv_cache_append", "repad",
     "attn_qk_varlen", "attn_pv_varlen", "scale_mask_softmax_packed", "packed_scores_elems",
 ]

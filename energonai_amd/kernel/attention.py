@@ -351,3 +351,33 @@ def decode_pv(p, v_cache, kv_len_list, *, out: Optional[torch.Tensor] = None):
                                             B, H, Smax, D, *vs, _lib.dtype_tag(p, "decode_pv"), _lib.stream_of(p)),
                    "decode_pv")
     return out
+
+
+def decode_attn(q, k_cache, v_cache, kv_len_list, *, scale: Optional[float] = None, out: Optional[torch.Tensor] = None):
+    """ctx[b,h,0,:] = sum_j softmax_j(scale * <q[b,h,0,:], k_cache[b,h,j,:]>) v_cache[b,h,j,:] over the cached
+    positions ``j < kv_len[b]``, in one pass over the caches: what ``decode_qk`` -> ``scale_mask_softmax`` ->
+    ``decode_pv`` compute in three launches (and the reference by recomputing the whole square,
+    energonai/model/attention.py:61-71,106-118).  ``[B,H,1,D]``; ``scale`` defaults to ``size_per_head ** -0.5``."""
+    _lib.require_gpu(q, "q", contiguous=False)
+    ks = _bhsd(k_cache, "k_cache")
+    vs = _bhsd(v_cache, "v_cache")
+    B, H, Smax, D = k_cache.shape
+    if v_cache.shape != k_cache.shape or v_cache.dtype != k_cache.dtype:
+        raise RuntimeError("decode_attn: k_cache and v_cache must share shape and dtype")
+    if q.numel() != B * H * D or q.dtype != k_cache.dtype:
+        raise RuntimeError("decode_attn: q must be [B,H,1,D] of the caches' dtype")
+    q_ = q.reshape(B, H, D).contiguous()
+    info = seq_info(kv_len_list, B, q.device)
+    if out is None:
+        out = torch.empty((B, H, 1, D), dtype=q.dtype, device=q.device)
+    else:
+        _lib.require_gpu(out, "out")
+        if out.numel() != B * H * D or out.dtype != q.dtype:
+            raise RuntimeError("decode_attn: out must be a contiguous [B,H,1,D] tensor of q's dtype")
+    arr = ctypes.c_int64 * 3
+    scale = float(D) ** -0.5 if scale is None else float(scale)
+    with _lib.device_guard(q):
+        _lib.check(_lib.fn.en_decode_attn(q_.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), out.data_ptr(),
+                                          info.lens.data_ptr(), B, H, Smax, D, arr(*ks), arr(*vs), scale,
+                                          _lib.dtype_tag(q, "decode_attn"), _lib.stream_of(q)), "decode_attn")
+    return out

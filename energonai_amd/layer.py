@@ -16,7 +16,7 @@ from typing import Dict, Optional
 
 import torch
 
-from .kernel import (attn_fused, attn_fused_packed, attn_pv, attn_pv_varlen, attn_qk, attn_qk_varlen, decode_pv, decode_qk,
+from .kernel import (attn_fused, attn_fused_packed, attn_pv, attn_pv_varlen, attn_qk, attn_qk_varlen, decode_attn, decode_pv, decode_qk,
                      depad, layer_norm_forward, scale_mask_softmax, scale_mask_softmax_packed, transpose_depad,
                      transpose_pad)
 from . import _lib
@@ -232,23 +232,30 @@ def padding_removal_layer_noalloc(hidden_padded: torch.Tensor, qkv_packed: torch
 
 def decode_layer(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, kv_lens, residual: torch.Tensor,
                  gamma: torch.Tensor, beta: torch.Tensor, eps: float = 1e-5, scale: Optional[float] = None,
-                 dense_out: Optional[torch.Tensor] = None, keep: bool = False):
+                 dense_out: Optional[torch.Tensor] = None, keep: bool = False, single_pass: Optional[bool] = None):
     """One cached decode step: a single new query per sequence against a ragged
     cache, then residual + LayerNorm on the B new tokens (transpose_depad of a
     one-row sequence is the identity, so the context is passed on as a view).
 
-    q [B,H,1,D]; caches [B,H,Smax,D]; residual [1,B,hid].
+    q [B,H,1,D]; caches [B,H,Smax,D]; residual [1,B,hid].  ``single_pass`` (default: on, unless ``keep`` asks
+    for the probabilities) runs QK^T, softmax and PV as one kernel that reads K and V once and writes no scores:
+    two launches per step.  Otherwise ``decode_qk`` -> ``scale_mask_softmax`` -> ``decode_pv``, four launches.
     """
     B, H, _, D = q.shape
     Smax = k_cache.shape[2]
     hid = gamma.numel()
     info = seq_info(kv_lens, B, q.device)
     scale = float(D) ** -0.5 if scale is None else scale
-    ones = _ones_info(B, q.device)
-
-    scores = decode_qk(q, k_cache, info)
-    probs = scale_mask_softmax(B, 1, H, scores, info, scale=scale, causal=True, k_seq_len=Smax, q_len_list=ones)
-    ctx = decode_pv(probs, v_cache, info)
+    if single_pass is None:
+        single_pass = not keep and scale > 0
+    probs = None
+    if single_pass:
+        ctx = decode_attn(q, k_cache, v_cache, info, scale=scale)
+    else:
+        ones = _ones_info(B, q.device)
+        scores = decode_qk(q, k_cache, info)
+        probs = scale_mask_softmax(B, 1, H, scores, info, scale=scale, causal=True, k_seq_len=Smax, q_len_list=ones)
+        ctx = decode_pv(probs, v_cache, info)
     ctx_packed = ctx.view(1, B, H, D)      # [B,H,1,D] with one query per sequence is [1,T=B,H,D] already
     attn_out = ctx_packed.view(1, B, H * D) if dense_out is None else dense_out
     y = layer_norm_forward(attn_out, gamma, beta, (hid,), eps, residual=residual)

@@ -14,7 +14,7 @@ from typing import Optional
 import torch
 from torch import nn
 
-from ..kernel import (attn_fused_varlen, attn_pv, attn_qk, decode_pv, decode_qk, depad, repad, scale_mask_softmax,
+from ..kernel import (attn_fused_varlen, attn_pv, attn_qk, decode_attn, decode_pv, decode_qk, depad, repad, scale_mask_softmax,
                       transpose_depad)
 from ..kernel.attention import kv_cache_fill
 from ..seqinfo import SeqInfo, seq_info
@@ -111,11 +111,7 @@ class MultiHeadAttention1D(nn.Module):
         cache = self.kv_cache
         q, k, v, _ = self._project(last)
         cache.append(k, v)
-        scores = decode_qk(q, cache.k, cache.info)
-        ones = seq_info(_ones(B, last.device), B, last.device)
-        probs = scale_mask_softmax(B, 1, H, scores, cache.info, scale=self.scaling, causal=True,
-                                   k_seq_len=cache.max_seq_len, q_len_list=ones)
-        ctx = decode_pv(probs, cache.v, cache.info)          # [B,H,1,D]
+        ctx = decode_attn(q, cache.k, cache.v, cache.info, scale=self.scaling)      # [B,H,1,D], one pass over the caches
         return project(self.dense, ctx.view(B, 1, self.hidden_size))
 
     def forward(self, hidden_states, attention_mask=None, first_cache=False, seq_lens=None):

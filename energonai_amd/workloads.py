@@ -139,7 +139,8 @@ def algorithmic_bytes(w: Workload, lens_list) -> Dict[str, float]:
     if w.decode:
         kv = sum(lens_list)
         return dict(decode_qk=H * kv * D * e + H * kv * e, decode_pv=H * kv * D * e + H * kv * e,
-                    scale_mask_softmax=2 * H * kv * e, layernorm_residual=3 * B * hid * e)
+                    scale_mask_softmax=2 * H * kv * e, layernorm_residual=3 * B * hid * e,
+                    decode_attn=2 * H * kv * D * e + 2 * B * H * D * e)    # K and V once; q in, ctx out
     T = sum(lens_list)
     vis = sum(n * (n + 1) // 2 for n in lens_list) if w.causal else sum(n * n for n in lens_list)
     return dict(

@@ -243,6 +243,19 @@ int en_decode_pv(const void *p, const void *v_cache, void *ctx, const int32_t *k
                  int k_seq_len, int size_per_head, int64_t v_stride_b, int64_t v_stride_h, int64_t v_stride_s,
                  int dtype, en_stream_t stream);
 
+/* Both contractions and the softmax between them in one pass over the cache:
+ * ctx[b,h,:] = sum_j softmax_j(scale * <q[b,h,:], k_cache[b,h,j,:]>) v_cache[b,h,j,:] over j < kv_lens[b].
+ * The reference recomputes the whole square from a concatenated history on every step and keeps its last row
+ * (energonai/model/attention.py:61-71,106-118); en_decode_qk -> en_scale_mask_softmax -> en_decode_pv compute the
+ * same row in three launches with the scores passing through memory; here K and V are each read once and nothing
+ * else touches memory.  q and ctx [B,H,D] contiguous; k_strides / v_strides point to three int64 in host memory
+ * (batch, head, position strides in elements) of the [B,H,Smax,D] caches.  scale must be positive.  A sequence
+ * with kv_lens[b] == 0 gets a zero row.  fp32 statistics and accumulation; dtypes and head sizes as
+ * en_decode_qk. */
+int en_decode_attn(const void *q, const void *k_cache, const void *v_cache, void *ctx, const int32_t *kv_lens, int batch,
+                   int head_num, int k_seq_len, int size_per_head, const int64_t *k_strides, const int64_t *v_strides,
+                   float scale, int dtype, en_stream_t stream);
+
 /* Appends the new token's K and V rows to [B,H,Smax,D] caches at position
  * kv_lens[b] (the caller then adds one to kv_lens); replaces the reference's
  * torch.cat of the whole projection history on every step

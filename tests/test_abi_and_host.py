@@ -96,6 +96,10 @@ def test_entry_points_validate_before_launch():
     assert lib.en_transpose_pad_heads(16, 32, 48, 1, 1, 4, 8, 6, 4, 1, 2, None) == -2   # heads 4..7 of a 6-row source
     assert lib.en_kv_append(16, 32, 48, 64, None, 1, 1, 1, 8, 8, 8, 8, 8, 8, 2, None, None) == -1
     assert lib.en_kv_append(16, 32, 48, 64, 80, 1, 1, 1, 8, 8, 8, 8, 8, 8, 3, None, None) == -3   # element size 3
+    assert lib.en_decode_attn(16, 32, None, 64, 80, 1, 1, 8, 64, i64x3, i64x3, 1.0, 1, None) == -1    # no V cache
+    assert lib.en_decode_attn(16, 32, 48, 64, 80, 1, 1, 8, 64, i64x3, i64x3, 0.0, 1, None) == -5      # scale must be positive
+    assert lib.en_decode_attn(16, 32, 48, 64, 80, 1, 1, 8, 60, i64x3, i64x3, 1.0, 1, None) == -5      # D not a multiple of 8
+    assert lib.en_decode_attn(16, 32, 48, 64, 80, 1, 1, 2 ** 24, 64, i64x3, i64x3, 1.0, 1, None) == -5   # 32-bit offsets inside a unit
     assert lib.en_attn_fused(16, 32, 48, 64, 80, None, 1, 1, 8, 8, 64, i64x3, i64x3, i64x3, i64x3, None, None, 1.0, 1, 0,
                              None, None) == -3                           # fp32 is not a fused-attention dtype
     assert lib.en_attn_fused(16, 32, 48, 64, 80, None, 1, 1, 8, 8, 64, i64x3, i64x3, i64x3, i64x3, None, None, 0.0, 1, 1,

@@ -191,6 +191,66 @@ def test_decode_qk_pv(dtype, B, H, S, D, kv):
     assert_ctx_close(ctx, want_ctx, dtype, "decode_pv")
 
 
+DECODE_ATTN_CASES = DECODE_CASES + [
+    (9, 3, 2048, 128, [3, 1989, 2048, 1, 0, 777, 1024, 65, 64]),   # an empty cache among full and short ones
+    (2, 2, 300, 96, [300, 131]),                                     # twelve vectors per key on sixteen lanes
+    (300, 1, 40, 64, None),                                          # more sequences than are ranked by length
+    (1, 2, 5000, 64, [4999]),                                        # a single sequence (no ranking), a long cache
+]
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("B,H,S,D,kv", DECODE_ATTN_CASES)
+def test_decode_attn_single_pass(dtype, B, H, S, D, kv):
+    """QK^T, softmax and PV of the decode step in one kernel against the float64 oracle (the last row of the
+    reference's recompute), NaN in every cache row past a sequence's length."""
+    k = _kernel()
+    g = torch.Generator().manual_seed(7 * S + D + B)
+    if kv is None:
+        kv = torch.randint(0, S + 1, (B,), generator=g).tolist()
+    announce("decode attn", dtype, B, H, S, D, kv[:12])
+    q = torch.randn(B, H, 1, D, generator=g).to(dtype)
+    kc = torch.randn(B, H, S, D, generator=g).to(dtype)
+    vc = torch.randn(B, H, S, D, generator=g).to(dtype)
+    for b, n in enumerate(kv):
+        kc[b, :, n:] = float("nan")
+        vc[b, :, n:] = float("nan")
+    kv_t = torch.tensor(kv, dtype=torch.int32).cuda()
+    scale = D ** -0.5
+    _, _, want = eager.decode_attention(q, torch.nan_to_num(kc, nan=0.0), torch.nan_to_num(vc, nan=0.0), kv, scale,
+                                        acc_dtype=torch.float64)
+    for b, n in enumerate(kv):
+        if n == 0:
+            want[b] = 0          # no key to attend to: a zero row (the oracle's softmax of nothing is NaN)
+    out = torch.full((B, H, 1, D), 777.0, dtype=dtype, device="cuda")
+    got = k.decode_attn(q.cuda(), kc.cuda(), vc.cuda(), kv_t, scale=scale, out=out)
+    assert got.data_ptr() == out.data_ptr()
+    assert_ctx_close(got.cpu(), want, dtype, "decode_attn")
+    # the caches as strided views of one [B,H,S,2D] buffer, K and V interleaved per position
+    both = torch.cat([kc, vc], dim=-1).cuda()
+    got2 = k.decode_attn(q.cuda(), both[..., :D], both[..., D:], kv_t, scale=scale)
+    assert torch.equal(got2, got)
+
+
+def test_decode_attn_agrees_with_the_three_launch_route():
+    """decode_qk -> scale_mask_softmax -> decode_pv store scores and probabilities in fp16 on the way; the single
+    pass keeps them in fp32.  Both meet the bound against the oracle, so they agree within twice that bound."""
+    k = _kernel()
+    B, H, S, D = 6, 8, 1024, 128
+    kv = [1024, 5, 600, 77, 1, 333]
+    announce("decode attn vs three launches")
+    g = torch.Generator().manual_seed(4)
+    q, kc, vc = (torch.randn(B, H, n, D, generator=g).half().cuda() for n in (1, S, S))
+    kv_t = torch.tensor(kv, dtype=torch.int32).cuda()
+    one = k.decode_attn(q, kc, vc, kv_t)
+    scores = k.decode_qk(q, kc, kv_t)
+    probs = k.scale_mask_softmax(B, 1, H, scores, kv_t, scale=D ** -0.5, k_seq_len=S,
+                                 q_len_list=torch.ones(B, dtype=torch.int32).cuda())
+    three = k.decode_pv(probs, vc, kv_t)
+    assert_stored_close(one.cpu(), three.cpu().double(), torch.float16, base=2 * BASE[torch.float16],
+                        what="single pass vs three launches")
+
+
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 @pytest.mark.parametrize("causal", [True, False])
 @pytest.mark.parametrize("B,H,S,D,lens", ATTN_CASES)

@@ -264,6 +264,23 @@ def test_decode_layer_c5_reduced_and_full():
                                       inp["beta"].cpu(), 1e-5, residual=inp["residual"].cpu(),
                                       out_dtype=torch.float32)
     assert_stored_close(got2["y"].cpu(), want2, w.dtype, what="LayerNorm output")
+    # the default form of the step: one pass over the caches, then the LayerNorm.  The context against the oracle
+    # on nine sequences (the shortest, the longest, and seven spread between them) at the stated bound.
+    got3 = layer.decode_layer(inp["q"], inp["k_cache"], inp["v_cache"], inp["lens"].cuda(), inp["residual"],
+                              inp["gamma"], inp["beta"], 1e-5, w.scale, single_pass=True, keep=True)
+    by_len = sorted(range(w.batch), key=lambda b: lens_l[b])
+    assert lens_l[by_len[0]] == 3 and lens_l[by_len[-1]] == 1989
+    for b in [by_len[i * (w.batch - 1) // 8] for i in range(9)]:
+        _, _, ctx = eager.decode_attention(inp["q"][b:b + 1].cpu(), inp["k_cache"][b:b + 1].cpu(),
+                                           inp["v_cache"][b:b + 1].cpu(), [lens_l[b]], w.scale)
+        assert_stored_close(got3["ctx"][b:b + 1].cpu(), ctx, w.dtype, what=f"single-pass context, sequence {b}")
+    want3, _, _, _ = eager.layer_norm(got3["ctx_packed"].reshape(1, w.batch, -1).cpu(), inp["gamma"].cpu(),
+                                      inp["beta"].cpu(), 1e-5, residual=inp["residual"].cpu(),
+                                      out_dtype=torch.float32)
+    assert_stored_close(got3["y"].cpu(), want3, w.dtype, what="LayerNorm output")
+    y_default = layer.decode_layer(inp["q"], inp["k_cache"], inp["v_cache"], inp["lens"].cuda(), inp["residual"],
+                                   inp["gamma"], inp["beta"], 1e-5, w.scale)
+    assert torch.equal(y_default, got3["y"])
 
 
 @pytest.mark.parametrize("mode", [True, "packed"])
