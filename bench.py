@@ -588,6 +588,12 @@ def kernel_table(torch, K, layer, workloads, w, d, info, steps, step_only=False,
                 ctx_pk = torch.empty(1, T, H * D, dtype=w.dtype, device="cuda")
                 api["attn_fused_packed"] = lambda: K.attn_fused_packed(d["qkv_packed"], B, S, info, H, D,
                                                                        scale=w.scale, causal=w.causal, out=ctx_pk)
+                if D > 64:
+                    # the same op with 64 queries per wave (256-row tiles): built, measured, not what the step runs
+                    alg["attn_fused_packed_wide"] = alg["attn_fused"]
+                    api["attn_fused_packed_wide"] = lambda: K.attn_fused_packed(d["qkv_packed"], B, S, info, H, D,
+                                                                                scale=w.scale, causal=w.causal, out=ctx_pk,
+                                                                                query_tile=256)
             api["transpose_depad"] = lambda: K.transpose_depad(ctx, B, T, S, info, H, D)
             api["layernorm_residual"] = lambda: K.layer_norm_forward(attn_out, d["gamma"], d["beta"], (w.hidden,),
                                                                      workloads.EPS, residual=keep["x"])
@@ -601,8 +607,9 @@ def kernel_table(torch, K, layer, workloads, w, d, info, steps, step_only=False,
             ms = _event_time_ms(fn, steps, torch)
             row = {"us": ms * 1e3, "alg_MB": bytes_of[name] / 1e6, "GBps": bytes_of[name] / (ms * 1e-3) / 1e9}
             row["hbm_frac"] = row["GBps"] / HBM_PEAK_GBS
-            if name in ("attn_qk", "attn_pv", "decode_qk", "decode_pv", "decode_attn", "attn_fused", "attn_fused_packed"):
-                row["TFLOPs"] = (2 if name in ("attn_fused", "attn_fused_packed", "decode_attn") else 1) * flops / (ms * 1e-3) / 1e12
+            if name in ("attn_qk", "attn_pv", "decode_qk", "decode_pv", "decode_attn", "attn_fused", "attn_fused_packed",
+                        "attn_fused_packed_wide"):
+                row["TFLOPs"] = (2 if name.startswith("attn_fused") or name == "decode_attn" else 1) * flops / (ms * 1e-3) / 1e12
                 row["mfma_frac"] = row["TFLOPs"] / MFMA_PEAK_TFLOPS[dt]
             table[name] = row
         return table

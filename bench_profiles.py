@@ -44,6 +44,7 @@ KERNEL_KEYS = [
     ("decode_attn", "decode_attn"),
     ("decode_qk", "decode_qk"),
     ("decode_pv", "decode_pv"),
+    ("attn_fused_wide", "attn_fused_packed_wide"),
     ("attn_fused", "attn_fused_packed"),
     ("copy_kernel", "copy"),
 ]

@@ -46,14 +46,15 @@ SIGNATURES = {
                            c_int, c_void_p, c_void_p]),
     "en_attn_pv": (c_int, [c_void_p] * 5 + [c_int] * 5 + [c_int64] * 6 + [c_int, c_int, c_int, c_void_p, c_void_p,
                            c_int, c_void_p, c_void_p]),
-    "en_attn_tile_table_elems": (c_int64, [c_int] * 3),
-    "en_attn_tile_table": (c_int, [c_void_p, c_int, c_int, c_int, c_int, c_void_p, c_void_p]),
+    "en_attn_tile_table_elems": (c_int64, [c_int] * 4),
+    "en_attn_tile_table": (c_int, [c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p, c_void_p]),
+    "en_attn_fused_query_tile": (c_int, [c_int] * 5),
     "en_packed_scores_elems": (c_int64, [c_int] * 4),
     "en_scale_mask_softmax_packed": (c_int, [c_void_p, c_void_p, c_int, c_int, c_int, c_float, c_int, c_void_p]),
     "en_decode_qk": (c_int, [c_void_p] * 4 + [c_int] * 4 + [c_int64] * 3 + [c_float, c_int, c_void_p]),
     "en_decode_pv": (c_int, [c_void_p] * 4 + [c_int] * 4 + [c_int64] * 3 + [c_int, c_void_p]),
     "en_decode_attn": (c_int, [c_void_p] * 5 + [c_int] * 4 + [c_void_p, c_void_p, c_float, c_int, c_void_p]),
-    "en_attn_fused": (c_int, [c_void_p] * 6 + [c_int] * 5 + [c_void_p] * 6 + [c_float, c_int, c_int, c_void_p, c_void_p]),
+    "en_attn_fused": (c_int, [c_void_p] * 6 + [c_int] * 5 + [c_void_p] * 6 + [c_float, c_int, c_int, c_void_p, c_int, c_void_p]),
     "en_padding_removal_layer": (c_int, [c_void_p] * 13 + [c_int] * 4 + [c_int64, c_int64, c_float, c_float] + [c_int] * 3 + [c_void_p, c_int, c_void_p, c_void_p]),
     "en_padding_removal_layer_noalloc": (c_int, [c_void_p] * 7 + [c_int] * 5 + [c_int64, c_int64, c_float, c_float] +
                                          [c_int] * 5 + [c_void_p]),

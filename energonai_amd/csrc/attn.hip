@@ -793,7 +793,7 @@ __global__ __launch_bounds__(kBlock, 3) void attn_pv_strip_kernel(AttnArgs a) {
 // One workgroup; the sort is a rank count (batch <= 1024), larger batches keep their order.
 __global__ __launch_bounds__(1024) void attn_tile_table_kernel(const int32_t *__restrict__ lens, int batch, int heads,
                                                                int seq_len, int ntq, int32_t *__restrict__ table,
-                                                               int capacity, int tiles_first) {
+                                                               int capacity, int tiles_first, int q_tile) {
   __shared__ int32_t s_len[1024];
   __shared__ int32_t s_order[1024];
   const int tid = threadIdx.x;
@@ -817,7 +817,7 @@ __global__ __launch_bounds__(1024) void attn_tile_table_kernel(const int32_t *__
       const int b = sorted ? s_order[p] : p;
       const int n = sorted ? s_len[b] : min(max(lens[b], 0), seq_len);
       unit = b * heads + h;
-      return (n + kQTile - 1) / kQTile;
+      return (n + q_tile - 1) / q_tile;
     };
     int j = 0, unit;
     if (tiles_first) {
@@ -935,21 +935,25 @@ static int check_common(const void *x, const void *y, const void *z, const int32
 
 extern "C" {
 
-int64_t en_attn_tile_table_elems(int batch, int head_num, int q_seq_len) {
+int64_t en_attn_tile_table_elems(int batch, int head_num, int q_seq_len, int query_tile) {
   using namespace en;
-  if (batch < 1 || head_num < 1 || q_seq_len < 1) return 0;
-  return ceil_div((int64_t)batch * head_num, (int64_t)kXcds) * kXcds * ceil_div(q_seq_len, kQTile);
+  if (query_tile == 0) query_tile = kQTile;
+  if (batch < 1 || head_num < 1 || q_seq_len < 1 || (query_tile != kQTile && query_tile != 2 * kQTile)) return 0;
+  return ceil_div((int64_t)batch * head_num, (int64_t)kXcds) * kXcds * ceil_div(q_seq_len, query_tile);
 }
 
 int en_attn_tile_table(const int32_t *seq_lens, int batch, int head_num, int q_seq_len, int tiles_first,
-                       int32_t *table, en_stream_t stream) {
+                       int query_tile, int32_t *table, en_stream_t stream) {
   using namespace en;
   if (!seq_lens || !table) return EN_ERR_NULL;
+  if (query_tile == 0) query_tile = kQTile;
   if (batch < 1 || head_num < 1 || q_seq_len < 1) return EN_ERR_SHAPE;
-  const int64_t cap = en_attn_tile_table_elems(batch, head_num, q_seq_len);
+  if (query_tile != kQTile && query_tile != 2 * kQTile) return EN_ERR_UNSUPPORTED;
+  const int64_t cap = en_attn_tile_table_elems(batch, head_num, q_seq_len, query_tile);
   if (cap > INT32_MAX || (int64_t)batch * head_num > INT32_MAX / 64) return EN_ERR_SHAPE;
   attn_tile_table_kernel<<<1, 1024, 0, (hipStream_t)stream>>>(seq_lens, batch, head_num, q_seq_len,
-                                                               (int)ceil_div(q_seq_len, kQTile), table, (int)cap, tiles_first ? 1 : 0);
+                                                               (int)ceil_div(q_seq_len, query_tile), table, (int)cap,
+                                                               tiles_first ? 1 : 0, query_tile);
   EN_RETURN_IF_LAUNCH_FAILED();
   return EN_OK;
 }

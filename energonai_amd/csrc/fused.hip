@@ -38,35 +38,9 @@
 // 16 bytes per lane).  A lane that fetches or stores pieces of a row of its own
 // makes every instruction touch 32 rows, and the queue of the address unit then
 // stands full and holds back the tile loads of every wave on the CU.
-#include "attn_common.hip.h"
+#include "fused_common.hip.h"
 
 namespace en {
-
-// The lane's number in its wave, counted afresh (two VALU instructions) where a value derived from it is needed only
-// now and then, instead of keeping that value in a register through the key loop: the kernel has none to spare.
-__device__ __forceinline__ int lane_now() {
-  int l;
-  asm volatile("v_mbcnt_lo_u32_b32 %0, -1, 0\n\tv_mbcnt_hi_u32_b32 %0, -1, %0" : "=v"(l));
-  return l;
-}
-
-struct FusedArgs {
-  AttnArgs base;             // a_ptr = q, b_ptr = k, out = ctx; q_s* = q strides, k_s* = k strides
-  const void *v;
-  int64_t v_sb, v_sh, v_ss;
-  int64_t c_sb, c_sh, c_ss;
-  const int32_t *q_row0;     // packed layout: first row of batch b in q / ctx (else null)
-  const int32_t *k_row0;     // packed layout: first row of batch b in k / v (else null)
-  float scale;
-  int c_vec16;               // ctx rows may be written with 128-bit stores (16-byte aligned base and strides)
-};
-
-// Both halves of the wave get (x of lanes 0..31, x of lanes 32..63): one VALU swap, no LDS round trip.
-__device__ __forceinline__ void halves_of(float x, float &lo, float &hi) {
-  const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
-  lo = __uint_as_float(r[0]);
-  hi = __uint_as_float(r[1]);
-}
 
 template <int DT, int DP>
 __global__ __launch_bounds__(kBlock, 3) void attn_fused_kernel(FusedArgs fa) {
@@ -396,18 +370,30 @@ static int launch_fused(FusedArgs &fa, hipStream_t s) {
 
 }  // namespace en
 
+extern "C" int en_attn_fused_query_tile(int q_seq_len, int k_seq_len, int size_per_head, int causal, int dtype) {
+  // The 256-row tile (64 queries per wave, fused_wide.hip) halves the LDS reads, tile loads and barriers per FLOP
+  // but runs two waves per SIMD instead of three, and measures slower on every shape tried (uniform 1024-key
+  // rows, 64 heads: 778 against 906 TFLOP/s; ragged batches lose more, having fewer and longer workgroups):
+  // never chosen by itself.
+  (void)q_seq_len; (void)k_seq_len; (void)size_per_head; (void)causal; (void)dtype;
+  return en::kQTile;
+}
+
 extern "C" int en_attn_fused(const void *q, const void *k, const void *v, void *ctx, const int32_t *k_lens,
                              const int32_t *q_lens, int batch, int head_num, int q_seq_len, int k_seq_len,
                              int size_per_head, const int64_t *q_strides, const int64_t *k_strides,
                              const int64_t *v_strides, const int64_t *c_strides, const int32_t *q_row_offsets,
                              const int32_t *k_row_offsets, float scale, int causal, int dtype,
-                             const int32_t *tile_table, en_stream_t stream) {
+                             const int32_t *tile_table, int query_tile, en_stream_t stream) {
   using namespace en;
   if (!q || !k || !v || !ctx || !k_lens || !q_strides || !k_strides || !v_strides || !c_strides) return EN_ERR_NULL;
   if (batch < 1 || head_num < 1 || q_seq_len < 1 || k_seq_len < 1 || size_per_head < 1) return EN_ERR_SHAPE;
   if (dtype != EN_F16 && dtype != EN_BF16) return EN_ERR_DTYPE;
   if (size_per_head > 128 || (size_per_head % 8) != 0) return EN_ERR_UNSUPPORTED;
   if (!(scale > 0.f)) return EN_ERR_UNSUPPORTED;  // masked scores are -inf; -inf * 0 would not stay masked
+  if (query_tile == 0) query_tile = en_attn_fused_query_tile(q_seq_len, k_seq_len, size_per_head, causal, dtype);
+  if (query_tile != kQTile && query_tile != kWideQTile) return EN_ERR_UNSUPPORTED;
+  if (query_tile == kWideQTile && size_per_head <= 64) return EN_ERR_UNSUPPORTED;   // the 64-query wave is built for 65..128 channels
   if ((int64_t)batch * head_num > INT32_MAX / 64) return EN_ERR_SHAPE;
   if (!aligned_to(q, 16) || !aligned_to(k, 16) || !aligned_to(v, 16) || !aligned_to(ctx, 8)) return EN_ERR_ALIGN;
   for (int i = 0; i < 3; ++i) {
@@ -436,5 +422,9 @@ extern "C" int en_attn_fused(const void *q, const void *k, const void *v, void *
   a.tile_table = tile_table;
   fa.scale = scale;
   hipStream_t s = (hipStream_t)stream;
+  if (query_tile == kWideQTile) {
+    a.ntq = (int)ceil_div(q_seq_len, kWideQTile);
+    return launch_fused_wide(dtype, fa, s);
+  }
   return dtype == EN_F16 ? launch_fused<EN_F16>(fa, s) : launch_fused<EN_BF16>(fa, s);
 }

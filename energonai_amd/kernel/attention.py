@@ -42,9 +42,21 @@ def _unit_kv_bytes(k_seq_len: int, size_per_head: int, t: torch.Tensor) -> int:
     return 2 * int(k_seq_len) * int(size_per_head) * t.element_size()
 
 
-def _tile_table_ptr(k_info, q_ptr, head_num: int, q_seq_len: int, unit_kv_bytes: int):
+def _tile_table_ptr(k_info, q_ptr, head_num: int, q_seq_len: int, unit_kv_bytes: int, query_tile: int = 128):
     """Workgroup order for the batch (cached in its SeqInfo) when the query lengths are the key lengths."""
-    return None if q_ptr else k_info.tile_table(head_num, q_seq_len, unit_kv_bytes).data_ptr()
+    return None if q_ptr else k_info.tile_table(head_num, q_seq_len, unit_kv_bytes, query_tile).data_ptr()
+
+
+def fused_query_tile(q_seq_len: int, k_seq_len: int, size_per_head: int, causal: bool, t: torch.Tensor,
+                     query_tile: Optional[int] = None) -> int:
+    """Query rows per workgroup of the fused kernel: the caller's choice (128, or 256 for the form with 64
+    queries per wave, heads of 65..128 channels) or what the library picks for the shape."""
+    if query_tile:
+        if query_tile not in (128, 256) or (query_tile == 256 and size_per_head <= 64):
+            raise RuntimeError("attn_fused: query_tile must be 128, or 256 for heads of 65..128 channels")
+        return int(query_tile)
+    return int(_lib.fn.en_attn_fused_query_tile(int(q_seq_len), int(k_seq_len), int(size_per_head), int(bool(causal)),
+                                                _lib.dtype_tag(t, "attn_fused")))
 
 
 def attn_qk(q, k, seq_len_list, *, alpha: float = 1.0, causal: bool = True, q_len_list=None,
@@ -107,12 +119,12 @@ def attn_pv(p, v, seq_len_list, *, causal: bool = True, q_len_list=None, zero_pa
 
 
 def attn_fused(q, k, v, seq_len_list, *, scale: Optional[float] = None, causal: bool = True, q_len_list=None,
-               out: Optional[torch.Tensor] = None):
+               out: Optional[torch.Tensor] = None, query_tile: Optional[int] = None):
     """ctx = softmax(scale * q k^T, mask) v in one kernel; the score tensor is never materialised.
 
     Same masking rule as ``scale_mask_softmax`` (``causal``, key lengths, optional query lengths);
     ``scale`` defaults to ``size_per_head ** -0.5``.  fp16 / bf16 only.  Returns ``[B,H,Sq,D]``; rows of
-    padded queries are left uninitialised.
+    padded queries are left uninitialised.  ``query_tile``: see :func:`fused_query_tile`.
     """
     qs = _bhsd(q, "q")
     ks = _bhsd(k, "k")
@@ -133,11 +145,13 @@ def attn_fused(q, k, v, seq_len_list, *, scale: Optional[float] = None, causal: 
     cs = (out.stride(0), out.stride(1), out.stride(2))
     arr = ctypes.c_int64 * 3
     scale = float(D) ** -0.5 if scale is None else float(scale)
+    qt = fused_query_tile(Sq, Sk, D, causal, q, query_tile)
     with _lib.device_guard(q):
         _lib.check(_lib.fn.en_attn_fused(q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(),
                                          k_info.lens.data_ptr(), q_ptr, B, H, Sq, Sk, D, arr(*qs), arr(*ks), arr(*vs),
                                          arr(*cs), None, None, scale, int(bool(causal)),
-                                         _lib.dtype_tag(q, "attn_fused"), _tile_table_ptr(k_info, q_ptr, H, Sq, _unit_kv_bytes(Sk, D, q)),
+                                         _lib.dtype_tag(q, "attn_fused"),
+                                         _tile_table_ptr(k_info, q_ptr, H, Sq, _unit_kv_bytes(Sk, D, q), qt), qt,
                                          _lib.stream_of(q)), "attn_fused")
     return out
 
@@ -150,7 +164,7 @@ def _thd(t: torch.Tensor, name: str):
 
 
 def attn_fused_varlen(q, k, v, batch_size: int, max_seq_len: int, seq_len_list, *, scale: Optional[float] = None,
-                      causal: bool = True, out: Optional[torch.Tensor] = None):
+                      causal: bool = True, out: Optional[torch.Tensor] = None, query_tile: Optional[int] = None):
     """Self-attention on packed tokens: ``q``, ``k``, ``v`` are ``[T,H,D]`` views (any token and head
     strides) of the projection output, the result is the packed context ``[1,T,H,D]``.  Batch ``b``
     occupies rows ``cu_seqlens[b] .. cu_seqlens[b+1]``; no padded tensor is built.  fp16 / bf16 only.
@@ -169,13 +183,14 @@ def attn_fused_varlen(q, k, v, batch_size: int, max_seq_len: int, seq_len_list, 
     arr = ctypes.c_int64 * 3
     cu = info.cu_seqlens.data_ptr()
     scale = float(D) ** -0.5 if scale is None else float(scale)
+    qt = fused_query_tile(max_seq_len, max_seq_len, D, causal, q, query_tile)
     with _lib.device_guard(q):
         _lib.check(_lib.fn.en_attn_fused(q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(),
                                          info.lens.data_ptr(), None, batch_size, H, int(max_seq_len),
                                          int(max_seq_len), D, arr(*qs), arr(*ks), arr(*vs), arr(0, D, H * D), cu, cu,
                                          scale, int(bool(causal)), _lib.dtype_tag(q, "attn_fused_varlen"),
-                                         info.tile_table(H, int(max_seq_len), _unit_kv_bytes(max_seq_len, D, q)).data_ptr(),
-                                         _lib.stream_of(q)), "attn_fused_varlen")
+                                         info.tile_table(H, int(max_seq_len), _unit_kv_bytes(max_seq_len, D, q), qt).data_ptr(),
+                                         qt, _lib.stream_of(q)), "attn_fused_varlen")
     return out
 
 
@@ -257,7 +272,8 @@ def attn_pv_varlen(p, v, batch_size: int, max_seq_len: int, seq_len_list, *, cau
 
 
 def attn_fused_packed(qkv, batch_size: int, max_seq_len: int, seq_len_list, head_num: int, size_per_head: int, *,
-                      scale: Optional[float] = None, causal: bool = True, out: Optional[torch.Tensor] = None):
+                      scale: Optional[float] = None, causal: bool = True, out: Optional[torch.Tensor] = None,
+                      query_tile: Optional[int] = None):
     """Self-attention straight on the packed projection output: ``qkv`` is ``[1,T,H,3D]`` (or ``[T,H,3D]``,
     the layout ``transpose_pad`` is fed with in examples/bert/bert.py:100-104), the result is the packed
     context ``[1,T,H,D]`` that ``transpose_depad`` would return (bert.py:123).  fp16 / bf16 only.
@@ -267,7 +283,8 @@ def attn_fused_packed(qkv, batch_size: int, max_seq_len: int, seq_len_list, head
     if qkv.numel() % (3 * H * D) != 0:
         raise RuntimeError("attn_fused_packed: qkv must be [1,T,H,3D]")
     q, k, v = torch.chunk(qkv.view(-1, H, 3 * D), 3, dim=-1)
-    return attn_fused_varlen(q, k, v, batch_size, max_seq_len, seq_len_list, scale=scale, causal=causal, out=out)
+    return attn_fused_varlen(q, k, v, batch_size, max_seq_len, seq_len_list, scale=scale, causal=causal, out=out,
+                             query_tile=query_tile)
 
 
 def kv_cache_fill(src, cache, batch_size: int, seq_len_list, head_first: int = 0, zero_padding: bool = True):

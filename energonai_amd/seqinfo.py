@@ -33,7 +33,7 @@ class SeqInfo:
         self._total = total
         self._source = source           # keeps the caller's tensor alive while cached
         self._row_offsets = {}          # (max_seq_len, left_padded, version of lens) -> int32 [T]
-        self._tile_tables = {}          # (head_num, q_seq_len, order, version of lens) -> int32 workgroup order
+        self._tile_tables = {}          # (head_num, q_seq_len, order, version of lens, tile height) -> int32 workgroup order
         self._ready = []                # events recorded behind the kernels that produced the arrays above
         self._ordered = set()           # raw streams already ordered behind every event of _ready
 
@@ -110,22 +110,23 @@ class SeqInfo:
         return self.cu_seqlens is None or self._source is self.lens
 
 
-    def tile_table(self, head_num: int, q_seq_len: int, unit_kv_bytes: int = 1 << 30) -> torch.Tensor:
+    def tile_table(self, head_num: int, q_seq_len: int, unit_kv_bytes: int = 1 << 30, query_tile: int = 128) -> torch.Tensor:
         """Workgroup order of the attention kernels for this batch (``en_attn_tile_table``): the query tiles the
         sequences really have, longest sequence first.  ``unit_kv_bytes`` is what one (batch, head) unit's K and V
         hold at full length: up to 256 KB the last tiles of all units run first, above that a unit's tiles stay
-        together.  Computed once per batch, head count, bucket and order by one small kernel and reused by every
-        layer."""
+        together.  ``query_tile`` is the tile height of the kernel that will read the table (128; 256 for the fused
+        kernel's 64-queries-per-wave form).  Computed once per batch, head count, bucket, order and tile height by one
+        small kernel and reused by every layer."""
         version = self._lens_version()
-        key = (int(head_num), int(q_seq_len), int(unit_kv_bytes) <= TILES_FIRST_MAX_KV_BYTES, version)
+        key = (int(head_num), int(q_seq_len), int(unit_kv_bytes) <= TILES_FIRST_MAX_KV_BYTES, version, int(query_tile))
         tab = None if version is None and self._mutable() else self._tile_tables.get(key)
         self.order_current_stream()
         if tab is None:
-            n = int(_lib.fn.en_attn_tile_table_elems(self.batch_size, key[0], key[1]))
+            n = int(_lib.fn.en_attn_tile_table_elems(self.batch_size, key[0], key[1], key[4]))
             tab = torch.empty(max(n, 1), dtype=torch.int32, device=self.lens.device)
             with _lib.device_guard(self.lens):
                 _lib.check(_lib.fn.en_attn_tile_table(self.lens.data_ptr(), self.batch_size, key[0], key[1], int(key[2]),
-                                                      tab.data_ptr(), _lib.stream_of(self.lens)), "attn_tile_table")
+                                                      key[4], tab.data_ptr(), _lib.stream_of(self.lens)), "attn_tile_table")
                 self.produced_on_current_stream()
             if version is not None or not self._mutable():
                 # tables of older versions of the lengths can never be found again: drop them

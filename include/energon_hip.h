@@ -283,24 +283,29 @@ int en_kv_append(const void *k_new, const void *v_new, void *k_cache, void *v_ca
  * transpose_pad before nor transpose_depad after is needed; q_seq_len / k_seq_len
  * are then upper bounds of the lengths.  Null offsets select the padded layout.
  * scale must be positive.  Rows i >= q_lens[b] of ctx are left untouched.  fp16 / bf16, fp32 accumulation and statistics; D a multiple of 8, D <= 128.
- * tile_table as in en_attn_qk. */
+ * query_tile: query rows per workgroup.  128 = four waves of 32 queries; 256 = four waves of 64 queries (heads of
+ * 65..128 channels only): half the LDS reads, tile loads and barriers per FLOP at two waves per SIMD instead of
+ * three; 0 = what en_attn_fused_query_tile names for these arguments.  tile_table as in en_attn_qk, built for the
+ * same query_tile. */
+int en_attn_fused_query_tile(int q_seq_len, int k_seq_len, int size_per_head, int causal, int dtype);
 int en_attn_fused(const void *q, const void *k, const void *v, void *ctx, const int32_t *k_lens,
                   const int32_t *q_lens, int batch, int head_num, int q_seq_len, int k_seq_len, int size_per_head,
                   const int64_t *q_strides, const int64_t *k_strides, const int64_t *v_strides,
                   const int64_t *c_strides, const int32_t *q_row_offsets, const int32_t *k_row_offsets, float scale,
-                  int causal, int dtype, const int32_t *tile_table, en_stream_t stream);
+                  int causal, int dtype, const int32_t *tile_table, int query_tile, en_stream_t stream);
 
 /* Workgroup order for en_attn_qk, en_attn_pv and en_attn_fused on one batch of sequences (no counterpart in the
- * reference, whose callers run torch.matmul): table gets en_attn_tile_table_elems(batch, head_num, q_seq_len) int32
- * entries that list the 128-row query tiles the sequences really have (min(seq_lens[b], q_seq_len) rows each), the
+ * reference, whose callers run torch.matmul): table gets en_attn_tile_table_elems(batch, head_num, q_seq_len,
+ * query_tile) int32 entries that list the query tiles of query_tile rows (128, or 256 for en_attn_fused with that
+ * query_tile; 0 = 128) the sequences really have (min(seq_lens[b], q_seq_len) rows each), the
  * longest sequence first, so that the launch wastes no workgroup slots on tiles past a sequence's end and its long
  * workgroups start first.  tiles_first == 0 keeps the query tiles of a (batch, head) unit together (they share its
  * K and V in L2); tiles_first != 0 runs the last tiles of all units first, then the second-to-last ... (the better
  * order when a unit's K and V are small: about 256 KB or less).  Built once per batch and reused by every layer;
  * one small kernel on `stream`. */
-int64_t en_attn_tile_table_elems(int batch, int head_num, int q_seq_len);
+int64_t en_attn_tile_table_elems(int batch, int head_num, int q_seq_len, int query_tile);
 int en_attn_tile_table(const int32_t *seq_lens, int batch, int head_num, int q_seq_len, int tiles_first,
-                       int32_t *table, en_stream_t stream);
+                       int query_tile, int32_t *table, en_stream_t stream);
 
 /* ---- measurement helper ------------------------------------------------- */
 

@@ -83,9 +83,11 @@ def test_entry_points_validate_before_launch():
                           96, None) == -5                                # a tile table is built from the key lengths alone
     assert lib.en_attn_pv(16, 32, 48, 64, None, 1, 1, 8, 8, 64, 0, 0, 64, 0, 0, 64, 1, 1, 1, 80, None, 0,
                           None, None) == -5                              # a packed context has no padding rows to zero
-    assert lib.en_attn_tile_table_elems(16, 56, 1024) == 16 * 56 * 8 and lib.en_attn_tile_table_elems(3, 3, 130) == 16 * 2
-    assert lib.en_attn_tile_table(None, 1, 1, 8, 0, 16, None) == -1
-    assert lib.en_attn_tile_table(16, 0, 1, 8, 1, 32, None) == -2
+    assert lib.en_attn_tile_table_elems(16, 56, 1024, 0) == 16 * 56 * 8 and lib.en_attn_tile_table_elems(3, 3, 130, 128) == 16 * 2
+    assert lib.en_attn_tile_table_elems(16, 56, 1024, 256) == 16 * 56 * 4 and lib.en_attn_tile_table_elems(3, 3, 130, 64) == 0
+    assert lib.en_attn_tile_table(None, 1, 1, 8, 0, 0, 16, None) == -1
+    assert lib.en_attn_tile_table(16, 0, 1, 8, 1, 128, 32, None) == -2
+    assert lib.en_attn_tile_table(16, 1, 1, 8, 1, 64, 32, None) == -5            # tiles of 128 or 256 rows
     assert lib.en_packed_scores_elems(2, 3, 16, 1) == 2 * 3 * 16 * 64 and lib.en_packed_scores_elems(1, 1, 130, 1) == 64 * (64 * 3 + 2 * 3) and lib.en_packed_scores_elems(0, 3, 16, 1) == 0
     assert lib.en_scale_mask_softmax_packed(16, 32, 1, 1, 4096, 1.0, 1, None) == -5     # rows of more than 256 vectors
     assert lib.en_copy_bytes(16, 32, 24, None) == -2                     # not a multiple of 16
@@ -101,11 +103,16 @@ def test_entry_points_validate_before_launch():
     assert lib.en_decode_attn(16, 32, 48, 64, 80, 1, 1, 8, 60, i64x3, i64x3, 1.0, 1, None) == -5      # D not a multiple of 8
     assert lib.en_decode_attn(16, 32, 48, 64, 80, 1, 1, 2 ** 24, 64, i64x3, i64x3, 1.0, 1, None) == -5   # 32-bit offsets inside a unit
     assert lib.en_attn_fused(16, 32, 48, 64, 80, None, 1, 1, 8, 8, 64, i64x3, i64x3, i64x3, i64x3, None, None, 1.0, 1, 0,
-                             None, None) == -3                           # fp32 is not a fused-attention dtype
+                             None, 0, None) == -3                        # fp32 is not a fused-attention dtype
     assert lib.en_attn_fused(16, 32, 48, 64, 80, None, 1, 1, 8, 8, 64, i64x3, i64x3, i64x3, i64x3, None, None, 0.0, 1, 1,
-                             None, None) == -5                           # scale must be positive
+                             None, 0, None) == -5                        # scale must be positive
+    assert lib.en_attn_fused(16, 32, 48, 64, 80, None, 1, 1, 8, 8, 64, i64x3, i64x3, i64x3, i64x3, None, None, 1.0, 1, 1,
+                             None, 256, None) == -5                      # 64 queries per wave: heads of 65..128 channels
+    assert lib.en_attn_fused(16, 32, 48, 64, 80, None, 1, 1, 8, 8, 128, i64x3, i64x3, i64x3, i64x3, None, None, 1.0, 1, 1,
+                             None, 64, None) == -5                       # no such tile
+    assert lib.en_attn_fused_query_tile(1024, 1024, 128, 1, 1) in (128, 256)
     assert lib.en_attn_fused(16, 32, 48, 64, 80, None, 1, 1, 8, 8, 200, i64x3, i64x3, i64x3, i64x3, None, None, 1.0, 1, 1,
-                             None, None) == -5                           # head size above 128
+                             None, 0, None) == -5                        # head size above 128
     assert lib.en_padding_removal_layer(16, 32, None, 48, 64, 80, 96, 112, 128, 144, 160, 176, 192, 1, 8, 2, 8, 16, 4,
                                         1.0, 1e-5, 1, 0, 5, None, 1, None, None) == -5   # unknown attention form
     assert lib.en_padding_removal_layer(16, 32, None, 48, 64, 80, 96, 112, 128, 144, 160, 176, 192, 1, 8, 2, 8, 32, 4,
@@ -193,7 +200,7 @@ def test_public_attention_calls_pass_the_tile_table_when_there_are_no_query_leng
         def __init__(self):
             self.asked = []
 
-        def tile_table(self, head_num, q_seq_len, unit_kv_bytes):
+        def tile_table(self, head_num, q_seq_len, unit_kv_bytes, query_tile=128):
             self.asked.append((head_num, q_seq_len, unit_kv_bytes))
             return Table()
 

@@ -624,7 +624,7 @@ def test_attn_tile_table_lists_every_real_query_tile_once_longest_sequence_first
     info = build_seq_info(torch.tensor(lens, dtype=torch.int32), B)
     tab = info.tile_table(H, S, (64 << 10) if tiles_first else (1 << 20)).cpu().tolist()
     ntq = -(-S // 128)
-    assert len(tab) == _lib.fn.en_attn_tile_table_elems(B, H, S) == -(-B * H // 8) * 8 * ntq
+    assert len(tab) == _lib.fn.en_attn_tile_table_elems(B, H, S, 128) == -(-B * H // 8) * 8 * ntq
     want = {(b * H + h) * ntq + qi for b in range(B) for h in range(H) for qi in range(-(-min(lens[b], S) // 128))}
     got = [c for c in tab if c >= 0]
     assert len(got) == len(set(got)) and set(got) == want
@@ -683,7 +683,7 @@ def test_attention_kernels_give_the_same_bits_with_and_without_a_tile_table(caus
                                       S, D, *strides, *strides, int(causal), 0, 1, None, None, 0, t, stream), "pv")
         _lib.check(_lib.fn.en_attn_fused(q.data_ptr(), kk.data_ptr(), v.data_ptr(), fused.data_ptr(), info.lens.data_ptr(),
                                          None, B, H, S, S, D, arr, arr, arr, arr, None, None, D ** -0.5, int(causal), 1,
-                                         t, stream), "fused")
+                                         t, 128, stream), "fused")
         outs.append((probs.clone(), ctx, fused))
     for a, b in zip(*outs):
         assert torch.equal(a, b)
@@ -744,3 +744,69 @@ def test_tile_table_follows_lengths_that_change_in_place():
     want_c = k.attn_pv(want_p, v, lens.clone(), causal=True)
     for b, n in enumerate([400, 360]):
         assert torch.equal(ctx[b, :, :n], want_c[b, :, :n])
+
+
+WIDE_CASES = [c for c in ATTN_CASES if c[3] > 64] + [
+    (3, 2, 700, 128, [700, 257, 64]),       # three, two and one 256-row tiles; a wave whose second block is empty
+    (2, 1, 1030, 128, [1030, 511]),         # a fifth tile of six rows
+    (2, 2, 512, 96, [512, 300]),
+]
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("causal", [True, False])
+@pytest.mark.parametrize("B,H,S,D,lens", WIDE_CASES)
+def test_attn_fused_with_64_queries_per_wave(dtype, causal, B, H, S, D, lens):
+    """The 256-row tile of the fused kernel (query_tile=256) against the float64 oracle of the three steps, NaN in
+    every padding position, untouched rows checked; the packed form gives the same bits as the padded one."""
+    k = _kernel()
+    announce("attn fused, 64 queries per wave", dtype, causal, B, H, S, D, lens)
+    T = sum(lens)
+    qkv_packed = packed_randn(max(T, 1), H * 3 * D, dtype, 500 + S)[:T].reshape(T, H, 3 * D)
+    qkv = pad_bhsd(qkv_packed, lens, S, H, 3 * D)
+    for b, n in enumerate(lens):
+        qkv[b, :, n:] = float("nan")
+    q, kk, v = torch.chunk(qkv, 3, dim=-1)
+    lens_t = torch.tensor(lens, dtype=torch.int32).cuda()
+    qg, kg, vg = torch.chunk(qkv.cuda(), 3, dim=-1)
+    scale = D ** -0.5
+    sentinel = 777.0
+    out = torch.full((B, H, S, D), sentinel, dtype=dtype, device="cuda")
+    ctx = k.attn_fused(qg, kg, vg, lens_t, scale=scale, causal=causal, out=out, query_tile=256).cpu()
+    qz, kz, vz = (torch.nan_to_num(t, nan=0.0) for t in (q, kk, v))
+    scores = eager.attn_qk(qz, kz, torch.float64)
+    probs = eager.scale_mask_softmax(B, S, H, scores, lens, scale=scale, causal=causal, acc_dtype=torch.float64,
+                                     out_dtype=torch.float64)
+    rows_pad = torch.ones(B, H, S, dtype=torch.bool)
+    for b, n in enumerate(lens):
+        rows_pad[b, :, :n] = False
+        probs[b, :, n:] = 0
+    want = eager.attn_pv(probs, vz, torch.float64)
+    if (~rows_pad).any():
+        assert_ctx_close(ctx[~rows_pad], want[~rows_pad], dtype, "attn_fused, query_tile 256")
+    assert bool((ctx[rows_pad] == sentinel).all())
+    if T:
+        guard = torch.full((T + 2, H * D), sentinel, dtype=dtype, device="cuda")
+        k.attn_fused_packed(qkv_packed.reshape(1, T, H, 3 * D).cuda(), B, S, lens_t, H, D, scale=scale, causal=causal,
+                            out=guard[1:T + 1], query_tile=256)
+        g = guard.cpu()
+        t = 0
+        for b, n in enumerate(lens):
+            assert torch.equal(g[1 + t:1 + t + n].view(n, H, D).permute(1, 0, 2), ctx[b, :, :n])
+            t += n
+        assert bool((g[0] == sentinel).all()) and bool((g[T + 1] == sentinel).all())
+
+
+def test_tile_table_of_256_row_tiles():
+    """The workgroup order for the 64-queries-per-wave kernel lists every real 256-row tile once."""
+    from energonai_amd.seqinfo import build_seq_info
+    B, H, S = 7, 3, 1000
+    lens = [1000, 1, 256, 257, 0, 513, 777]
+    announce("tile table, 256-row tiles")
+    info = build_seq_info(torch.tensor(lens, dtype=torch.int32), B)
+    tab = info.tile_table(H, S, query_tile=256).cpu().tolist()
+    ntq = 4
+    want = {(b * H + h) * ntq + qi for b in range(B) for h in range(H) for qi in range(-(-lens[b] // 256))}
+    got = [c for c in tab if c >= 0]
+    assert len(got) == len(set(got)) and set(got) == want
+    assert len(tab) == -(-B * H // 8) * 8 * ntq
