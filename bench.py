@@ -598,7 +598,10 @@ def kernel_table(torch, K, layer, workloads, w, d, info, steps, step_only=False,
             api["layernorm_residual"] = lambda: K.layer_norm_forward(attn_out, d["gamma"], d["beta"], (w.hidden,),
                                                                      workloads.EPS, residual=keep["x"])
 
-    def measure(fns, bytes_of):
+    yard = {} if step_only else workload_yardsticks(torch, w, d, info,
+                                                    (not w.decode) and layer.three_kernel_form(w.causal, w.dtype, S) == "varlen_packed")
+
+    def measure(fns, bytes_of, layout="padded"):
         table = {}
         for name, fn in fns.items():
             for _ in range(3):
@@ -611,11 +614,20 @@ def kernel_table(torch, K, layer, workloads, w, d, info, steps, step_only=False,
                         "attn_fused_packed_wide"):
                 row["TFLOPs"] = (2 if name.startswith("attn_fused") or name == "decode_attn" else 1) * flops / (ms * 1e-3) / 1e12
                 row["mfma_frac"] = row["TFLOPs"] / MFMA_PEAK_TFLOPS[dt]
+            # what a kernel that only moves the bytes reaches in this kernel's access pattern, and this kernel's share of it
+            key = YARDSTICK_OF.get(name)
+            if key is not None and key.startswith("prefix_"):
+                key = f"{key}_{layout}"
+            if key in yard:
+                row["yardstick_GBps"] = yard[key]
+                row["yardstick_pattern"] = key
+                row["frac_of_yardstick"] = row["GBps"] / yard[key]
             table[name] = row
         return table
-    step_table = measure(step, alg if w.decode else step_alg)
-    three_table = measure(three, alg if w.decode else step_alg)
-    api_table = measure(api, alg)
+    step_layout = "packed" if ("prefix_read_packed" in yard) else "padded"
+    step_table = measure(step, alg if w.decode else step_alg, step_layout)
+    three_table = measure(three, alg if w.decode else step_alg, step_layout)
+    api_table = measure(api, alg, "padded")
     return step_table, three_table, api_table
 
 
@@ -694,7 +706,8 @@ def cpu_baseline(torch, w, full_batch, passes=3):
 
 
 def copy_yardstick(torch, iters):
-    """en_copy_bytes at 64 MiB, 256 MiB and 1 GiB (read n + write n bytes per launch)."""
+    """en_copy_bytes at 64 MiB, 256 MiB and 1 GiB (read n + write n bytes per launch); with it the stream and
+    causal-prefix yardsticks (see stream_yardsticks)."""
     from energonai_amd import _lib
     out = {"kernel": "copy_kernel", "unit": "GB/s", "sizes": {}}
     stream = torch.cuda.current_stream().cuda_stream
@@ -711,6 +724,108 @@ def copy_yardstick(torch, iters):
         out["sizes"][f"{mib}MiB"] = {"bytes_read": n, "bytes_written": n, "us": ms * 1e3, "GBps": 2 * n / (ms * 1e-3) / 1e9}
         del a, b
     return out
+
+
+STREAM_MODES = {"copy": 0, "read": 1, "write": 2, "inplace": 0}
+PREFIX_MODES = {"inplace": 0, "write": 1, "read": 2, "out_of_place": 3}
+
+
+def _preheat(torch, fn):
+    t0 = time.perf_counter()
+    while time.perf_counter() - t0 < PREHEAT_S:
+        for _ in range(5):
+            fn()
+        torch.cuda.synchronize()
+
+
+def stream_yardstick_GBps(torch, nbytes, mode, nt, iters=10):
+    """en_stream_yardstick over one contiguous range: bytes moved per second (a copy moves 2 x nbytes)."""
+    from energonai_amd import _lib
+    nbytes = max(16, (int(nbytes) // 16) * 16)
+    a = torch.empty(nbytes, dtype=torch.uint8, device="cuda")
+    b = torch.empty(nbytes if mode in ("copy", "write") else 16, dtype=torch.uint8, device="cuda")
+    a.fill_(1)
+    stream = torch.cuda.current_stream().cuda_stream
+    dst = a if mode == "inplace" else b
+    fn = lambda: _lib.check(_lib.fn.en_stream_yardstick(a.data_ptr(), dst.data_ptr(), nbytes, STREAM_MODES[mode], int(nt),
+                                                        stream), "stream_yardstick")
+    _preheat(torch, fn)
+    ms = _event_time_ms(fn, iters, torch)
+    return (2 if mode in ("copy", "inplace") else 1) * nbytes / (ms * 1e-3) / 1e9
+
+
+def prefix_yardstick_GBps(torch, lens_dev, lens_list, B, H, S, dtype, packed, mode, nt, iters=10):
+    """en_prefix_yardstick over the causal prefixes of a batch's score tensor: bytes of the visible prefixes
+    (H x element size x sum n(n+1)/2, once per direction moved) per second."""
+    from energonai_amd import _lib
+    from energonai_amd.kernel.attention import packed_scores_elems
+    es = torch.empty(0, dtype=dtype).element_size()
+    n = packed_scores_elems(B, H, S, dtype) if packed else B * H * S * S
+    a = torch.zeros(n, dtype=dtype, device="cuda")
+    b = torch.zeros(n, dtype=dtype, device="cuda") if mode == "out_of_place" else None
+    vis = H * es * sum(m * (m + 1) // 2 for m in lens_list)
+    stream = torch.cuda.current_stream().cuda_stream
+    fn = lambda: _lib.check(_lib.fn.en_prefix_yardstick(a.data_ptr(), _lib.ptr(b), lens_dev.data_ptr(), B, H, S, int(packed),
+                                                        PREFIX_MODES[mode], int(nt), es, stream), "prefix_yardstick")
+    _preheat(torch, fn)
+    ms = _event_time_ms(fn, iters, torch)
+    return (2 if mode in ("inplace", "out_of_place") else 1) * vis / (ms * 1e-3) / 1e9
+
+
+def stream_yardsticks(torch, iters):
+    """Every yardstick at the sizes and sequence lengths of the two large prefill workloads and of the decode
+    workload: what a kernel that does nothing but move the bytes reaches in each access pattern."""
+    from energonai_amd import workloads
+    out = {"unit": "GB/s", "stream": {}, "prefix": {}}
+    for mib in (128, 512, 2048):
+        row = {}
+        for mode in STREAM_MODES:
+            for nt in (0, 1):
+                row[f"{mode}{'_nt' if nt else ''}"] = stream_yardstick_GBps(torch, mib << 20, mode, nt, iters)
+        out["stream"][f"{mib}MiB"] = row
+    for name in ("c3", "c4"):
+        w = workloads.BY_NAME[name]
+        lens = workloads.make_lens(w)
+        ll = [int(v) for v in lens]
+        lens_dev = lens.to("cuda")
+        for packed in (0, 1):
+            row = {}
+            for mode in PREFIX_MODES:
+                for nt in (0, 1):
+                    row[f"{mode}{'_nt' if nt else ''}"] = prefix_yardstick_GBps(torch, lens_dev, ll, w.batch, w.heads, w.seq,
+                                                                                w.dtype, packed, mode, nt, iters)
+            out["prefix"][f"{name}_{'packed' if packed else 'padded'}"] = row
+    return out
+
+
+# which yardstick speaks for which kernel row of the tables (prefix patterns: causal prefill workloads only)
+YARDSTICK_OF = {"depad": "copy", "transpose_pad": "copy", "transpose_pad_valid_rows": "copy", "transpose_depad": "copy",
+                "layernorm_residual": "copy", "scale_mask_softmax": "prefix_inplace",
+                "scale_mask_softmax_no_tail": "prefix_inplace", "attn_qk": "prefix_write", "attn_pv": "prefix_read",
+                "decode_qk": "read", "decode_pv": "read", "decode_attn": "read"}
+
+
+def workload_yardsticks(torch, w, d, info, packed_scores):
+    """The yardsticks of one workload, best of plain and non-temporal accesses: {"copy", "read",
+    "prefix_*_packed", "prefix_*_padded"} -> GB/s."""
+    es = torch.empty(0, dtype=w.dtype).element_size()
+    y = {}
+    if w.decode:
+        nbytes = w.heads * sum(d["lens_list"]) * w.head_dim * es
+        y["read"] = max(stream_yardstick_GBps(torch, nbytes, "read", nt) for nt in (0, 1))
+        y["copy"] = max(stream_yardstick_GBps(torch, 64 << 20, "copy", nt) for nt in (0, 1))
+        return y
+    nbytes = max(d["total"] * w.hidden * es, 1 << 20)
+    y["copy"] = max(stream_yardstick_GBps(torch, nbytes, "copy", nt) for nt in (0, 1))
+    if w.causal:
+        for layout, packed in (("padded", 0), ("packed", 1)):
+            if packed and not packed_scores:
+                continue
+            for mode in ("inplace", "write", "read"):
+                y[f"prefix_{mode}_{layout}"] = max(
+                    prefix_yardstick_GBps(torch, info.lens, d["lens_list"], w.batch, w.heads, w.seq, w.dtype, packed, mode, nt)
+                    for nt in (0, 1))
+    return y
 
 
 def roofline_of(res, workload_name, form="default"):
@@ -762,8 +877,11 @@ def main(argv=None) -> int:
     ap.add_argument("--step-only", action="store_true",
                     help="with --no-extra: launch nothing but the step and its own kernels (for profiles)")
     ap.add_argument("--copy-yardstick", action="store_true",
-                    help="instead of the benchmark, time en_copy_bytes (plain 128-bit copy) at known sizes; "
-                         "used as the bandwidth yardstick and to calibrate the FETCH_SIZE / WRITE_SIZE counters")
+                    help="instead of the benchmark, time en_copy_bytes (plain 128-bit copy) at known sizes (used to "
+                         "calibrate the FETCH_SIZE / WRITE_SIZE counters) and the stream and causal-prefix yardsticks: "
+                         "copy / read only / write only with plain and non-temporal accesses, and in-place, write-only, "
+                         "read-only and out-of-place passes over the causal prefixes of the c3 and c4 score tensors in "
+                         "the [B,H,S,S] and the packed layout")
     ns = ap.parse_args(argv)
     if ns.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this build measures one GPU's share of the path; --gpus must be 1 "
@@ -781,7 +899,11 @@ def main(argv=None) -> int:
     from energonai_amd import workloads
 
     if ns.copy_yardstick:
-        print(json.dumps(copy_yardstick(torch, ns.steps)))
+        out = copy_yardstick(torch, ns.steps)
+        if not ns.step_only:      # --step-only: the plain copy alone (the counter calibration run of bench_profiles.py)
+            out["yardsticks"] = stream_yardsticks(torch, max(5, ns.steps))
+        out["library_source_hash"] = library_source_hash()
+        print(json.dumps(out))
         return 0
 
     w = workloads.BY_NAME[ns.workload]

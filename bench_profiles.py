@@ -6,6 +6,7 @@
     python3 bench_profiles.py counters --workload c3     # one --pmc run of SQ counters: MFMA and VALU busy, LDS, waits
     python3 bench_profiles.py issue --workload c3        # one --pmc run: matrix / vector co-execution, address unit queues
     python3 bench_profiles.py memsys --workload c3       # three --pmc runs: L2 hit rate, requests to memory, stalled channels
+    python3 bench_profiles.py yardstick                  # no profiler: `bench.py --copy-yardstick` as a table
 
 Each sub-command starts rocprofv3 as a child process with `python3 bench.py ...` after `--`, reads the CSV files it
 leaves in a scratch directory (--raw-dir, default: a fresh temporary one), and prints a markdown summary (redirect it
@@ -153,7 +154,7 @@ def cmd_traffic(ns) -> int:
         d, line, shown = run_profiler(f"pmc_{counter}_{ns.workload}_{ns.form}", ["--pmc", counter], bench_args, ns.timeout)
         shown_cmds.append(shown)
         per_counter[counter] = counter_rows(find_csv(d, "counter_collection.csv"), counter)
-        d, cline, shown = run_profiler(f"pmc_{counter}_copy", ["--pmc", counter], ["--copy-yardstick", "--steps", "5"],
+        d, cline, shown = run_profiler(f"pmc_{counter}_copy", ["--pmc", counter], ["--copy-yardstick", "--step-only", "--steps", "5"],
                                        ns.timeout)
         shown_cmds.append(shown)
         rows = counter_rows(find_csv(d, "counter_collection.csv"), counter)
@@ -349,9 +350,51 @@ def cmd_memsys(ns) -> int:
     return 0
 
 
+def cmd_yardstick(ns) -> int:
+    """bench.py --copy-yardstick (no profiler: event timings) as a table: what a kernel that only moves the bytes
+    reaches in each access pattern of the library's memory-bound kernels."""
+    cmd = ["python3", os.path.join(ROOT, "bench.py"), "--copy-yardstick", "--steps", str(ns.steps)]
+    proc = subprocess.run(cmd, cwd=ROOT, stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True, timeout=ns.timeout)
+    if proc.returncode != 0:
+        sys.stderr.write(proc.stderr[-3000:])
+        raise SystemExit(f"bench.py exited with {proc.returncode}")
+    line = [json.loads(ln) for ln in proc.stdout.splitlines() if ln.startswith("{")][-1]
+    y = line["yardsticks"]
+    print("# Bandwidth yardsticks: kernels that only move bytes, in the access patterns of the memory-bound kernels\n")
+    print("Command (MI355X box, repo root; the summary below is this command's stdout; HIP-event timings, no profiler):\n")
+    print(f"```\npython3 bench_profiles.py yardstick\n  -> python3 bench.py --copy-yardstick --steps {ns.steps}\n```\n")
+    print_sources(line)
+    print("All figures are GB/s of the bytes the pattern moves (a copy and an in-place or out-of-place pass move every "
+          "byte twice: once in, once out); `_nt` = non-temporal loads and stores.  Kernels: "
+          "`energonai_amd/csrc/yardstick.hip` (`en_stream_yardstick`, `en_prefix_yardstick`) and `copy_kernel` "
+          "(`en_copy_bytes`).\n")
+    print("## One contiguous range (depad, the transposes, LayerNorm, the decode kernels' cache reads)\n")
+    cols = ["copy", "copy_nt", "inplace", "inplace_nt", "read", "read_nt", "write", "write_nt"]
+    print("| size | " + " | ".join(cols) + " | `en_copy_bytes` |\n|---|" + "---|" * (len(cols) + 1))
+    plain = {k: v["GBps"] for k, v in line["sizes"].items()}
+    for size, row in y["stream"].items():
+        print(f"| {size} | " + " | ".join(f"{row[c]:.0f}" for c in cols) + f" | {plain.get(size, float('nan')):.0f} |")
+    print("\n`en_copy_bytes` (the counter-calibration copy) at its own sizes: " +
+          ", ".join(f"{k} {v:.0f}" for k, v in plain.items()) + " GB/s.\n")
+    print("## Causal prefixes of a score tensor (row q of a unit: q + 1 fp16 scores; rows below the sequence length only)\n")
+    print("`inplace`: read and written back (scale_mask_softmax without a tail); `write`: written only (QK^T); `read`: read "
+          "only (PV); `out_of_place`: read from one tensor, written to another.  `padded` = `[B,H,S,S]`, `packed` = the "
+          "packed causal layout.  c3: 16 sequences of 142..1014 tokens, 56 heads; c4: 16 of 360..2019, 12 heads.\n")
+    cols = [f"{m}{t}" for m in ("inplace", "write", "read", "out_of_place") for t in ("", "_nt")]
+    print("| lengths, layout | " + " | ".join(cols) + " |\n|---|" + "---|" * len(cols))
+    for name, row in y["prefix"].items():
+        print(f"| {name.replace('_', ', ')} | " + " | ".join(f"{row[c]:.0f}" for c in cols) + " |")
+    return 0
+
+
 def main(argv=None) -> int:
     ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
     sub = ap.add_subparsers(dest="cmd", required=True)
+    p = sub.add_parser("yardstick")
+    p.add_argument("--steps", type=int, default=10)
+    p.add_argument("--timeout", type=int, default=300)
+    p.add_argument("--raw-dir", default=None)
+    p.set_defaults(fn=cmd_yardstick)
     for name, fn in (("trace", cmd_trace), ("traffic", cmd_traffic), ("counters", cmd_counters), ("issue", cmd_issue),
                      ("memsys", cmd_memsys)):
         p = sub.add_parser(name)

@@ -59,6 +59,8 @@ SIGNATURES = {
     "en_padding_removal_layer_noalloc": (c_int, [c_void_p] * 7 + [c_int] * 5 + [c_int64, c_int64, c_float, c_float] +
                                          [c_int] * 5 + [c_void_p]),
     "en_copy_bytes": (c_int, [c_void_p, c_void_p, c_int64, c_void_p]),
+    "en_stream_yardstick": (c_int, [c_void_p, c_void_p, c_int64, c_int, c_int, c_void_p]),
+    "en_prefix_yardstick": (c_int, [c_void_p, c_void_p, c_void_p] + [c_int] * 7 + [c_void_p]),
 }
 
 LINEAR_LIB_NAME = "libenergon_linear.so"

@@ -366,6 +366,18 @@ int en_padding_removal_layer_noalloc(const void *hidden_padded, const void *qkv_
  * bandwidth yardstick and to calibrate hardware byte counters. */
 int en_copy_bytes(const void *src, void *dst, int64_t nbytes, en_stream_t stream);
 
+/* Bandwidth yardsticks (measurement helpers like en_copy_bytes; no counterpart in the reference; no op of the
+ * library calls them).  en_stream_yardstick moves one contiguous range of nbytes (multiple of 16): mode 0 copies
+ * src to dst (dst == src: a pass in place), 1 only reads src (dst: any valid 16-byte aligned address, not written), 2 only writes dst;
+ * nontemporal != 0 uses non-temporal loads and stores.  en_prefix_yardstick walks the causal prefixes of a score
+ * tensor -- row q of (batch, head) unit u holds q + 1 elements, rows q < seq_lens[b] only -- in the [B,H,S,S]
+ * layout or (packed != 0) the packed layout of en_packed_scores_elems: mode 0 reads every prefix and writes it
+ * back in place (the pattern of en_scale_mask_softmax with tail_rows 1), 1 only writes (en_attn_qk), 2 only
+ * reads (en_attn_pv), 3 reads scores and writes scores_out.  Whole 16-byte vectors are moved. */
+int en_stream_yardstick(const void *src, void *dst, int64_t nbytes, int mode, int nontemporal, en_stream_t stream);
+int en_prefix_yardstick(void *scores, void *scores_out, const int32_t *seq_lens, int batch, int head_num, int seq_len,
+                        int packed, int mode, int nontemporal, int elem_size, en_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -215,3 +215,55 @@ def test_cached_offsets_used_on_another_stream():
     left = torch.cat([x[b, S - n:] for b, n in enumerate(lens)])
     assert max_abs(y.cpu()[0], torch.nn.functional.layer_norm(left, (hid,))) <= 1e-5
     assert off.data_ptr() == info.row_offsets(S, True).data_ptr()
+
+
+def test_yardstick_kernels_touch_exactly_their_pattern():
+    """The bandwidth yardsticks are measuring sticks, but a stick that moved other bytes than it claims would
+    mislead: the copy copies, the write-only pass writes its whole range, the prefix passes write the causal
+    prefixes of the valid rows (whole 16-byte vectors) and nothing else."""
+    import torch
+    from energonai_amd import _lib
+    from energonai_amd.kernel.attention import packed_scores_elems
+    lib = _lib.load()
+    stream = torch.cuda.current_stream().cuda_stream
+    n = 1 << 20
+    a = torch.randint(0, 255, (n,), dtype=torch.uint8, device="cuda")
+    for nt in (0, 1):
+        b = torch.zeros(n, dtype=torch.uint8, device="cuda")
+        _lib.check(lib.en_stream_yardstick(a.data_ptr(), b.data_ptr(), n, 0, nt, stream), "copy")
+        assert torch.equal(a, b)
+        b.fill_(7)
+        _lib.check(lib.en_stream_yardstick(None, b.data_ptr(), n, 2, nt, stream), "write")
+        assert bool((b == 0).all())
+        b.fill_(7)
+        _lib.check(lib.en_stream_yardstick(a.data_ptr(), b.data_ptr(), n, 1, nt, stream), "read")
+        assert bool((b == 7).all())
+    B, H, S = 3, 2, 200
+    lens = [200, 0, 77]
+    lens_t = torch.tensor(lens, dtype=torch.int32, device="cuda")
+    for packed in (0, 1):
+        numel = packed_scores_elems(B, H, S, torch.float16) if packed else B * H * S * S
+        src = torch.randn(numel, device="cuda").half()
+        for mode in (0, 1, 2, 3):
+            buf = src.clone()
+            out = torch.full_like(src, 5.0)
+            _lib.check(lib.en_prefix_yardstick(buf.data_ptr(), out.data_ptr(), lens_t.data_ptr(), B, H, S, packed, mode, 0, 2,
+                                               stream), "prefix")
+            touched = torch.zeros(numel, dtype=torch.bool)
+            for b in range(B):
+                for h in range(H):
+                    unit = b * H + h
+                    if packed:       # a unit's valid rows are one contiguous range: rows back to back, 128-byte groups
+                        t = lens[b] // 64
+                        end = 64 * (64 * t * (t + 1) // 2 + (lens[b] - 64 * t) * (t + 1))
+                        touched[unit * (numel // (B * H)):unit * (numel // (B * H)) + end] = True
+                        continue
+                    for q in range(lens[b]):
+                        start = (unit * S + q) * S
+                        touched[start:start + -(-(q + 1) // 8) * 8] = True
+            if mode in (0, 2):
+                assert torch.equal(buf, src)
+            if mode == 1:
+                assert bool((buf.cpu()[touched] == 0).all()) and torch.equal(buf.cpu()[~touched], src.cpu()[~touched])
+            if mode == 3:
+                assert torch.equal(out.cpu()[touched], src.cpu()[touched]) and bool((out.cpu()[~touched] == 5.0).all())
