@@ -375,8 +375,8 @@ extern "C" int en_attn_fused_query_tile(int q_seq_len, int k_seq_len, int size_p
   // but runs two waves per SIMD instead of three, and measures slower on every shape tried (uniform 1024-key
   // rows, 64 heads: 778 against 906 TFLOP/s; ragged batches lose more, having fewer and longer workgroups):
   // never chosen by itself.
-  (void)q_seq_len; (void)k_seq_len; (void)size_per_head; (void)causal; (void)dtype;
-  return en::kQTile;
+  (void)q_seq_len; (void)k_seq_len; (void)size_per_head; (void)causal;
+  return dtype == EN_F32 ? 64 : en::kQTile;     // fp32: the kernel of fused_f32.hip, 64-row tiles
 }
 
 extern "C" int en_attn_fused(const void *q, const void *k, const void *v, void *ctx, const int32_t *k_lens,
@@ -388,22 +388,26 @@ extern "C" int en_attn_fused(const void *q, const void *k, const void *v, void *
   using namespace en;
   if (!q || !k || !v || !ctx || !k_lens || !q_strides || !k_strides || !v_strides || !c_strides) return EN_ERR_NULL;
   if (batch < 1 || head_num < 1 || q_seq_len < 1 || k_seq_len < 1 || size_per_head < 1) return EN_ERR_SHAPE;
-  if (dtype != EN_F16 && dtype != EN_BF16) return EN_ERR_DTYPE;
-  if (size_per_head > 128 || (size_per_head % 8) != 0) return EN_ERR_UNSUPPORTED;
+  if (dtype != EN_F16 && dtype != EN_BF16 && dtype != EN_F32) return EN_ERR_DTYPE;
+  const bool f32 = dtype == EN_F32;
+  const int es = f32 ? 4 : 2, epv = 16 / es;
+  if (size_per_head > 128 || (size_per_head % epv) != 0) return EN_ERR_UNSUPPORTED;
+  if (f32 && size_per_head > 64) return EN_ERR_UNSUPPORTED;   // the fp32 kernel is built for heads of up to 64 channels
   if (!(scale > 0.f)) return EN_ERR_UNSUPPORTED;  // masked scores are -inf; -inf * 0 would not stay masked
   if (query_tile == 0) query_tile = en_attn_fused_query_tile(q_seq_len, k_seq_len, size_per_head, causal, dtype);
-  if (query_tile != kQTile && query_tile != kWideQTile) return EN_ERR_UNSUPPORTED;
+  if (f32 ? query_tile != 64 : (query_tile != kQTile && query_tile != kWideQTile)) return EN_ERR_UNSUPPORTED;
   if (query_tile == kWideQTile && size_per_head <= 64) return EN_ERR_UNSUPPORTED;   // the 64-query wave is built for 65..128 channels
   if ((int64_t)batch * head_num > INT32_MAX / 64) return EN_ERR_SHAPE;
-  if (!aligned_to(q, 16) || !aligned_to(k, 16) || !aligned_to(v, 16) || !aligned_to(ctx, 8)) return EN_ERR_ALIGN;
+  if (!aligned_to(q, 16) || !aligned_to(k, 16) || !aligned_to(v, 16) || !aligned_to(ctx, 4 * es)) return EN_ERR_ALIGN;
   for (int i = 0; i < 3; ++i) {
-    if ((q_strides[i] % 8) || (k_strides[i] % 8) || (v_strides[i] % 8) || (c_strides[i] % 4)) return EN_ERR_ALIGN;
+    if ((q_strides[i] % epv) || (k_strides[i] % epv) || (v_strides[i] % epv) || (c_strides[i] % 4)) return EN_ERR_ALIGN;
     if (q_strides[i] < 0 || k_strides[i] < 0 || v_strides[i] < 0 || c_strides[i] < 0) return EN_ERR_UNSUPPORTED;
   }
   // 32-bit byte offsets, advanced a tile at a time up to two tiles past the end
-  if ((int64_t)q_seq_len * q_strides[2] * 2 >= (1ll << 31) || ((int64_t)k_seq_len + 256) * k_strides[2] * 2 >= (1ll << 31) ||
-      ((int64_t)k_seq_len + 256) * v_strides[2] * 2 >= (1ll << 31))
+  if ((int64_t)q_seq_len * q_strides[2] * es >= (1ll << 31) || ((int64_t)k_seq_len + 256) * k_strides[2] * es >= (1ll << 31) ||
+      ((int64_t)k_seq_len + 256) * v_strides[2] * es >= (1ll << 31))
     return EN_ERR_UNSUPPORTED;
+  if (f32 && tile_table) return EN_ERR_UNSUPPORTED;            // the table lists 128- or 256-row tiles; the fp32 kernel has 64-row ones
   FusedArgs fa{};
   AttnArgs &a = fa.base;
   a.a_ptr = q; a.b_ptr = k; a.out = ctx; a.k_lens = k_lens; a.q_lens = q_lens;
@@ -417,11 +421,12 @@ extern "C" int en_attn_fused(const void *q, const void *k, const void *v, void *
   fa.v_sb = v_strides[0]; fa.v_sh = v_strides[1]; fa.v_ss = v_strides[2];
   fa.c_sb = c_strides[0]; fa.c_sh = c_strides[1]; fa.c_ss = c_strides[2];
   fa.q_row0 = q_row_offsets; fa.k_row0 = k_row_offsets;
-  fa.c_vec16 = aligned_to(ctx, 16) && (c_strides[0] % 8) == 0 && (c_strides[1] % 8) == 0 && (c_strides[2] % 8) == 0;
+  fa.c_vec16 = aligned_to(ctx, 16) && (c_strides[0] % epv) == 0 && (c_strides[1] % epv) == 0 && (c_strides[2] % epv) == 0;
   if (tile_table && q_lens) return EN_ERR_UNSUPPORTED;      // the table lists the query tiles of min(k_lens, q_seq_len) rows
   a.tile_table = tile_table;
   fa.scale = scale;
   hipStream_t s = (hipStream_t)stream;
+  if (f32) return launch_fused_f32(fa, s);
   if (query_tile == kWideQTile) {
     a.ntq = (int)ceil_div(q_seq_len, kWideQTile);
     return launch_fused_wide(dtype, fa, s);

@@ -34,5 +34,7 @@ __device__ __forceinline__ void halves_of(float x, float &lo, float &hi) {
 // fused_wide.hip: the kernel whose waves own 64 queries each (256-query workgroups), for heads of 65..128 channels.
 constexpr int kWideQTile = 256;
 int launch_fused_wide(int dtype, FusedArgs &fa, hipStream_t s);
+// fused_f32.hip: fp32 storage, heads of up to 64 channels, 64-row query tiles.
+int launch_fused_f32(FusedArgs &fa, hipStream_t s);
 
 }  // namespace en

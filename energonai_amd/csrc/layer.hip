@@ -105,7 +105,7 @@ extern "C" int en_padding_removal_layer(const void *hidden_padded, const void *q
     const int64_t out_strides[3] = {0, D, (int64_t)H * D};
     rc = en_attn_fused(pk, pk + (int64_t)D * es, pk + (int64_t)2 * D * es, ctx_packed, seq_lens, nullptr, B, H, S, S, D,
                        in_strides, in_strides, in_strides, out_strides, cu_seqlens, cu_seqlens, scale, causal, dtype,
-                       tile_table, 0, stream);
+                       dtype == EN_F32 ? nullptr : tile_table, 0, stream);      // the fp32 kernel's tiles are not the table's
     if (rc) return rc;
   } else if (attention_form >= 3) {
     // The three kernels on the packed projections: q, k, v are read where the projection left them (batch b at
@@ -140,7 +140,8 @@ extern "C" int en_padding_removal_layer(const void *hidden_padded, const void *q
       const int64_t in_strides[3] = {sb, sh, ss};
       const int64_t out_strides[3] = {cb, ch, cs};
       rc = en_attn_fused(q, k, v, ctx, seq_lens, nullptr, B, H, S, S, D, in_strides, in_strides, in_strides,
-                         out_strides, nullptr, nullptr, scale, causal, dtype, tile_table, 0, stream);
+                         out_strides, nullptr, nullptr, scale, causal, dtype, dtype == EN_F32 ? nullptr : tile_table, 0,
+                         stream);
       if (rc) return rc;
     } else {
       rc = en_attn_qk(q, k, scores, seq_lens, nullptr, B, H, S, S, D, sb, sh, ss, sb, sh, ss, 1.0f, causal, dtype,

@@ -47,11 +47,20 @@ def _tile_table_ptr(k_info, q_ptr, head_num: int, q_seq_len: int, unit_kv_bytes:
     return None if q_ptr else k_info.tile_table(head_num, q_seq_len, unit_kv_bytes, query_tile).data_ptr()
 
 
+def _fused_dtype_ok(t: torch.Tensor, size_per_head: int, who: str) -> None:
+    """float16 / bfloat16 with heads of up to 128 channels, float32 with heads of up to 64."""
+    if t.dtype in (torch.float16, torch.bfloat16):
+        return
+    if t.dtype == torch.float32 and size_per_head <= 64:
+        return
+    raise RuntimeError(f"{who}: Datatype not implemented (float16 and bfloat16; float32 for heads of up to 64 channels)")
+
+
 def fused_query_tile(q_seq_len: int, k_seq_len: int, size_per_head: int, causal: bool, t: torch.Tensor,
                      query_tile: Optional[int] = None) -> int:
     """Query rows per workgroup of the fused kernel: the caller's choice (128, or 256 for the form with 64
     queries per wave, heads of 65..128 channels) or what the library picks for the shape."""
-    if query_tile:
+    if query_tile and t.dtype != torch.float32:
         if query_tile not in (128, 256) or (query_tile == 256 and size_per_head <= 64):
             raise RuntimeError("attn_fused: query_tile must be 128, or 256 for heads of 65..128 channels")
         return int(query_tile)
@@ -123,7 +132,8 @@ def attn_fused(q, k, v, seq_len_list, *, scale: Optional[float] = None, causal: 
     """ctx = softmax(scale * q k^T, mask) v in one kernel; the score tensor is never materialised.
 
     Same masking rule as ``scale_mask_softmax`` (``causal``, key lengths, optional query lengths);
-    ``scale`` defaults to ``size_per_head ** -0.5``.  fp16 / bf16 only.  Returns ``[B,H,Sq,D]``; rows of
+    ``scale`` defaults to ``size_per_head ** -0.5``.  fp16 / bf16 (heads of up to 128 channels) and fp32 (up to 64).
+    Returns ``[B,H,Sq,D]``; rows of
     padded queries are left uninitialised.  ``query_tile``: see :func:`fused_query_tile`.
     """
     qs = _bhsd(q, "q")
@@ -133,8 +143,7 @@ def attn_fused(q, k, v, seq_len_list, *, scale: Optional[float] = None, causal: 
     Sk = k.shape[2]
     if k.shape != (B, H, Sk, D) or v.shape != (B, H, Sk, D) or k.dtype != q.dtype or v.dtype != q.dtype:
         raise RuntimeError("attn_fused: q, k, v disagree in batch, heads, size_per_head, key length or dtype")
-    if q.dtype not in (torch.float16, torch.bfloat16):
-        raise RuntimeError("attn_fused: Datatype not implemented (float16 and bfloat16 only)")
+    _fused_dtype_ok(q, D, "attn_fused")
     k_info, q_info, q_ptr = _lens_ptrs(seq_len_list, q_len_list, B, q.device)
     if out is None:
         out = torch.empty((B, H, Sq, D), dtype=q.dtype, device=q.device)
@@ -151,8 +160,8 @@ def attn_fused(q, k, v, seq_len_list, *, scale: Optional[float] = None, causal: 
                                          k_info.lens.data_ptr(), q_ptr, B, H, Sq, Sk, D, arr(*qs), arr(*ks), arr(*vs),
                                          arr(*cs), None, None, scale, int(bool(causal)),
                                          _lib.dtype_tag(q, "attn_fused"),
-                                         _tile_table_ptr(k_info, q_ptr, H, Sq, _unit_kv_bytes(Sk, D, q), qt), qt,
-                                         _lib.stream_of(q)), "attn_fused")
+                                         None if qt == 64 else _tile_table_ptr(k_info, q_ptr, H, Sq, _unit_kv_bytes(Sk, D, q), qt),
+                                         qt, _lib.stream_of(q)), "attn_fused")
     return out
 
 
@@ -173,8 +182,7 @@ def attn_fused_varlen(q, k, v, batch_size: int, max_seq_len: int, seq_len_list, 
     T, H, D = q.shape
     if k.shape != q.shape or v.shape != q.shape or k.dtype != q.dtype or v.dtype != q.dtype:
         raise RuntimeError("attn_fused_varlen: q, k, v disagree in shape or dtype")
-    if q.dtype not in (torch.float16, torch.bfloat16):
-        raise RuntimeError("attn_fused_varlen: Datatype not implemented (float16 and bfloat16 only)")
+    _fused_dtype_ok(q, D, "attn_fused_varlen")
     info = seq_info(seq_len_list, batch_size, q.device)
     if out is None:
         out = torch.empty((1, T, H, D), dtype=q.dtype, device=q.device)
@@ -189,6 +197,7 @@ def attn_fused_varlen(q, k, v, batch_size: int, max_seq_len: int, seq_len_list, 
                                          info.lens.data_ptr(), None, batch_size, H, int(max_seq_len),
                                          int(max_seq_len), D, arr(*qs), arr(*ks), arr(*vs), arr(0, D, H * D), cu, cu,
                                          scale, int(bool(causal)), _lib.dtype_tag(q, "attn_fused_varlen"),
+                                         None if qt == 64 else
                                          info.tile_table(H, int(max_seq_len), _unit_kv_bytes(max_seq_len, D, q), qt).data_ptr(),
                                          qt, _lib.stream_of(q)), "attn_fused_varlen")
     return out

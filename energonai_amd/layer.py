@@ -39,10 +39,13 @@ def three_kernel_form(causal: bool, dtype: torch.dtype, max_seq_len: int) -> str
 def default_attention_form(causal: bool, dtype: torch.dtype, max_seq_len: int, size_per_head: int,
                            scale: float = 1.0) -> str:
     """The form ``padding_removal_layer`` runs when the caller names none: the fused kernel on the packed
-    projections wherever it applies (16-bit storage, heads of at most 128 channels in multiples of 8, a positive
-    scale) -- the score tensor then never exists and the step is two launches -- else the three kernels."""
+    projections wherever it applies (16-bit storage with heads of at most 128 channels in multiples of 8, fp32
+    with heads of at most 64 in multiples of 4, a positive scale) -- the score tensor then never exists and the
+    step is two launches -- else the three kernels."""
     if dtype in (torch.float16, torch.bfloat16) and size_per_head <= 128 and size_per_head % 8 == 0 and scale > 0:
         return "packed"
+    if dtype == torch.float32 and size_per_head <= 64 and size_per_head % 4 == 0 and scale > 0:
+        return "packed"      # the fp32 fused kernel (heads of up to 64 channels: the BERT-base shape)
     return three_kernel_form(causal, dtype, max_seq_len)
 
 
@@ -147,8 +150,10 @@ def _layer_one_call(hidden_padded, qkv_packed, info, B, S, H, D, hid, T, gamma, 
             raise RuntimeError("padding_removal_layer: dense_out must be [1,T,hidden] of the activation dtype")
     elif hid != H * D:
         raise RuntimeError("padding_removal_layer: without dense_out the LayerNorm width must equal heads * size_per_head")
-    if form in (1, 2, 4) and dt == torch.float32:
-        raise RuntimeError("padding_removal_layer: the fused kernel and the packed scores are for float16 and bfloat16")
+    if form == 4 and dt == torch.float32:
+        raise RuntimeError("padding_removal_layer: the packed scores are for float16 and bfloat16")
+    if form in (1, 2) and dt == torch.float32 and D > 64:
+        raise RuntimeError("padding_removal_layer: the fused kernel takes float32 heads of up to 64 channels")
     if form == 4 and not causal:
         raise RuntimeError("padding_removal_layer: the packed score layout is that of a causal mask")
     x = None if fold_depad else torch.empty((1, T, hid), dtype=dt, device=dev)

@@ -102,8 +102,13 @@ def test_entry_points_validate_before_launch():
     assert lib.en_decode_attn(16, 32, 48, 64, 80, 1, 1, 8, 64, i64x3, i64x3, 0.0, 1, None) == -5      # scale must be positive
     assert lib.en_decode_attn(16, 32, 48, 64, 80, 1, 1, 8, 60, i64x3, i64x3, 1.0, 1, None) == -5      # D not a multiple of 8
     assert lib.en_decode_attn(16, 32, 48, 64, 80, 1, 1, 2 ** 24, 64, i64x3, i64x3, 1.0, 1, None) == -5   # 32-bit offsets inside a unit
+    assert lib.en_attn_fused(16, 32, 48, 64, 80, None, 1, 1, 8, 8, 128, i64x3, i64x3, i64x3, i64x3, None, None, 1.0, 1, 0,
+                             None, 0, None) == -5                        # fp32: heads of up to 64 channels
     assert lib.en_attn_fused(16, 32, 48, 64, 80, None, 1, 1, 8, 8, 64, i64x3, i64x3, i64x3, i64x3, None, None, 1.0, 1, 0,
-                             None, 0, None) == -3                        # fp32 is not a fused-attention dtype
+                             96, 0, None) == -5                          # fp32: 64-row tiles, no table of 128-row ones
+    assert lib.en_attn_fused(16, 32, 48, 64, 80, None, 1, 1, 8, 8, 64, i64x3, i64x3, i64x3, i64x3, None, None, 1.0, 1, 3,
+                             None, 0, None) == -3                        # no such dtype
+    assert lib.en_attn_fused_query_tile(128, 128, 64, 0, 0) == 64
     assert lib.en_attn_fused(16, 32, 48, 64, 80, None, 1, 1, 8, 8, 64, i64x3, i64x3, i64x3, i64x3, None, None, 0.0, 1, 1,
                              None, 0, None) == -5                        # scale must be positive
     assert lib.en_attn_fused(16, 32, 48, 64, 80, None, 1, 1, 8, 8, 64, i64x3, i64x3, i64x3, i64x3, None, None, 1.0, 1, 1,

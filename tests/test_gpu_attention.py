@@ -251,12 +251,16 @@ def test_decode_attn_agrees_with_the_three_launch_route():
                         what="single pass vs three launches")
 
 
-@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16, torch.float32])
 @pytest.mark.parametrize("causal", [True, False])
 @pytest.mark.parametrize("B,H,S,D,lens", ATTN_CASES)
 def test_attn_fused(dtype, causal, B, H, S, D, lens):
     """One kernel for QK^T + mask/softmax + PV against the float64 oracle of the three steps."""
     k = _kernel()
+    if dtype == torch.float32 and D > 64:
+        with pytest.raises(RuntimeError, match="Datatype not implemented"):
+            k.attn_fused(*(torch.zeros(B, H, S, D, device="cuda") for _ in range(3)), torch.tensor(lens).cuda())
+        return
     announce("attn fused", dtype, causal, B, H, S, D, lens)
     T = sum(lens)
     qkv_packed = packed_randn(max(T, 1), H * 3 * D, dtype, 300 + S)[:T].reshape(T, H, 3 * D)
@@ -316,9 +320,13 @@ def test_attn_fused_and_pv_write_an_output_that_is_not_16_byte_aligned(D):
     assert bool((wide[..., :4] == 5.0).all()) and bool((wide[..., 4 + D:] == 5.0).all())
 
 
-@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+# fp16 / bf16: every case; fp32: the cases with heads of up to 64 channels (what the fp32 fused kernel takes)
+FUSED_PACKED_CASES = [(dt,) + c for dt in (torch.float16, torch.bfloat16) for c in ATTN_CASES] + \
+                     [(torch.float32,) + c for c in ATTN_CASES if c[3] <= 64]
+
+
 @pytest.mark.parametrize("causal", [True, False])
-@pytest.mark.parametrize("B,H,S,D,lens", ATTN_CASES)
+@pytest.mark.parametrize("dtype,B,H,S,D,lens", FUSED_PACKED_CASES)
 def test_attn_fused_packed(dtype, causal, B, H, S, D, lens):
     """The fused kernel addressing the packed [T,H,3D] projections and the packed [T,H*D] context
     directly: same result as pad -> attention -> depad, with no padded tensor in between."""

@@ -325,10 +325,11 @@ def test_layer_single_call_equals_the_op_by_op_sequence(name, form):
         assert torch.equal(once, ref["y"]) and torch.equal(steps["ctx_packed"], ref["ctx_packed"])
 
 
-@pytest.mark.parametrize("name,want_form", [("c1", "varlen"), ("c2", "packed")])
+@pytest.mark.parametrize("name,want_form", [("c1", "packed"), ("c2", "packed")])
 def test_layer_default_form(name, want_form):
     """With no form named the step runs the fused kernel on the packed projections where it applies (16-bit
-    storage), else the three kernels on packed operands; depad is folded into the LayerNorm either way."""
+    storage; fp32 with heads of up to 64 channels), else the three kernels on packed operands; depad is folded
+    into the LayerNorm either way."""
     layer, wl = _mods()
     w = wl.BY_NAME[name]
     announce("layer default form", name)
@@ -341,6 +342,16 @@ def test_layer_default_form(name, want_form):
     default = layer.padding_removal_layer(*args, dense_out=dense)
     named = layer.padding_removal_layer(*args, dense_out=dense, fused_attention=want_form, fold_depad=True)
     assert torch.equal(default, named)
+    # fp32 heads above 64 channels have no fused kernel: the three kernels on packed operands
+    assert layer.default_attention_form(False, torch.float32, 128, 128, 0.1) == "varlen"
+    assert layer.default_attention_form(True, torch.float32, 128, 64, 0.1) == "packed"
+    # and the default form meets the bound against the oracle that rounds nothing in between
+    want = eager.layer_unpadded(inp["hidden_padded"], inp["qkv_packed"], inp["lens_list"], w.heads, w.head_dim,
+                                inp["gamma"], inp["beta"], 1e-5, w.scale, w.causal, w.left_padded,
+                                dense_out=inp.get("dense_out"))
+    assert_stored_close(default.cpu(), want["y"], w.dtype,
+                        base=BASE[w.dtype] * (max(1.0, float(want["y"].abs().max())) if w.dtype == torch.float32 else 1.0),
+                        what="LayerNorm output of the default form")
 
 
 @pytest.mark.parametrize("name,form", [("c1", False), ("c2", False), ("c2", "packed"), ("c2", "varlen_packed")])
