@@ -44,7 +44,7 @@ def _unit_kv_bytes(k_seq_len: int, size_per_head: int, t: torch.Tensor) -> int:
 
 def _tile_table_ptr(k_info, q_ptr, head_num: int, q_seq_len: int, unit_kv_bytes: int, query_tile: int = 128):
     """Workgroup order for the batch (cached in its SeqInfo) when the query lengths are the key lengths."""
-    return None if q_ptr else k_info.tile_table(head_num, q_seq_len, unit_kv_bytes, query_tile).data_ptr()
+    return None if q_ptr else k_info.tile_table_ptr(head_num, q_seq_len, unit_kv_bytes, query_tile)
 
 
 def _fused_dtype_ok(t: torch.Tensor, size_per_head: int, who: str) -> None:
@@ -198,7 +198,7 @@ def attn_fused_varlen(q, k, v, batch_size: int, max_seq_len: int, seq_len_list, 
                                          int(max_seq_len), D, arr(*qs), arr(*ks), arr(*vs), arr(0, D, H * D), cu, cu,
                                          scale, int(bool(causal)), _lib.dtype_tag(q, "attn_fused_varlen"),
                                          None if qt == 64 else
-                                         info.tile_table(H, int(max_seq_len), _unit_kv_bytes(max_seq_len, D, q), qt).data_ptr(),
+                                         info.tile_table_ptr(H, int(max_seq_len), _unit_kv_bytes(max_seq_len, D, q), qt),
                                          qt, _lib.stream_of(q)), "attn_fused_varlen")
     return out
 
@@ -236,7 +236,7 @@ def attn_qk_varlen(q, k, batch_size: int, max_seq_len: int, seq_len_list, *, alp
     with _lib.device_guard(q):
         _lib.check(_lib.fn.en_attn_qk(q.data_ptr(), k.data_ptr(), out.data_ptr(), info.lens.data_ptr(), None, B, H, S, S, D,
                                       *qs, *ks, float(alpha), int(bool(causal)), _lib.dtype_tag(q, "attn_qk_varlen"), cu, cu,
-                                      int(bool(packed_scores)), info.tile_table(H, S, _unit_kv_bytes(S, D, q)).data_ptr(),
+                                      int(bool(packed_scores)), info.tile_table_ptr(H, S, _unit_kv_bytes(S, D, q)),
                                       _lib.stream_of(q)), "attn_qk_varlen")
     return out
 
@@ -275,7 +275,7 @@ def attn_pv_varlen(p, v, batch_size: int, max_seq_len: int, seq_len_list, *, cau
     with _lib.device_guard(v):
         _lib.check(_lib.fn.en_attn_pv(p.data_ptr(), v.data_ptr(), out.data_ptr(), info.lens.data_ptr(), None, B, H, S, S, D,
                                       *vs, 0, D, H * D, int(bool(causal)), 0, _lib.dtype_tag(v, "attn_pv_varlen"), cu, cu,
-                                      int(bool(packed_scores)), info.tile_table(H, S, _unit_kv_bytes(S, D, v)).data_ptr(),
+                                      int(bool(packed_scores)), info.tile_table_ptr(H, S, _unit_kv_bytes(S, D, v)),
                                       _lib.stream_of(v)), "attn_pv_varlen")
     return out
 

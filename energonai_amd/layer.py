@@ -180,7 +180,7 @@ def _layer_one_call(hidden_padded, qkv_packed, info, B, S, H, D, hid, T, gamma, 
             info.cu_seqlens.data_ptr(), info.lens.data_ptr(), B, S, H, D, hid, T, float(scale), float(eps),
             int(bool(causal)), int(bool(left_padded)), form, _lib.ptr(offs),
             _lib.dtype_tag(hidden_padded, "padding_removal_layer"),
-            info.tile_table(H, S, 2 * S * D * hidden_padded.element_size()).data_ptr(),
+            info.tile_table_ptr(H, S, 2 * S * D * hidden_padded.element_size()),
             _lib.stream_of(hidden_padded)), "padding_removal_layer")
     return y
 

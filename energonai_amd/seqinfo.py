@@ -24,7 +24,7 @@ class SeqInfo:
     """Device-resident int32 lengths and exclusive prefix for one batch."""
 
     __slots__ = ("lens", "cu_seqlens", "batch_size", "_total", "_source", "_row_offsets", "_tile_tables", "_ready",
-                 "_ordered")
+                 "_ordered", "ephemeral")
 
     def __init__(self, lens: torch.Tensor, cu_seqlens: torch.Tensor, batch_size: int, total: Optional[int], source):
         self.lens = lens                # int32 [B] on the device
@@ -36,6 +36,7 @@ class SeqInfo:
         self._tile_tables = {}          # (head_num, q_seq_len, order, version of lens, tile height) -> int32 workgroup order
         self._ready = []                # events recorded behind the kernels that produced the arrays above
         self._ordered = set()           # raw streams already ordered behind every event of _ready
+        self.ephemeral = False          # built for one call only (lengths that cannot be cached): see tile_table_ptr
 
     def produced_on_current_stream(self) -> None:
         """Call right after launching a kernel that writes one of this object's arrays: remembers the point
@@ -135,6 +136,16 @@ class SeqInfo:
         return tab
 
 
+    def tile_table_ptr(self, head_num: int, q_seq_len: int, unit_kv_bytes: int = 1 << 30, query_tile: int = 128):
+        """Raw pointer of the workgroup order for an attention call, or ``None`` (the kernels then compute their
+        own order) when this object lives for one call only: building the table is a launch of its own, which pays
+        off when every layer reuses it, not when every call would rebuild it (lengths given as Python lists or as
+        tensors made under ``torch.inference_mode()`` are never cached -- pass a ``SeqInfo`` to keep one)."""
+        if self.ephemeral:
+            return None
+        return self.tile_table(head_num, q_seq_len, unit_kv_bytes, query_tile).data_ptr()
+
+
 _cache: "OrderedDict[tuple, SeqInfo]" = OrderedDict()
 
 
@@ -185,7 +196,9 @@ def seq_info(seq_lens, batch_size: int, device=None) -> SeqInfo:
         seq_lens.order_current_stream()
         return seq_lens
     if not isinstance(seq_lens, torch.Tensor) or torch.is_inference(seq_lens):
-        return build_seq_info(seq_lens, batch_size, device)
+        info = build_seq_info(seq_lens, batch_size, device)
+        info.ephemeral = True
+        return info
     key = (id(seq_lens), seq_lens._version, seq_lens.data_ptr(), batch_size, str(device))
     hit = _cache.get(key)
     if hit is not None and hit._source is seq_lens:

@@ -205,9 +205,9 @@ def test_public_attention_calls_pass_the_tile_table_when_there_are_no_query_leng
         def __init__(self):
             self.asked = []
 
-        def tile_table(self, head_num, q_seq_len, unit_kv_bytes, query_tile=128):
+        def tile_table_ptr(self, head_num, q_seq_len, unit_kv_bytes, query_tile=128):
             self.asked.append((head_num, q_seq_len, unit_kv_bytes))
-            return Table()
+            return Table().data_ptr()
 
     info = Info()
     assert attention._tile_table_ptr(info, 0, 12, 512, 1 << 17) == 4096 and info.asked == [(12, 512, 1 << 17)]
