@@ -790,7 +790,9 @@ __global__ __launch_bounds__(kBlock, 3) void attn_pv_strip_kernel(AttnArgs a) {
 //   tile index by tile index from the last to the first, every unit that has the tile (tiles_first == 1): the
 //     long workgroups of all units start first -- the better schedule when a unit's K and V are small enough
 //     to be re-read cheaply (512-key, 64-channel units: 21.3 -> 19.6 us; 1024 x 128: 213 -> 225 us).
-// One workgroup; the sort is a rank count (batch <= 1024), larger batches keep their order.
+// One workgroup; the sort is a rank count (batch <= 1024), larger batches keep their order.  The fill is spread over
+// the whole workgroup when the batch is sorted (a serial walk by eight threads took 43 us for 896 units of up to
+// eight tiles).
 __global__ __launch_bounds__(1024) void attn_tile_table_kernel(const int32_t *__restrict__ lens, int batch, int heads,
                                                                int seq_len, int ntq, int32_t *__restrict__ table,
                                                                int capacity, int tiles_first, int q_tile) {
@@ -810,15 +812,63 @@ __global__ __launch_bounds__(1024) void attn_tile_table_kernel(const int32_t *__
     }
   }
   __syncthreads();   // also orders the -1 fill before the entries written below
-  if (tid < kXcds) {
-    const int units = batch * heads;
-    auto tiles_of = [&](int u, int &unit) {          // u-th unit in sorted order -> its index and tile count
-      const int p = u / heads, h = u - p * heads;
-      const int b = sorted ? s_order[p] : p;
-      const int n = sorted ? s_len[b] : min(max(lens[b], 0), seq_len);
-      unit = b * heads + h;
-      return (n + q_tile - 1) / q_tile;
-    };
+  const int units = batch * heads;
+  auto tiles_of = [&](int u, int &unit) {          // u-th unit in sorted order -> its index and tile count
+    const int p = u / heads, h = u - p * heads;
+    const int b = sorted ? s_order[p] : p;
+    const int n = sorted ? s_len[b] : min(max(lens[b], 0), seq_len);
+    unit = b * heads + h;
+    return (n + q_tile - 1) / q_tile;
+  };
+  constexpr int kChunks = 1024 / kXcds;             // threads per XCD list
+  constexpr int kMaxTiles = 256;
+  if (sorted && ntq <= kMaxTiles) {
+    // Every thread takes a contiguous chunk of one XCD's unit list (units x, x + 8, x + 16, ... of the sorted order).
+    // Sorted by length, the tile counts along a list never increase, so the units that have tile qi are a prefix of
+    // the list: a unit's place among them is its place in the list.
+    __shared__ int32_t s_sum[kXcds][kChunks + 1];   // unit-major: tiles in the chunks before this one
+    __shared__ int32_t s_cnt[kXcds][kMaxTiles + 1]; // tiles-first: units of the list that have tile qi
+    const int x = tid % kXcds, c = tid / kXcds;
+    const int list_len = (units - x + kXcds - 1) / kXcds;            // units x + 8 i, i < list_len
+    const int per = (list_len + kChunks - 1) / kChunks;
+    const int i0 = min(c * per, list_len), i1 = min(i0 + per, list_len);
+    for (int i = tid; i < kXcds * (kMaxTiles + 1); i += 1024) (&s_cnt[0][0])[i] = 0;
+    __syncthreads();
+    int mine = 0, unit;
+    for (int i = i0; i < i1; ++i) {
+      const int nt = tiles_of(x + kXcds * i, unit);
+      mine += nt;
+      if (tiles_first && nt > 0) atomicAdd(&s_cnt[x][nt - 1], 1);     // units whose LAST tile is nt - 1
+    }
+    s_sum[x][c] = mine;
+    __syncthreads();
+    if (tid < kXcds) {
+      if (tiles_first) {      // units that have tile qi = units whose last tile is >= qi; then where tile qi's run starts
+        int run = 0;
+        for (int qi = ntq - 1; qi >= 0; --qi) { run += s_cnt[tid][qi]; s_cnt[tid][qi] = run; }
+        int start = 0;
+        for (int qi = ntq - 1; qi >= 0; --qi) { const int n = s_cnt[tid][qi]; s_cnt[tid][qi] = start; start += n; }
+      } else {
+        int run = 0;
+        for (int k = 0; k < kChunks; ++k) { const int n = s_sum[tid][k]; s_sum[tid][k] = run; run += n; }
+      }
+    }
+    __syncthreads();
+    if (tiles_first) {
+      for (int i = i0; i < i1; ++i) {
+        const int nt = tiles_of(x + kXcds * i, unit);
+        for (int qi = nt - 1; qi >= 0; --qi) table[(s_cnt[x][qi] + i) * kXcds + x] = unit * ntq + qi;
+      }
+    } else {
+      int j = s_sum[x][c];
+      for (int i = i0; i < i1; ++i) {
+        const int nt = tiles_of(x + kXcds * i, unit);
+        for (int qi = nt - 1; qi >= 0; --qi) table[j++ * kXcds + x] = unit * ntq + qi;
+      }
+    }
+    return;
+  }
+  if (tid < kXcds) {      // batches too large to sort, rows of more than 256 tiles: one thread per XCD walks its list
     int j = 0, unit;
     if (tiles_first) {
       for (int qi = ntq - 1; qi >= 0; --qi)
