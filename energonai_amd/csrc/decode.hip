@@ -200,13 +200,15 @@ struct DecodeAttnArgs {
   int B, H, Sk, D;
   int64_t k_sb, k_sh, k_ss, v_sb, v_sh, v_ss;
   float c_exp;        // scale * log2(e)
+  int nsplit;         // workgroups that share one (batch, head) unit's keys (grid z); 1: none
+  float *partial;     // nsplit > 1: [B*H][nsplit][D + 2] unnormalised output, maximum (log2 domain), sum
 };
 
 constexpr int kRankBatch = 256;
 
-template <int DT, int LPK, bool STREAM>
-__global__ __launch_bounds__(STREAM ? kStreamBlock : kBlock, 8) void decode_attn_kernel(DecodeAttnArgs a) {
-  constexpr int NT = STREAM ? kStreamBlock : en::kBlock;
+template <int DT, int LPK, bool STREAM, bool BIG>
+__global__ __launch_bounds__(BIG ? kStreamBlock : kBlock, 8) void decode_attn_kernel(DecodeAttnArgs a) {
+  constexpr int NT = BIG ? kStreamBlock : en::kBlock;
   typedef Elem<DT> E;
   typedef typename E::T T;
   constexpr int EPV = 16 / E::kSize;
@@ -238,6 +240,11 @@ __global__ __launch_bounds__(STREAM ? kStreamBlock : kBlock, 8) void decode_attn
   }
   const int c = tid % LPK, g = tid / LPK;
   const int kl = max(min(a.kv_lens[b], a.Sk), 0);
+  // with the keys of a unit split over nsplit workgroups this one takes [kbeg, kend); a share past the end has no
+  // workgroup's worth of work and leaves no partial (the combine kernel derives the same shares from the length)
+  const int share = (kl + a.nsplit - 1) / a.nsplit;
+  const int kbeg = (int)blockIdx.z * share, kend = min(kl, kbeg + share);
+  if (a.nsplit > 1 && kbeg >= kl) return;
   const T *q = reinterpret_cast<const T *>(a.q) + ((int64_t)b * a.H + h) * a.D;
   const T *kbase = reinterpret_cast<const T *>(a.k) + (int64_t)b * a.k_sb + (int64_t)h * a.k_sh;
   const T *vbase = reinterpret_cast<const T *>(a.v) + (int64_t)b * a.v_sb + (int64_t)h * a.v_sh;
@@ -270,7 +277,7 @@ __global__ __launch_bounds__(STREAM ? kStreamBlock : kBlock, 8) void decode_attn
 #pragma unroll
     for (int u = 0; u < U; ++u) {
       const int key = k0 + u * G + g;
-      const uint32_t in = key < kl ? 0u : kOutOfRange;       // past the end: out of range whatever the stride
+      const uint32_t in = key < kend ? 0u : kOutOfRange;     // past the end: out of range whatever the stride
       kk[u] = buffer_load16<AUX>(k_rsrc, (uint32_t)key * k_row + col | in);
       vv[u] = buffer_load16<AUX>(v_rsrc, (uint32_t)key * v_row + col | in);
     }
@@ -286,7 +293,7 @@ __global__ __launch_bounds__(STREAM ? kStreamBlock : kBlock, 8) void decode_attn
 #pragma unroll
       for (int e = 0; e < EPV; ++e) dot += qv[e] * E::to_float(kp.v[e]);
       dot = group_allreduce<OpSum, LPK>(dot);
-      sc[u] = key < kl ? dot : -INFINITY;
+      sc[u] = key < kend ? dot : -INFINITY;
       m_new = fmaxf(m_new, sc[u]);
     }
     if (m_new > -INFINITY) {            // this group has seen a key: (-inf) - (-inf) never reaches exp2
@@ -311,8 +318,8 @@ __global__ __launch_bounds__(STREAM ? kStreamBlock : kBlock, 8) void decode_attn
   static_assert((2 * NS - 1) * STEP <= 4096, "the host check allows 4096 keys past the end");
   uint4 kr[NS][U], vr[NS][U];
 #pragma unroll
-  for (int st = 0; st < NS - 1; ++st) load_stage(kr[st], vr[st], st * STEP);
-  for (int k0 = 0; k0 < kl; k0 += NS * STEP) {   // uniform trip count: all lanes reach the reductions
+  for (int st = 0; st < NS - 1; ++st) load_stage(kr[st], vr[st], kbeg + st * STEP);
+  for (int k0 = kbeg; k0 < kend; k0 += NS * STEP) {   // uniform trip count: all lanes reach the reductions
 #pragma unroll
     for (int st = 0; st < NS; ++st) {
       load_stage(kr[(st + NS - 1) % NS], vr[(st + NS - 1) % NS], k0 + (st + NS - 1) * STEP);
@@ -327,6 +334,7 @@ __global__ __launch_bounds__(STREAM ? kStreamBlock : kBlock, 8) void decode_attn
   for (int j = 0; j < G; ++j) m_all = fmaxf(m_all, s_m[j]);
   if (tid < G) s_w[tid] = s_m[tid] > -INFINITY ? __builtin_amdgcn_exp2f(s_m[tid] - m_all) : 0.f;
   __syncthreads();
+  float *part = a.nsplit > 1 ? a.partial + (((int64_t)b * a.H + h) * a.nsplit + blockIdx.z) * (a.D + 2) : nullptr;
   for (int d = tid; d < a.D; d += NT) {
     float l = 0.f, o = 0.f;
 #pragma unroll 4
@@ -334,14 +342,51 @@ __global__ __launch_bounds__(STREAM ? kStreamBlock : kBlock, 8) void decode_attn
       l += s_l[j] * s_w[j];
       o += s_acc[j][d] * s_w[j];
     }
-    ctx[d] = E::from_float(l > 0.f ? o / l : 0.f);
+    if (part) {
+      part[d] = o;
+      if (d == 0) { part[a.D] = m_all; part[a.D + 1] = l; }
+    } else {
+      ctx[d] = E::from_float(l > 0.f ? o / l : 0.f);
+    }
+  }
+}
+
+// Combines the partial results of the workgroups that shared a unit's keys: one workgroup per (batch, head).
+template <int DT>
+__global__ __launch_bounds__(kBlock) void decode_attn_combine_kernel(DecodeAttnArgs a) {
+  typedef Elem<DT> E;
+  typedef typename E::T T;
+  const int unit = blockIdx.x, b = unit / a.H;
+  const int kl = max(min(a.kv_lens[b], a.Sk), 0);
+  const int share = (kl + a.nsplit - 1) / a.nsplit;
+  const int nvalid = share > 0 ? (kl + share - 1) / share : 0;       // shares that had keys
+  const float *part = a.partial + (int64_t)unit * a.nsplit * (a.D + 2);
+  T *ctx = reinterpret_cast<T *>(a.ctx) + (int64_t)unit * a.D;
+  float m_all = -INFINITY;
+  for (int z = 0; z < nvalid; ++z) m_all = fmaxf(m_all, part[z * (a.D + 2) + a.D]);
+  float l = 0.f;
+  for (int z = 0; z < nvalid; ++z) {
+    const float m = part[z * (a.D + 2) + a.D];
+    l += m > -INFINITY ? part[z * (a.D + 2) + a.D + 1] * __builtin_amdgcn_exp2f(m - m_all) : 0.f;
+  }
+  const float inv = l > 0.f ? 1.0f / l : 0.f;
+  for (int d = threadIdx.x; d < a.D; d += kBlock) {
+    float o = 0.f;
+    for (int z = 0; z < nvalid; ++z) {
+      const float m = part[z * (a.D + 2) + a.D];
+      o += m > -INFINITY ? part[z * (a.D + 2) + d] * __builtin_amdgcn_exp2f(m - m_all) : 0.f;
+    }
+    ctx[d] = E::from_float(o * inv);
   }
 }
 
 template <int DT, int LPK> struct AttnLauncher {
-  static void go(const DecodeAttnArgs &a, dim3 grid, bool stream_cache, hipStream_t s) {
-    if (stream_cache) decode_attn_kernel<DT, LPK, true><<<grid, kStreamBlock, 0, s>>>(a);
-    else decode_attn_kernel<DT, LPK, false><<<grid, kBlock, 0, s>>>(a);
+  // stream_cache: caches too large to stay in the memory-side cache between steps are read with non-temporal loads;
+  // big: 1024-lane workgroups (large caches, and whenever a unit's keys are split: few units, long rows)
+  static void go(const DecodeAttnArgs &a, dim3 grid, bool stream_cache, bool big, hipStream_t s) {
+    if (stream_cache) decode_attn_kernel<DT, LPK, true, true><<<grid, kStreamBlock, 0, s>>>(a);
+    else if (big) decode_attn_kernel<DT, LPK, false, true><<<grid, kStreamBlock, 0, s>>>(a);
+    else decode_attn_kernel<DT, LPK, false, false><<<grid, kBlock, 0, s>>>(a);
   }
 };
 
@@ -350,17 +395,35 @@ static int dispatch_attn(const DecodeAttnArgs &a, bool stream_cache, hipStream_t
   constexpr int EPV = 16 / Elem<DT>::kSize;
   int lpk = 4;
   while (lpk * EPV < a.D) lpk *= 2;
-  dim3 grid((unsigned)a.H, (unsigned)a.B, 1);
+  dim3 grid((unsigned)a.H, (unsigned)a.B, (unsigned)a.nsplit);
+  const bool big = stream_cache || a.nsplit > 1;
   switch (lpk) {
-    case 4: AttnLauncher<DT, 4>::go(a, grid, stream_cache, s); break;
-    case 8: AttnLauncher<DT, 8>::go(a, grid, stream_cache, s); break;
-    case 16: AttnLauncher<DT, 16>::go(a, grid, stream_cache, s); break;
-    case 32: AttnLauncher<DT, 32>::go(a, grid, stream_cache, s); break;
-    case 64: AttnLauncher<DT, 64>::go(a, grid, stream_cache, s); break;
+    case 4: AttnLauncher<DT, 4>::go(a, grid, stream_cache, big, s); break;
+    case 8: AttnLauncher<DT, 8>::go(a, grid, stream_cache, big, s); break;
+    case 16: AttnLauncher<DT, 16>::go(a, grid, stream_cache, big, s); break;
+    case 32: AttnLauncher<DT, 32>::go(a, grid, stream_cache, big, s); break;
+    case 64: AttnLauncher<DT, 64>::go(a, grid, stream_cache, big, s); break;
     default: return EN_ERR_UNSUPPORTED;
   }
   EN_RETURN_IF_LAUNCH_FAILED();
+  if (a.nsplit > 1) {
+    decode_attn_combine_kernel<DT><<<(unsigned)(a.B * a.H), kBlock, 0, s>>>(a);
+    EN_RETURN_IF_LAUNCH_FAILED();
+  }
   return EN_OK;
+}
+
+// How many workgroups share one unit's keys: none while the units alone fill the chip's 512 slots of 1024 lanes;
+// else enough for about two slots' worth per CU, each share at least 512 keys long (shorter shares cost more in
+// workgroup start-up and in the combine pass than they win: 22 us instead of 25 for one sequence of 2048 keys).
+static int decode_split(int batch, int head_num, int k_seq_len) {
+  constexpr int kTargetWorkgroups = 1024, kMinShare = 512;
+  const int64_t units = (int64_t)batch * head_num;
+  if (units >= 512 || k_seq_len < 2 * kMinShare) return 1;
+  int64_t n = (kTargetWorkgroups + units - 1) / units;
+  if (n > k_seq_len / kMinShare) n = k_seq_len / kMinShare;
+  if (n > 64) n = 64;
+  return n < 1 ? 1 : (int)n;
 }
 
 // Appends one new K row and one new V row per (batch, head) to the caches at position
@@ -432,9 +495,16 @@ int en_kv_append(const void *k_new, const void *v_new, void *k_cache, void *v_ca
   return EN_OK;
 }
 
+int64_t en_decode_attn_workspace_bytes(int batch, int head_num, int k_seq_len, int size_per_head) {
+  using namespace en;
+  if (batch < 1 || head_num < 1 || k_seq_len < 1 || size_per_head < 1) return 0;
+  const int n = decode_split(batch, head_num, k_seq_len);
+  return n > 1 ? (int64_t)batch * head_num * n * (size_per_head + 2) * (int64_t)sizeof(float) : 0;
+}
+
 int en_decode_attn(const void *q, const void *k_cache, const void *v_cache, void *ctx, const int32_t *kv_lens, int batch,
                    int head_num, int k_seq_len, int size_per_head, const int64_t *k_strides, const int64_t *v_strides,
-                   float scale, int dtype, en_stream_t stream) {
+                   float scale, int dtype, void *workspace, int64_t workspace_bytes, en_stream_t stream) {
   using namespace en;
   if (!k_strides || !v_strides || !v_cache) return EN_ERR_NULL;
   int rc = check_decode(q, k_cache, ctx, kv_lens, batch, head_num, k_seq_len, size_per_head, k_strides[0], k_strides[1],
@@ -450,8 +520,12 @@ int en_decode_attn(const void *q, const void *k_cache, const void *v_cache, void
   if (!(scale > 0.f)) return EN_ERR_UNSUPPORTED;     // the running maximum is kept in units of scale * log2(e)
   for (int i = 0; i < 3; ++i)
     if (k_strides[i] < 0 || v_strides[i] < 0) return EN_ERR_UNSUPPORTED;
+  // a unit's keys are shared between workgroups only when the caller brought the room for their partial results
+  const int64_t need = en_decode_attn_workspace_bytes(batch, head_num, k_seq_len, size_per_head);
+  const bool split = need > 0 && workspace && workspace_bytes >= need && aligned_to(workspace, 4);
   DecodeAttnArgs a{q, k_cache, v_cache, ctx, kv_lens, batch, head_num, k_seq_len, size_per_head, k_strides[0], k_strides[1],
-                   k_strides[2], v_strides[0], v_strides[1], v_strides[2], scale * 1.4426950408889634f};
+                   k_strides[2], v_strides[0], v_strides[1], v_strides[2], scale * 1.4426950408889634f,
+                   split ? decode_split(batch, head_num, k_seq_len) : 1, static_cast<float *>(workspace)};
   const bool stream_cache = 2 * cache_bytes(batch, head_num, k_seq_len, size_per_head, dtype) >= kStreamCacheBytes;
   hipStream_t s = (hipStream_t)stream;
   switch (dtype) {

@@ -16,6 +16,7 @@ from .cuda_native import (ft_build_padding_offsets, ft_remove_padding, ft_rebuil
 from .cuda_native import linear, find_algo
 from .cuda_native import LayerNorm, layer_norm_forward
 from .attention import (attn_qk, attn_pv, attn_fused, attn_fused_packed, attn_fused_varlen, decode_qk, decode_pv, decode_attn,
+                        decode_attn_workspace_bytes,
                         kv_cache_fill, kv_cache_append, attn_qk_varlen, attn_pv_varlen, scale_mask_softmax_packed,
                         packed_scores_elems)
 
@@ -23,6 +24,6 @@ __all__ = [
     "transpose_pad", "transpose_depad", "depad", "scale_mask_softmax", "ft_build_padding_offsets",
     "ft_remove_padding", "ft_rebuild_padding", "ft_transpose_remove_padding", "ft_transpose_rebuild_padding",
     "linear", "find_algo", "LayerNorm", "layer_norm_forward", "attn_qk", "attn_pv", "attn_fused",
-    "attn_fused_packed", "attn_fused_varlen", "decode_qk", "decode_pv", "decode_attn", "kv_cache_fill", "kv_cache_append", "repad",
+    "attn_fused_packed", "attn_fused_varlen", "decode_qk", "decode_pv", "decode_attn", "decode_attn_workspace_bytes", "kv_cache_fill", "kv_cache_append", "repad",
     "attn_qk_varlen", "attn_pv_varlen", "scale_mask_softmax_packed", "packed_scores_elems",
 ]

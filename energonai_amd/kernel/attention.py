@@ -379,11 +379,16 @@ def decode_pv(p, v_cache, kv_len_list, *, out: Optional[torch.Tensor] = None):
     return out
 
 
-def decode_attn(q, k_cache, v_cache, kv_len_list, *, scale: Optional[float] = None, out: Optional[torch.Tensor] = None):
+def decode_attn(q, k_cache, v_cache, kv_len_list, *, scale: Optional[float] = None, out: Optional[torch.Tensor] = None,
+                workspace: Optional[torch.Tensor] = None, split: bool = True):
     """ctx[b,h,0,:] = sum_j softmax_j(scale * <q[b,h,0,:], k_cache[b,h,j,:]>) v_cache[b,h,j,:] over the cached
     positions ``j < kv_len[b]``, in one pass over the caches: what ``decode_qk`` -> ``scale_mask_softmax`` ->
     ``decode_pv`` compute in three launches (and the reference by recomputing the whole square,
-    energonai/model/attention.py:61-71,106-118).  ``[B,H,1,D]``; ``scale`` defaults to ``size_per_head ** -0.5``."""
+    energonai/model/attention.py:61-71,106-118).  ``[B,H,1,D]``; ``scale`` defaults to ``size_per_head ** -0.5``.
+    A batch with fewer than 512 (batch, head) units shares each unit's keys between several workgroups and combines
+    their partial results in a second small kernel; the fp32 buffer they pass through is ``workspace`` (any
+    tensor of at least ``decode_attn_workspace_bytes`` bytes) or a temporary; ``split=False`` keeps one workgroup
+    per unit."""
     _lib.require_gpu(q, "q", contiguous=False)
     ks = _bhsd(k_cache, "k_cache")
     vs = _bhsd(v_cache, "v_cache")
@@ -402,8 +407,22 @@ def decode_attn(q, k_cache, v_cache, kv_len_list, *, scale: Optional[float] = No
             raise RuntimeError("decode_attn: out must be a contiguous [B,H,1,D] tensor of q's dtype")
     arr = ctypes.c_int64 * 3
     scale = float(D) ** -0.5 if scale is None else float(scale)
+    need = decode_attn_workspace_bytes(B, H, Smax, D) if split else 0
+    if need and workspace is None:
+        workspace = torch.empty(need, dtype=torch.uint8, device=q.device)
+    ws_bytes = 0
+    if workspace is not None and need:
+        _lib.require_gpu(workspace, "workspace")
+        ws_bytes = workspace.numel() * workspace.element_size()
     with _lib.device_guard(q):
         _lib.check(_lib.fn.en_decode_attn(q_.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), out.data_ptr(),
                                           info.lens.data_ptr(), B, H, Smax, D, arr(*ks), arr(*vs), scale,
-                                          _lib.dtype_tag(q, "decode_attn"), _lib.stream_of(q)), "decode_attn")
+                                          _lib.dtype_tag(q, "decode_attn"), _lib.ptr(workspace) if ws_bytes else None,
+                                          ws_bytes, _lib.stream_of(q)), "decode_attn")
     return out
+
+
+def decode_attn_workspace_bytes(batch_size: int, head_num: int, max_seq_len: int, size_per_head: int) -> int:
+    """Bytes of the buffer through which ``decode_attn`` passes partial results when it shares a unit's keys between
+    workgroups (0: this shape gets one workgroup per unit)."""
+    return int(_lib.fn.en_decode_attn_workspace_bytes(int(batch_size), int(head_num), int(max_seq_len), int(size_per_head)))

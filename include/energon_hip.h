@@ -251,10 +251,16 @@ int en_decode_pv(const void *p, const void *v_cache, void *ctx, const int32_t *k
  * else touches memory.  q and ctx [B,H,D] contiguous; k_strides / v_strides point to three int64 in host memory
  * (batch, head, position strides in elements) of the [B,H,Smax,D] caches.  scale must be positive.  A sequence
  * with kv_lens[b] == 0 gets a zero row.  fp32 statistics and accumulation; dtypes and head sizes as
- * en_decode_qk. */
+ * en_decode_qk.
+ * workspace (device, 4-byte aligned, or NULL): a batch too small to fill the chip with one workgroup per
+ * (batch, head) -- fewer than 512 such units -- has the keys of each unit shared between several workgroups, whose
+ * partial results (fp32) pass through this buffer and are combined by a second small kernel;
+ * en_decode_attn_workspace_bytes gives the size that asks for (0: no sharing for this shape).  With NULL, or fewer
+ * bytes than that, every unit keeps one workgroup.  Nothing in the buffer has to be initialised or kept. */
+int64_t en_decode_attn_workspace_bytes(int batch, int head_num, int k_seq_len, int size_per_head);
 int en_decode_attn(const void *q, const void *k_cache, const void *v_cache, void *ctx, const int32_t *kv_lens, int batch,
                    int head_num, int k_seq_len, int size_per_head, const int64_t *k_strides, const int64_t *v_strides,
-                   float scale, int dtype, en_stream_t stream);
+                   float scale, int dtype, void *workspace, int64_t workspace_bytes, en_stream_t stream);
 
 /* Appends the new token's K and V rows to [B,H,Smax,D] caches at position
  * kv_lens[b] (the caller then adds one to kv_lens); replaces the reference's

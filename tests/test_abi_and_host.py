@@ -98,10 +98,13 @@ def test_entry_points_validate_before_launch():
     assert lib.en_transpose_pad_heads(16, 32, 48, 1, 1, 4, 8, 6, 4, 1, 2, None) == -2   # heads 4..7 of a 6-row source
     assert lib.en_kv_append(16, 32, 48, 64, None, 1, 1, 1, 8, 8, 8, 8, 8, 8, 2, None, None) == -1
     assert lib.en_kv_append(16, 32, 48, 64, 80, 1, 1, 1, 8, 8, 8, 8, 8, 8, 3, None, None) == -3   # element size 3
-    assert lib.en_decode_attn(16, 32, None, 64, 80, 1, 1, 8, 64, i64x3, i64x3, 1.0, 1, None) == -1    # no V cache
-    assert lib.en_decode_attn(16, 32, 48, 64, 80, 1, 1, 8, 64, i64x3, i64x3, 0.0, 1, None) == -5      # scale must be positive
-    assert lib.en_decode_attn(16, 32, 48, 64, 80, 1, 1, 8, 60, i64x3, i64x3, 1.0, 1, None) == -5      # D not a multiple of 8
-    assert lib.en_decode_attn(16, 32, 48, 64, 80, 1, 1, 2 ** 24, 64, i64x3, i64x3, 1.0, 1, None) == -5   # 32-bit offsets inside a unit
+    assert lib.en_decode_attn(16, 32, None, 64, 80, 1, 1, 8, 64, i64x3, i64x3, 1.0, 1, None, 0, None) == -1    # no V cache
+    assert lib.en_decode_attn(16, 32, 48, 64, 80, 1, 1, 8, 64, i64x3, i64x3, 0.0, 1, None, 0, None) == -5      # scale must be positive
+    assert lib.en_decode_attn(16, 32, 48, 64, 80, 1, 1, 8, 60, i64x3, i64x3, 1.0, 1, None, 0, None) == -5      # D not a multiple of 8
+    assert lib.en_decode_attn(16, 32, 48, 64, 80, 1, 1, 2 ** 24, 64, i64x3, i64x3, 1.0, 1, None, 0, None) == -5   # 32-bit offsets inside a unit
+    assert lib.en_decode_attn_workspace_bytes(64, 72, 2048, 128) == 0          # 4608 units fill the chip
+    assert lib.en_decode_attn_workspace_bytes(1, 72, 2048, 128) == 72 * 4 * 130 * 4   # 72 units: four shares of 512 keys each
+    assert lib.en_decode_attn_workspace_bytes(4, 72, 300, 128) == 0            # short caches are not shared
     assert lib.en_attn_fused(16, 32, 48, 64, 80, None, 1, 1, 8, 8, 128, i64x3, i64x3, i64x3, i64x3, None, None, 1.0, 1, 0,
                              None, 0, None) == -5                        # fp32: heads of up to 64 channels
     assert lib.en_attn_fused(16, 32, 48, 64, 80, None, 1, 1, 8, 8, 64, i64x3, i64x3, i64x3, i64x3, None, None, 1.0, 1, 0,

@@ -230,6 +230,18 @@ def test_decode_attn_single_pass(dtype, B, H, S, D, kv):
     both = torch.cat([kc, vc], dim=-1).cuda()
     got2 = k.decode_attn(q.cuda(), both[..., :D], both[..., D:], kv_t, scale=scale)
     assert torch.equal(got2, got)
+    # small batches share a unit's keys between workgroups (partial results through a workspace, then a combine
+    # kernel); with one workgroup per unit the result meets the same bound, and a caller's own workspace gives the
+    # bits of the temporary one
+    one_wg = k.decode_attn(q.cuda(), kc.cuda(), vc.cuda(), kv_t, scale=scale, split=False)
+    assert_ctx_close(one_wg.cpu(), want, dtype, "decode_attn, one workgroup per unit")
+    need = k.decode_attn_workspace_bytes(B, H, S, D)
+    assert (need > 0) == (B * H < 512 and S >= 1024)
+    if need:
+        ws = torch.full((need + 64,), 0xFF, dtype=torch.uint8, device="cuda")
+        got3 = k.decode_attn(q.cuda(), kc.cuda(), vc.cuda(), kv_t, scale=scale, workspace=ws)
+        assert torch.equal(got3, got)
+        assert bool((ws[need:] == 0xFF).all())
 
 
 def test_decode_attn_agrees_with_the_three_launch_route():
