@@ -68,8 +68,17 @@ __global__ __launch_bounds__(kBlock, 3) void attn_fused_kernel(FusedArgs fa) {
   const int b = unit / a.H, h = unit % a.H;
   int kl, ql;
   seq_extents(a, b, kl, ql);
+#ifdef EN_FUSED_START_ANCHORED
   const int q0 = qi * kQTile;
   if (q0 >= ql) return;
+#else
+  // The query tiles of a sequence are laid from its END: tile i of n covers rows ql - (n - i) * 128 .. and the ragged
+  // tile is the first one (rows below 0 do not exist), whose walk over the keys is the shortest under a causal mask.
+  // Laid from the start, the ragged tile would be the last one: a few rows holding a slot for the longest walk.
+  const int ntl = (ql + kQTile - 1) / kQTile;
+  if (qi >= ntl) return;
+  const int q0 = ql - (ntl - qi) * kQTile;
+#endif
   const int nk = tile_key_extent(a, min(q0 + kQTile, ql) - 1, kl, ql);
   const int nkt = (nk + BK - 1) / BK;
 
@@ -80,7 +89,7 @@ __global__ __launch_bounds__(kBlock, 3) void attn_fused_kernel(FusedArgs fa) {
   // smallest need no masking, tiles from the largest on hold nothing for this wave
   const int q_first = q0 + wave * 32;
   const int vis_min = (q_first + 31 < ql) ? (a.causal ? min(kl, q_first + (kl - ql) + 1) : kl) : 0;
-  const int vis_max = (q_first < ql) ? (a.causal ? min(kl, min(q_first + 31, ql - 1) + (kl - ql) + 1) : kl) : 0;
+  const int vis_max = (q_first < ql && q_first + 31 >= 0) ? (a.causal ? min(kl, min(q_first + 31, ql - 1) + (kl - ql) + 1) : kl) : 0;
 
   // batch base: b * batch stride (padded layout) or first-row * row stride (packed layout)
   const int64_t qr = fa.q_row0 ? fa.q_row0[b] : 0, kr = fa.k_row0 ? fa.k_row0[b] : 0;
@@ -106,7 +115,7 @@ __global__ __launch_bounds__(kBlock, 3) void attn_fused_kernel(FusedArgs fa) {
       const int c = slot ^ (DP == 128 ? (rr & 15) : ((rr >> 1) & 7));
       const int qq = q0 + wave * 32 + rr;
       const uint32_t off = (uint32_t)(((int64_t)qq * a.q_ss + c * EPV) * E::kSize);
-      buffer_load16_to_lds(q_desc, lds_address(q_stage) + n * kWave * 16, (qq < ql && c * EPV < a.D) ? off : kOutOfRange);
+      buffer_load16_to_lds(q_desc, lds_address(q_stage) + n * kWave * 16, ((unsigned)qq < (unsigned)ql && c * EPV < a.D) ? off : kOutOfRange);
     }
   }
 
@@ -225,7 +234,7 @@ __global__ __launch_bounds__(kBlock, 3) void attn_fused_kernel(FusedArgs fa) {
       } else {
         // this lane's query and the keys it may see (k < vis_l), counted afresh: only the tiles on the diagonal come here
         const int l = lane_now(), ql_ = q0 + wave * 32 + (l & 31);
-        const int vis_l = (ql_ < ql) ? (a.causal ? min(kl, ql_ + (kl - ql) + 1) : kl) : 0;
+        const int vis_l = ((unsigned)ql_ < (unsigned)ql) ? (a.causal ? min(kl, ql_ + (kl - ql) + 1) : kl) : 0;
         const int lim = vis_l - k0 - 4 * (l >> 5);   // register (kb, x) is visible iff 32kb + 8(x/4) + x%4 < lim
 #pragma unroll
         for (int kb = 0; kb < KB; ++kb)
@@ -337,12 +346,12 @@ __global__ __launch_bounds__(kBlock, 3) void attn_fused_kernel(FusedArgs fa) {
       const int row = i * RPI + lane_e / KVEC_ROW, c = lane_e % KVEC_ROW;
       const uint4 v = *reinterpret_cast<const uint4 *>(stage + row * ROW * E::kSize + ((c ^ (row & (KVEC_ROW - 1))) * 16));
       const int qrow = q0 + wave * 32 + row;
-      if (qrow < ql && c * EPV < a.D) *reinterpret_cast<uint4 *>(cbase + (int64_t)qrow * fa.c_ss + c * EPV) = v;
+      if ((unsigned)qrow < (unsigned)ql && c * EPV < a.D) *reinterpret_cast<uint4 *>(cbase + (int64_t)qrow * fa.c_ss + c * EPV) = v;
     }
     return;
   }
   const int q_e = q0 + wave * 32 + r_e;
-  if (q_e >= ql) return;
+  if ((unsigned)q_e >= (unsigned)ql) return;
   T *crow = cbase + (int64_t)q_e * fa.c_ss;
 #pragma unroll
   for (int mt = 0; mt < DMT; ++mt)
