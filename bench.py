@@ -542,6 +542,23 @@ def kernel_table(torch, K, layer, workloads, w, d, info, steps, step_only=False,
             api["scale_mask_softmax"] = lambda: K.scale_mask_softmax(B, 1, H, probs, info, scale=w.scale, k_seq_len=S,
                                                                      q_len_list=ones)
             api["decode_pv"] = lambda: K.decode_pv(probs, d["v_cache"], info, out=ctx)
+            # the single pass over the same cache contents kept in pages of 64 positions, page ids shuffled over a pool
+            P = 64
+            pages = B * (S // P)
+            perm = torch.randperm(pages, device=d["q"].device)
+            table = perm.view(B, S // P).to(torch.int32).contiguous()
+
+            def paged(cache):
+                pool = torch.empty((pages, H, P, D), dtype=w.dtype, device=cache.device)
+                pool[perm] = cache.view(B, H, S // P, P, D).permute(0, 2, 1, 3, 4).reshape(pages, H, P, D)
+                return pool
+            k_pool, v_pool = paged(d["k_cache"]), paged(d["v_cache"])
+            ctx_paged = K.decode_attn_paged(d["q"], k_pool, v_pool, info, table, scale=w.scale)
+            if not torch.equal(ctx_paged, K.decode_attn(d["q"], d["k_cache"], d["v_cache"], info, scale=w.scale)):
+                raise RuntimeError("decode_attn_paged and decode_attn disagree on the same cache contents")
+            api["decode_attn_paged"] = lambda: K.decode_attn_paged(d["q"], k_pool, v_pool, info, table, scale=w.scale,
+                                                                   out=ctx_paged)
+            alg["decode_attn_paged"] = alg["decode_attn"]
     else:
         T = d["total"]
         # ---- the kernels of the three-kernel form
@@ -631,9 +648,9 @@ def kernel_table(torch, K, layer, workloads, w, d, info, steps, step_only=False,
             ms = _event_time_ms(fn, steps, torch)
             row = {"us": ms * 1e3, "alg_MB": bytes_of[name] / 1e6, "GBps": bytes_of[name] / (ms * 1e-3) / 1e9}
             row["hbm_frac"] = row["GBps"] / HBM_PEAK_GBS
-            if name in ("attn_qk", "attn_pv", "decode_qk", "decode_pv", "decode_attn", "attn_fused", "attn_fused_packed",
-                        "attn_fused_packed_wide"):
-                row["TFLOPs"] = (2 if name.startswith("attn_fused") or name == "decode_attn" else 1) * flops / (ms * 1e-3) / 1e12
+            if name in ("attn_qk", "attn_pv", "decode_qk", "decode_pv", "decode_attn", "decode_attn_paged", "attn_fused",
+                        "attn_fused_packed", "attn_fused_packed_wide"):
+                row["TFLOPs"] = (2 if name.startswith("attn_fused") or name.startswith("decode_attn") else 1) * flops / (ms * 1e-3) / 1e12
                 row["mfma_frac"] = row["TFLOPs"] / MFMA_PEAK_TFLOPS[dt]
             # what a kernel that only moves the bytes reaches in this kernel's access pattern, and this kernel's share of it
             key = YARDSTICK_OF.get(name)
@@ -823,7 +840,7 @@ def stream_yardsticks(torch, iters):
 YARDSTICK_OF = {"depad": "copy", "transpose_pad": "copy", "transpose_pad_valid_rows": "copy", "transpose_depad": "copy",
                 "layernorm_residual": "copy", "scale_mask_softmax": "prefix_inplace",
                 "scale_mask_softmax_no_tail": "prefix_inplace", "attn_qk": "prefix_write", "attn_pv": "prefix_read",
-                "decode_qk": "read", "decode_pv": "read", "decode_attn": "read"}
+                "decode_qk": "read", "decode_pv": "read", "decode_attn": "read", "decode_attn_paged": "read"}
 
 
 def workload_yardsticks(torch, w, d, info, packed_scores):

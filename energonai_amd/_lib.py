@@ -55,6 +55,9 @@ SIGNATURES = {
     "en_decode_pv": (c_int, [c_void_p] * 4 + [c_int] * 4 + [c_int64] * 3 + [c_int, c_void_p]),
     "en_decode_attn": (c_int, [c_void_p] * 5 + [c_int] * 4 + [c_void_p, c_void_p, c_float, c_int, c_void_p, c_int64, c_void_p]),
     "en_decode_attn_workspace_bytes": (c_int64, [c_int] * 4),
+    "en_decode_attn_paged": (c_int, [c_void_p] * 6 + [c_int] * 6 + [c_void_p, c_void_p, c_float, c_int, c_void_p, c_int64, c_void_p]),
+    "en_kv_append_paged": (c_int, [c_void_p] * 6 + [c_int] * 6 + [c_int64, c_int64, c_void_p, c_int, c_void_p, c_void_p]),
+    "en_kv_fill_paged": (c_int, [c_void_p] * 4 + [c_int] * 9 + [c_void_p, c_int, c_void_p, c_void_p]),
     "en_attn_fused": (c_int, [c_void_p] * 6 + [c_int] * 5 + [c_void_p] * 6 + [c_float, c_int, c_int, c_void_p, c_int, c_void_p]),
     "en_padding_removal_layer": (c_int, [c_void_p] * 13 + [c_int] * 4 + [c_int64, c_int64, c_float, c_float] + [c_int] * 3 + [c_void_p, c_int, c_void_p, c_void_p]),
     "en_padding_removal_layer_noalloc": (c_int, [c_void_p] * 7 + [c_int] * 5 + [c_int64, c_int64, c_float, c_float] +

@@ -202,11 +202,21 @@ struct DecodeAttnArgs {
   float c_exp;        // scale * log2(e)
   int nsplit;         // workgroups that share one (batch, head) unit's keys (grid z); 1: none
   float *partial;     // nsplit > 1: [B*H][nsplit][D + 2] unnormalised output, maximum (log2 domain), sum
+  // paged caches: k and v are pools of pages, page p of head h at p * k_sb + h * k_sh (k_sb is the page stride),
+  // position s of sequence b in page page_table[b * max_pages + s / page] at row s % page
+  const int32_t *page_table;
+  int max_pages, lg_page, num_pages;
 };
+
+// Keys of one workgroup when nsplit share a unit: a multiple of 64, so that the keys of one wave (at most 16) never
+// straddle a share or a page.  The combine kernel derives the same shares from the length.
+__device__ __forceinline__ int split_share(int kl, int nsplit) {
+  return nsplit > 1 ? ((kl + nsplit - 1) / nsplit + 63) & ~63 : kl;
+}
 
 constexpr int kRankBatch = 256;
 
-template <int DT, int LPK, bool STREAM, bool BIG>
+template <int DT, int LPK, bool STREAM, bool BIG, bool PAGED = false>
 __global__ __launch_bounds__(BIG ? kStreamBlock : kBlock, 8) void decode_attn_kernel(DecodeAttnArgs a) {
   constexpr int NT = BIG ? kStreamBlock : en::kBlock;
   typedef Elem<DT> E;
@@ -242,12 +252,12 @@ __global__ __launch_bounds__(BIG ? kStreamBlock : kBlock, 8) void decode_attn_ke
   const int kl = max(min(a.kv_lens[b], a.Sk), 0);
   // with the keys of a unit split over nsplit workgroups this one takes [kbeg, kend); a share past the end has no
   // workgroup's worth of work and leaves no partial (the combine kernel derives the same shares from the length)
-  const int share = (kl + a.nsplit - 1) / a.nsplit;
+  const int share = split_share(kl, a.nsplit);
   const int kbeg = (int)blockIdx.z * share, kend = min(kl, kbeg + share);
   if (a.nsplit > 1 && kbeg >= kl) return;
   const T *q = reinterpret_cast<const T *>(a.q) + ((int64_t)b * a.H + h) * a.D;
-  const T *kbase = reinterpret_cast<const T *>(a.k) + (int64_t)b * a.k_sb + (int64_t)h * a.k_sh;
-  const T *vbase = reinterpret_cast<const T *>(a.v) + (int64_t)b * a.v_sb + (int64_t)h * a.v_sh;
+  const T *kbase = reinterpret_cast<const T *>(a.k) + (PAGED ? 0 : (int64_t)b * a.k_sb) + (int64_t)h * a.k_sh;
+  const T *vbase = reinterpret_cast<const T *>(a.v) + (PAGED ? 0 : (int64_t)b * a.v_sb) + (int64_t)h * a.v_sh;
   T *ctx = reinterpret_cast<T *>(a.ctx) + ((int64_t)b * a.H + h) * a.D;
   const bool cv = c * EPV < a.D;     // lanes past the head size idle (head sizes such as 80 and 96)
 
@@ -273,13 +283,41 @@ __global__ __launch_bounds__(BIG ? kStreamBlock : kBlock, 8) void decode_attn_ke
   const uint32_t k_row = (uint32_t)(a.k_ss * E::kSize), v_row = (uint32_t)(a.v_ss * E::kSize);
   const uint32_t col = cv ? (uint32_t)(c * 16) : kOutOfRange;
   constexpr int AUX = STREAM ? 2 : 0;
+  // Paged caches: the keys of one wave (64 / LPK of them, first one a multiple of that) lie in one page, so the
+  // page is a wave-uniform choice of buffer.  Each wave keeps the ids of 64 pages of the sequence in one register,
+  // lane i the id of page tab0 + i, and takes the one it needs with a lane read; the register is filled again when
+  // the walk leaves its range (every 64 pages).  An id outside the pool makes an empty buffer: zeros, no access.
+  constexpr int KPW = kWave / LPK;                   // keys of one wave and step
+  const int wkey = __builtin_amdgcn_readfirstlane(tid / kWave) * KPW;
+  const uint32_t page_mask = PAGED ? (1u << a.lg_page) - 1u : 0u;
+  const uint32_t k_page_bytes = PAGED ? (uint32_t)((((int64_t)page_mask) * a.k_ss + a.D) * E::kSize) : 0u;
+  const uint32_t v_page_bytes = PAGED ? (uint32_t)((((int64_t)page_mask) * a.v_ss + a.D) * E::kSize) : 0u;
+  int tab = -1, tab0 = 0;
+  auto fill_tab = [&](int first_page) {
+    tab0 = first_page;
+    const int pi = first_page + (tid % kWave);
+    tab = pi < a.max_pages ? a.page_table[(int64_t)b * a.max_pages + pi] : -1;
+  };
+  if constexpr (PAGED) fill_tab((kbeg + wkey) >> a.lg_page);
   auto load_stage = [&](uint4 (&kk)[U], uint4 (&vv)[U], int k0) {
 #pragma unroll
     for (int u = 0; u < U; ++u) {
       const int key = k0 + u * G + g;
       const uint32_t in = key < kend ? 0u : kOutOfRange;     // past the end: out of range whatever the stride
-      kk[u] = buffer_load16<AUX>(k_rsrc, (uint32_t)key * k_row + col | in);
-      vv[u] = buffer_load16<AUX>(v_rsrc, (uint32_t)key * v_row + col | in);
+      if constexpr (PAGED) {
+        const int pi = (k0 + u * G + wkey) >> a.lg_page;      // wave-uniform
+        if (pi - tab0 >= kWave) fill_tab(pi);
+        const int id = __builtin_amdgcn_readlane(tab, pi - tab0);
+        const bool ok = (unsigned)id < (unsigned)a.num_pages;
+        const rsrc_t kr = make_rsrc(kbase + (int64_t)id * a.k_sb, ok ? k_page_bytes : 0u);
+        const rsrc_t vr = make_rsrc(vbase + (int64_t)id * a.v_sb, ok ? v_page_bytes : 0u);
+        const uint32_t row = (uint32_t)key & page_mask;
+        kk[u] = buffer_load16<AUX>(kr, row * k_row + col | in);
+        vv[u] = buffer_load16<AUX>(vr, row * v_row + col | in);
+      } else {
+        kk[u] = buffer_load16<AUX>(k_rsrc, (uint32_t)key * k_row + col | in);
+        vv[u] = buffer_load16<AUX>(v_rsrc, (uint32_t)key * v_row + col | in);
+      }
     }
   };
   auto compute_stage = [&](const uint4 (&kk)[U], const uint4 (&vv)[U], int k0) {
@@ -358,7 +396,7 @@ __global__ __launch_bounds__(kBlock) void decode_attn_combine_kernel(DecodeAttnA
   typedef typename E::T T;
   const int unit = blockIdx.x, b = unit / a.H;
   const int kl = max(min(a.kv_lens[b], a.Sk), 0);
-  const int share = (kl + a.nsplit - 1) / a.nsplit;
+  const int share = split_share(kl, a.nsplit);
   const int nvalid = share > 0 ? (kl + share - 1) / share : 0;       // shares that had keys
   const float *part = a.partial + (int64_t)unit * a.nsplit * (a.D + 2);
   T *ctx = reinterpret_cast<T *>(a.ctx) + (int64_t)unit * a.D;
@@ -380,17 +418,17 @@ __global__ __launch_bounds__(kBlock) void decode_attn_combine_kernel(DecodeAttnA
   }
 }
 
-template <int DT, int LPK> struct AttnLauncher {
+template <int DT, int LPK, bool PAGED = false> struct AttnLauncher {
   // stream_cache: caches too large to stay in the memory-side cache between steps are read with non-temporal loads;
   // big: 1024-lane workgroups (large caches, and whenever a unit's keys are split: few units, long rows)
   static void go(const DecodeAttnArgs &a, dim3 grid, bool stream_cache, bool big, hipStream_t s) {
-    if (stream_cache) decode_attn_kernel<DT, LPK, true, true><<<grid, kStreamBlock, 0, s>>>(a);
-    else if (big) decode_attn_kernel<DT, LPK, false, true><<<grid, kStreamBlock, 0, s>>>(a);
-    else decode_attn_kernel<DT, LPK, false, false><<<grid, kBlock, 0, s>>>(a);
+    if (stream_cache) decode_attn_kernel<DT, LPK, true, true, PAGED><<<grid, kStreamBlock, 0, s>>>(a);
+    else if (big) decode_attn_kernel<DT, LPK, false, true, PAGED><<<grid, kStreamBlock, 0, s>>>(a);
+    else decode_attn_kernel<DT, LPK, false, false, PAGED><<<grid, kBlock, 0, s>>>(a);
   }
 };
 
-template <int DT>
+template <int DT, bool PAGED = false>
 static int dispatch_attn(const DecodeAttnArgs &a, bool stream_cache, hipStream_t s) {
   constexpr int EPV = 16 / Elem<DT>::kSize;
   int lpk = 4;
@@ -398,11 +436,11 @@ static int dispatch_attn(const DecodeAttnArgs &a, bool stream_cache, hipStream_t
   dim3 grid((unsigned)a.H, (unsigned)a.B, (unsigned)a.nsplit);
   const bool big = stream_cache || a.nsplit > 1;
   switch (lpk) {
-    case 4: AttnLauncher<DT, 4>::go(a, grid, stream_cache, big, s); break;
-    case 8: AttnLauncher<DT, 8>::go(a, grid, stream_cache, big, s); break;
-    case 16: AttnLauncher<DT, 16>::go(a, grid, stream_cache, big, s); break;
-    case 32: AttnLauncher<DT, 32>::go(a, grid, stream_cache, big, s); break;
-    case 64: AttnLauncher<DT, 64>::go(a, grid, stream_cache, big, s); break;
+    case 4: AttnLauncher<DT, 4, PAGED>::go(a, grid, stream_cache, big, s); break;
+    case 8: AttnLauncher<DT, 8, PAGED>::go(a, grid, stream_cache, big, s); break;
+    case 16: AttnLauncher<DT, 16, PAGED>::go(a, grid, stream_cache, big, s); break;
+    case 32: AttnLauncher<DT, 32, PAGED>::go(a, grid, stream_cache, big, s); break;
+    case 64: AttnLauncher<DT, 64, PAGED>::go(a, grid, stream_cache, big, s); break;
     default: return EN_ERR_UNSUPPORTED;
   }
   EN_RETURN_IF_LAUNCH_FAILED();
@@ -453,6 +491,81 @@ __global__ __launch_bounds__(kWave) void kv_append_kernel(AppendArgs a) {
     *reinterpret_cast<Vec *>(a.k_cache + dst + i) = *reinterpret_cast<const Vec *>(a.k_new + src + i);
     *reinterpret_cast<Vec *>(a.v_cache + dst + i) = *reinterpret_cast<const Vec *>(a.v_new + src + i);
   }
+}
+
+
+// Paged caches: the same append, the row found through the page table.  A sequence whose next position has no page
+// (position past max_pages * page, id outside the pool) is left alone and counted.
+struct PagedAppendArgs {
+  const unsigned char *k_new, *v_new;
+  unsigned char *k_pool, *v_pool;
+  const int32_t *kv_lens, *page_table;
+  int H, max_pages, lg_page, num_pages;
+  int row_bytes;
+  int64_t n_sb, n_sh;           // strides of the new rows, bytes
+  int64_t p_sp, p_sh, p_ss;     // page, head and row strides of the pools, bytes
+  int32_t *overflow;
+};
+
+__global__ __launch_bounds__(kWave) void kv_append_paged_kernel(PagedAppendArgs a) {
+  const int h = blockIdx.x, b = blockIdx.y;
+  const int pos = a.kv_lens[b];
+  const int pi = pos >> a.lg_page;
+  const int id = (pos >= 0 && pi < a.max_pages) ? a.page_table[(int64_t)b * a.max_pages + pi] : -1;
+  if ((unsigned)id >= (unsigned)a.num_pages) {
+    if (a.overflow && h == 0 && threadIdx.x == 0) atomicAdd(a.overflow, 1);
+    return;
+  }
+  const int64_t src = (int64_t)b * a.n_sb + (int64_t)h * a.n_sh;
+  const int64_t dst = (int64_t)id * a.p_sp + (int64_t)h * a.p_sh + (int64_t)(pos & ((1 << a.lg_page) - 1)) * a.p_ss;
+  for (int i = threadIdx.x * 16; i < a.row_bytes; i += kWave * 16) {
+    *reinterpret_cast<uint4 *>(a.k_pool + dst + i) = *reinterpret_cast<const uint4 *>(a.k_new + src + i);
+    *reinterpret_cast<uint4 *>(a.v_pool + dst + i) = *reinterpret_cast<const uint4 *>(a.v_new + src + i);
+  }
+}
+
+// Prefill into pages: the rows of sequence b, packed tokens cu[b] .. of a [T, src_head_rows, D] source of which heads
+// src_head_first .. + H - 1 are taken, go to rows 0 .. len - 1 of the sequence's pages.
+struct PagedFillArgs {
+  const unsigned char *src;
+  unsigned char *pool;
+  const int32_t *cu, *page_table;
+  int H, S, max_pages, lg_page, num_pages;
+  int vecs_per_row;             // 16-byte vectors per head row
+  int64_t s_row, s_head;        // source: bytes per token, bytes per head row
+  int64_t head_first_bytes;
+  int64_t p_sp, p_sh, p_ss;
+  int32_t *overflow;
+};
+
+__global__ __launch_bounds__(kBlock) void kv_fill_paged_kernel(PagedFillArgs a) {
+  constexpr int ROWS = 4;
+  const int b = blockIdx.y;
+  const int t0 = a.cu[b], len = min(a.cu[b + 1] - t0, a.S);
+  const int per_row = a.H * a.vecs_per_row;
+  for (int r = 0; r < ROWS; ++r) {
+    const int s = blockIdx.x * ROWS + r;
+    if (s >= len) return;
+    const int pi = s >> a.lg_page;
+    const int id = pi < a.max_pages ? a.page_table[(int64_t)b * a.max_pages + pi] : -1;
+    if ((unsigned)id >= (unsigned)a.num_pages) {
+      if (a.overflow && threadIdx.x == 0) atomicAdd(a.overflow, 1);
+      continue;
+    }
+    const unsigned char *src = a.src + (int64_t)(t0 + s) * a.s_row + a.head_first_bytes;
+    unsigned char *dst = a.pool + (int64_t)id * a.p_sp + (int64_t)(s & ((1 << a.lg_page) - 1)) * a.p_ss;
+    for (int i = threadIdx.x; i < per_row; i += kBlock) {
+      const int h = i / a.vecs_per_row, c = i - h * a.vecs_per_row;
+      *reinterpret_cast<uint4 *>(dst + (int64_t)h * a.p_sh + c * 16) =
+          *reinterpret_cast<const uint4 *>(src + (int64_t)h * a.s_head + c * 16);
+    }
+  }
+}
+
+static int log2_exact(int v) {
+  int lg = 0;
+  while ((1 << lg) < v) ++lg;
+  return (1 << lg) == v ? lg : -1;
 }
 
 }  // namespace en
@@ -532,6 +645,100 @@ int en_decode_attn(const void *q, const void *k_cache, const void *v_cache, void
     case EN_F32: return dispatch_attn<EN_F32>(a, stream_cache, s);
     case EN_F16: return dispatch_attn<EN_F16>(a, stream_cache, s);
     default: return dispatch_attn<EN_BF16>(a, stream_cache, s);
+  }
+}
+
+int en_kv_append_paged(const void *k_new, const void *v_new, void *k_pool, void *v_pool, const int32_t *kv_lens,
+                       const int32_t *page_table, int batch, int head_num, int max_pages_per_seq, int page_size,
+                       int num_pages, int size_per_head, int64_t new_stride_b, int64_t new_stride_h,
+                       const int64_t *pool_strides, int elem_size, int32_t *overflow, en_stream_t stream) {
+  using namespace en;
+  if (!k_new || !v_new || !k_pool || !v_pool || !kv_lens || !page_table || !pool_strides) return EN_ERR_NULL;
+  if (overflow && !aligned_to(overflow, 4)) return EN_ERR_ALIGN;
+  if (elem_size != 2 && elem_size != 4) return EN_ERR_DTYPE;
+  if (batch < 1 || batch > 65535 || head_num < 1 || max_pages_per_seq < 1 || num_pages < 1 || size_per_head < 1) return EN_ERR_SHAPE;
+  const int lg = log2_exact(page_size);
+  if (lg < 4) return EN_ERR_UNSUPPORTED;                                  // a power of two, at least 16
+  if ((int64_t)max_pages_per_seq * page_size >= (1ll << 31)) return EN_ERR_SHAPE;
+  if (new_stride_b < 0 || new_stride_h < 0 || pool_strides[0] < 0 || pool_strides[1] < 0 || pool_strides[2] < 0)
+    return EN_ERR_UNSUPPORTED;
+  PagedAppendArgs a{(const unsigned char *)k_new, (const unsigned char *)v_new, (unsigned char *)k_pool,
+                    (unsigned char *)v_pool, kv_lens, page_table, head_num, max_pages_per_seq, lg, num_pages,
+                    size_per_head * elem_size, new_stride_b * elem_size, new_stride_h * elem_size,
+                    pool_strides[0] * elem_size, pool_strides[1] * elem_size, pool_strides[2] * elem_size, overflow};
+  if ((a.row_bytes % 16) || !aligned_to(k_new, 16) || !aligned_to(v_new, 16) || !aligned_to(k_pool, 16) ||
+      !aligned_to(v_pool, 16) || (a.n_sb % 16) || (a.n_sh % 16) || (a.p_sp % 16) || (a.p_sh % 16) || (a.p_ss % 16))
+    return EN_ERR_ALIGN;
+  kv_append_paged_kernel<<<dim3((unsigned)head_num, (unsigned)batch, 1), kWave, 0, (hipStream_t)stream>>>(a);
+  EN_RETURN_IF_LAUNCH_FAILED();
+  return EN_OK;
+}
+
+int en_kv_fill_paged(const void *src, void *pool, const int32_t *cu_seqlens, const int32_t *page_table, int batch,
+                     int max_seq_len, int head_num, int size_per_head, int src_head_rows, int src_head_first,
+                     int max_pages_per_seq, int page_size, int num_pages, const int64_t *pool_strides, int elem_size,
+                     int32_t *overflow, en_stream_t stream) {
+  using namespace en;
+  if (!src || !pool || !cu_seqlens || !page_table || !pool_strides) return EN_ERR_NULL;
+  if (overflow && !aligned_to(overflow, 4)) return EN_ERR_ALIGN;
+  if (elem_size != 2 && elem_size != 4) return EN_ERR_DTYPE;
+  if (batch < 1 || batch > 65535 || max_seq_len < 1 || head_num < 1 || size_per_head < 1 || max_pages_per_seq < 1 ||
+      num_pages < 1)
+    return EN_ERR_SHAPE;
+  if (src_head_first < 0 || src_head_rows < src_head_first + head_num) return EN_ERR_SHAPE;
+  const int lg = log2_exact(page_size);
+  if (lg < 4) return EN_ERR_UNSUPPORTED;
+  if ((int64_t)max_pages_per_seq * page_size >= (1ll << 31)) return EN_ERR_SHAPE;
+  if (pool_strides[0] < 0 || pool_strides[1] < 0 || pool_strides[2] < 0) return EN_ERR_UNSUPPORTED;
+  const int64_t row_bytes = (int64_t)size_per_head * elem_size;
+  PagedFillArgs a{(const unsigned char *)src, (unsigned char *)pool, cu_seqlens, page_table, head_num, max_seq_len,
+                  max_pages_per_seq, lg, num_pages, (int)(row_bytes / 16), (int64_t)src_head_rows * row_bytes, row_bytes,
+                  (int64_t)src_head_first * row_bytes, pool_strides[0] * elem_size, pool_strides[1] * elem_size,
+                  pool_strides[2] * elem_size, overflow};
+  if ((row_bytes % 16) || !aligned_to(src, 16) || !aligned_to(pool, 16) || (a.p_sp % 16) || (a.p_sh % 16) || (a.p_ss % 16))
+    return EN_ERR_ALIGN;
+  const dim3 grid((unsigned)ceil_div(max_seq_len, 4), (unsigned)batch, 1);
+  kv_fill_paged_kernel<<<grid, kBlock, 0, (hipStream_t)stream>>>(a);
+  EN_RETURN_IF_LAUNCH_FAILED();
+  return EN_OK;
+}
+
+int en_decode_attn_paged(const void *q, const void *k_pool, const void *v_pool, void *ctx, const int32_t *kv_lens,
+                         const int32_t *page_table, int batch, int head_num, int max_pages_per_seq, int page_size,
+                         int num_pages, int size_per_head, const int64_t *k_strides, const int64_t *v_strides, float scale,
+                         int dtype, void *workspace, int64_t workspace_bytes, en_stream_t stream) {
+  using namespace en;
+  if (!k_strides || !v_strides || !v_pool || !page_table) return EN_ERR_NULL;
+  if (max_pages_per_seq < 1 || num_pages < 1) return EN_ERR_SHAPE;
+  const int lg = log2_exact(page_size);
+  if (lg < 4) return EN_ERR_UNSUPPORTED;                                  // a power of two, at least 16: a wave's keys share a page
+  if ((int64_t)max_pages_per_seq * page_size >= (1ll << 30)) return EN_ERR_SHAPE;
+  const int k_seq_len = max_pages_per_seq * page_size;
+  int rc = check_decode(q, k_pool, ctx, kv_lens, batch, head_num, k_seq_len, size_per_head, k_strides[0], k_strides[1],
+                        k_strides[2], dtype);
+  if (rc) return rc;
+  const int es = dtype_size(dtype), epv = 16 / es;
+  if (!aligned_to(v_pool, 16) || (v_strides[0] % epv) || (v_strides[1] % epv) || (v_strides[2] % epv)) return EN_ERR_ALIGN;
+  if (!aligned_to(q, 16) || !aligned_to(ctx, es)) return EN_ERR_ALIGN;
+  if (size_per_head > 64 * epv) return EN_ERR_UNSUPPORTED;
+  // 32-bit byte offsets inside a page
+  if ((int64_t)page_size * k_strides[2] * es >= (1ll << 31) || (int64_t)page_size * v_strides[2] * es >= (1ll << 31))
+    return EN_ERR_UNSUPPORTED;
+  if (!(scale > 0.f)) return EN_ERR_UNSUPPORTED;
+  for (int i = 0; i < 3; ++i)
+    if (k_strides[i] < 0 || v_strides[i] < 0) return EN_ERR_UNSUPPORTED;
+  const int64_t need = en_decode_attn_workspace_bytes(batch, head_num, k_seq_len, size_per_head);
+  const bool split = need > 0 && workspace && workspace_bytes >= need && aligned_to(workspace, 4);
+  DecodeAttnArgs a{q, k_pool, v_pool, ctx, kv_lens, batch, head_num, k_seq_len, size_per_head, k_strides[0], k_strides[1],
+                   k_strides[2], v_strides[0], v_strides[1], v_strides[2], scale * 1.4426950408889634f,
+                   split ? decode_split(batch, head_num, k_seq_len) : 1, static_cast<float *>(workspace),
+                   page_table, max_pages_per_seq, lg, num_pages};
+  const bool stream_cache = 2 * cache_bytes(batch, head_num, k_seq_len, size_per_head, dtype) >= kStreamCacheBytes;
+  hipStream_t s = (hipStream_t)stream;
+  switch (dtype) {
+    case EN_F32: return dispatch_attn<EN_F32, true>(a, stream_cache, s);
+    case EN_F16: return dispatch_attn<EN_F16, true>(a, stream_cache, s);
+    default: return dispatch_attn<EN_BF16, true>(a, stream_cache, s);
   }
 }
 

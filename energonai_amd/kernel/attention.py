@@ -344,6 +344,117 @@ def kv_cache_append(k_new, v_new, k_cache, v_cache, kv_len_list, overflow: Optio
                    "kv_cache_append")
 
 
+def _pool(t, name: str):
+    """Strides (page, head, row) in elements of a ``[pages, H, page_size, D]`` pool with contiguous channels."""
+    _lib.require_gpu(t, name, contiguous=False)
+    if t.dim() != 4 or t.stride(3) != 1:
+        raise RuntimeError(f"{name} must be a [pages, H, page_size, D] tensor with contiguous channels")
+    return (t.stride(0), t.stride(1), t.stride(2))
+
+
+def _page_table(page_table, batch: int, name: str):
+    _lib.require_gpu(page_table, "page_table")
+    if page_table.dim() != 2 or page_table.shape[0] != batch or page_table.dtype != torch.int32:
+        raise RuntimeError(f"{name}: page_table must be a contiguous int32 [batch, max_pages_per_seq] tensor")
+    return int(page_table.shape[1])
+
+
+def _overflow(overflow, name: str):
+    if overflow is not None:
+        _lib.require_gpu(overflow, "overflow")
+        if overflow.dtype != torch.int32 or overflow.numel() < 1:
+            raise RuntimeError(f"{name}: overflow must be an int32 tensor of at least one element")
+
+
+def kv_pages_fill(src, pool, batch_size: int, max_seq_len: int, seq_len_list, page_table, head_first: int = 0,
+                  overflow: Optional[torch.Tensor] = None):
+    """Prefill of a paged cache: ``pool[page_table[b, s // P], h, s % P, :] = src[cu[b]+s, head_first+h, :]`` for
+    ``s < len[b]``; ``src`` is the packed projection output seen as ``[T,Hs,D]`` (as ``kv_cache_fill``), ``pool`` is
+    ``[pages, H, P, D]``.  A row whose page id lies outside the pool is not written and counted in ``overflow``."""
+    _lib.require_gpu(src, "src")
+    ps = _pool(pool, "pool")
+    if src.dim() != 3 or pool.shape[3] != src.shape[2] or pool.dtype != src.dtype:
+        raise RuntimeError("kv_pages_fill: src must be [T,Hs,D] and pool [pages,H,P,D] of one dtype")
+    N, H, P, D = pool.shape
+    max_pages = _page_table(page_table, batch_size, "kv_pages_fill")
+    _overflow(overflow, "kv_pages_fill")
+    info = seq_info(seq_len_list, batch_size, src.device)
+    arr = ctypes.c_int64 * 3
+    with _lib.device_guard(src):
+        _lib.check(_lib.fn.en_kv_fill_paged(src.data_ptr(), pool.data_ptr(), info.cu_seqlens.data_ptr(),
+                                            page_table.data_ptr(), int(batch_size), int(max_seq_len), H, D, src.shape[1],
+                                            int(head_first), max_pages, P, N, arr(*ps), src.element_size(),
+                                            _lib.ptr(overflow), _lib.stream_of(src)), "kv_pages_fill")
+    return pool
+
+
+def kv_pages_append(k_new, v_new, k_pool, v_pool, kv_len_list, page_table, overflow: Optional[torch.Tensor] = None):
+    """``kv_cache_append`` for paged caches: the new ``[B,H,D]`` rows go to row ``kv_len[b] % P`` of page
+    ``page_table[b, kv_len[b] // P]``.  A sequence whose next position has no page in the pool keeps its rows, loses
+    the new one and is counted in ``overflow``."""
+    for t, n in ((k_new, "k_new"), (v_new, "v_new")):
+        _lib.require_gpu(t, n, contiguous=False)
+        if t.dim() != 3 or t.stride(2) != 1:
+            raise RuntimeError(f"kv_pages_append: {n} must be a [B,H,D] view with contiguous channels")
+    ps = _pool(k_pool, "k_pool")
+    if _pool(v_pool, "v_pool") != ps or k_new.stride() != v_new.stride() or k_pool.shape != v_pool.shape:
+        raise RuntimeError("kv_pages_append: K and V must share shapes and strides")
+    N, H, P, D = k_pool.shape
+    B = k_new.shape[0]
+    if k_new.shape != (B, H, D) or v_new.shape != (B, H, D) or k_new.dtype != k_pool.dtype:
+        raise RuntimeError("kv_pages_append: new rows must be [B,H,D] of the pool dtype")
+    max_pages = _page_table(page_table, B, "kv_pages_append")
+    _overflow(overflow, "kv_pages_append")
+    info = seq_info(kv_len_list, B, k_pool.device)
+    arr = ctypes.c_int64 * 3
+    with _lib.device_guard(k_pool):
+        _lib.check(_lib.fn.en_kv_append_paged(k_new.data_ptr(), v_new.data_ptr(), k_pool.data_ptr(), v_pool.data_ptr(),
+                                              info.lens.data_ptr(), page_table.data_ptr(), B, H, max_pages, P, N, D,
+                                              k_new.stride(0), k_new.stride(1), arr(*ps), k_pool.element_size(),
+                                              _lib.ptr(overflow), _lib.stream_of(k_pool)), "kv_pages_append")
+
+
+def decode_attn_paged(q, k_pool, v_pool, kv_len_list, page_table, *, scale: Optional[float] = None,
+                      out: Optional[torch.Tensor] = None, workspace: Optional[torch.Tensor] = None, split: bool = True):
+    """``decode_attn`` over paged caches: position ``j`` of sequence ``b`` is row ``j % P`` of page
+    ``page_table[b, j // P]`` of the ``[pages, H, P, D]`` pools (``P`` a power of two, at least 16).  ``[B,H,1,D]``.
+    A page id outside the pool reads as zeros."""
+    _lib.require_gpu(q, "q", contiguous=False)
+    ks = _pool(k_pool, "k_pool")
+    vs = _pool(v_pool, "v_pool")
+    N, H, P, D = k_pool.shape
+    if v_pool.shape != k_pool.shape or v_pool.dtype != k_pool.dtype:
+        raise RuntimeError("decode_attn_paged: k_pool and v_pool must share shape and dtype")
+    if q.dim() < 2 or q.numel() % (H * D) != 0 or q.dtype != k_pool.dtype:
+        raise RuntimeError("decode_attn_paged: q must be [B,H,1,D] of the pools' dtype")
+    B = q.numel() // (H * D)
+    max_pages = _page_table(page_table, B, "decode_attn_paged")
+    q_ = q.reshape(B, H, D).contiguous()
+    info = seq_info(kv_len_list, B, q.device)
+    if out is None:
+        out = torch.empty((B, H, 1, D), dtype=q.dtype, device=q.device)
+    else:
+        _lib.require_gpu(out, "out")
+        if out.numel() != B * H * D or out.dtype != q.dtype:
+            raise RuntimeError("decode_attn_paged: out must be a contiguous [B,H,1,D] tensor of q's dtype")
+    arr = ctypes.c_int64 * 3
+    scale = float(D) ** -0.5 if scale is None else float(scale)
+    need = decode_attn_workspace_bytes(B, H, max_pages * P, D) if split else 0
+    if need and workspace is None:
+        workspace = torch.empty(need, dtype=torch.uint8, device=q.device)
+    ws_bytes = 0
+    if workspace is not None and need:
+        _lib.require_gpu(workspace, "workspace")
+        ws_bytes = workspace.numel() * workspace.element_size()
+    with _lib.device_guard(q):
+        _lib.check(_lib.fn.en_decode_attn_paged(q_.data_ptr(), k_pool.data_ptr(), v_pool.data_ptr(), out.data_ptr(),
+                                                info.lens.data_ptr(), page_table.data_ptr(), B, H, max_pages, P, N, D,
+                                                arr(*ks), arr(*vs), scale, _lib.dtype_tag(q, "decode_attn_paged"),
+                                                _lib.ptr(workspace) if ws_bytes else None, ws_bytes,
+                                                _lib.stream_of(q)), "decode_attn_paged")
+    return out
+
+
 def decode_qk(q, k_cache, kv_len_list, *, alpha: float = 1.0, out: Optional[torch.Tensor] = None):
     """scores[b,h,0,j] = alpha * <q[b,h,0,:], k_cache[b,h,j,:]> for j < kv_len[b]; ``[B,H,1,Smax]``."""
     _lib.require_gpu(q, "q", contiguous=False)

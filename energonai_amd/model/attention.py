@@ -19,7 +19,7 @@ from ..kernel import (attn_fused_varlen, attn_pv, attn_qk, decode_attn, decode_p
 from ..kernel.attention import kv_cache_fill
 from ..seqinfo import SeqInfo, seq_info
 from .gemm import project
-from .kv_cache import KVCache, OutputHistory
+from .kv_cache import KVCache, OutputHistory, PagedKVCache
 
 
 def lens_from_mask(attention_mask: torch.Tensor) -> torch.Tensor:
@@ -32,7 +32,8 @@ def lens_from_mask(attention_mask: torch.Tensor) -> torch.Tensor:
 class MultiHeadAttention1D(nn.Module):
     def __init__(self, hidden_size: int, num_heads: int, bias: bool = True, dtype: torch.dtype = torch.float16,
                  max_seq_len: int = 512, fused_qkv: bool = True, is_decoder: bool = True, disable_past_cache=False,
-                 left_padded: Optional[bool] = None) -> None:
+                 left_padded: Optional[bool] = None, kv_page_size: Optional[int] = None,
+                 kv_pool_pages: Optional[int] = None) -> None:
         super().__init__()
         if hidden_size % num_heads != 0:
             raise ValueError(f"{hidden_size} is not divisible by {num_heads}")
@@ -53,7 +54,10 @@ class MultiHeadAttention1D(nn.Module):
             self.key_ = nn.Linear(hidden_size, hidden_size, bias=bias, dtype=dtype)
             self.value_ = nn.Linear(hidden_size, hidden_size, bias=bias, dtype=dtype)
         self.dense = nn.Linear(hidden_size, hidden_size, bias=True, dtype=dtype)
-        self.kv_cache: Optional[KVCache] = None
+        # None: one [B,H,max_seq_len,D] buffer per cache; a page size: pages of a pool (PagedKVCache)
+        self.kv_page_size = kv_page_size
+        self.kv_pool_pages = kv_pool_pages
+        self.kv_cache = None
         self._history = OutputHistory()     # what the reference keeps in past_cache['dense']
 
     # ---- projections: packed rows in, [rows, H, D] views of q, k, v out --------------------
@@ -94,7 +98,11 @@ class MultiHeadAttention1D(nn.Module):
             if max_seq_len > self.max_seq_len:
                 raise RuntimeError(f"the batch is padded to {max_seq_len} positions but the K/V cache was planned for "
                                    f"max_seq_len = {self.max_seq_len}")
-            self.kv_cache = KVCache(batch_size, H, self.max_seq_len, D, x.dtype, x.device)
+            if self.kv_page_size:
+                self.kv_cache = PagedKVCache(batch_size, H, self.max_seq_len, D, x.dtype, x.device,
+                                             page_size=self.kv_page_size, pool_pages=self.kv_pool_pages)
+            else:
+                self.kv_cache = KVCache(batch_size, H, self.max_seq_len, D, x.dtype, x.device)
             if kvq is not None:
                 self.kv_cache.fill(kvq, kvq, info, 0, H, longest=max_seq_len)
             else:
@@ -111,7 +119,7 @@ class MultiHeadAttention1D(nn.Module):
         cache = self.kv_cache
         q, k, v, _ = self._project(last)
         cache.append(k, v)
-        ctx = decode_attn(q, cache.k, cache.v, cache.info, scale=self.scaling)      # [B,H,1,D], one pass over the caches
+        ctx = cache.attend(q, self.scaling)      # [B,H,1,D], one pass over the caches
         return project(self.dense, ctx.view(B, 1, self.hidden_size))
 
     def forward(self, hidden_states, attention_mask=None, first_cache=False, seq_lens=None):

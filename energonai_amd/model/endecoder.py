@@ -5,7 +5,7 @@ LayerNorm is fused into that LayerNorm.
 """
 from __future__ import annotations
 
-from typing import Callable
+from typing import Callable, Optional
 
 import torch
 from torch import nn
@@ -21,14 +21,16 @@ class Block1D(nn.Module):
     def __init__(self, hidden_size: int, num_heads: int, mlp_ratio: float, activation: Callable = nn.functional.gelu,
                  layernorm_epsilon: float = 1e-5, dtype: torch.dtype = torch.float16, bias: bool = True,
                  apply_post_layernorm: bool = False, max_seq_len: int = 512, fused_qkv: bool = True,
-                 is_decoder: bool = True, disable_past_cache=False) -> None:
+                 is_decoder: bool = True, disable_past_cache=False, kv_page_size: Optional[int] = None,
+                 kv_pool_pages: Optional[int] = None) -> None:
         super().__init__()
         self.apply_post_layernorm = apply_post_layernorm
         self.disable_past_cache = disable_past_cache
         self.norm1 = LayerNorm(hidden_size, eps=layernorm_epsilon, dtype=dtype)
         self.attn = MultiHeadAttention1D(hidden_size=hidden_size, num_heads=num_heads, bias=bias, dtype=dtype,
                                          max_seq_len=max_seq_len, fused_qkv=fused_qkv, is_decoder=is_decoder,
-                                         disable_past_cache=disable_past_cache)
+                                         disable_past_cache=disable_past_cache, kv_page_size=kv_page_size,
+                                         kv_pool_pages=kv_pool_pages)
         self.norm2 = LayerNorm(hidden_size, eps=layernorm_epsilon, dtype=dtype)
         self.mlp = MLP1D(hidden_size=hidden_size, mlp_ratio=mlp_ratio, activation=activation, dtype=dtype, bias=bias,
                          disable_past_cache=disable_past_cache)

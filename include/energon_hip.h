@@ -276,6 +276,34 @@ int en_kv_append(const void *k_new, const void *v_new, void *k_cache, void *v_ca
                  int64_t new_stride_h, int64_t cache_stride_b, int64_t cache_stride_h, int64_t cache_stride_s,
                  int elem_size, int32_t *overflow, en_stream_t stream);
 
+/* The K/V cache in pages (a further form of the cache that replaces the reference's concatenated history,
+ * energonai/model/attention.py:61-71,89-98; the reference has no counterpart): K and V live in pools of
+ * num_pages pages of page_size positions (a power of two, at least 16), page p, head h, row r, channel d at
+ * p*strides[0] + h*strides[1] + r*strides[2] + d elements, e.g. a contiguous [num_pages, H, page_size, D] tensor.
+ * page_table (device, int32 [batch, max_pages_per_seq]) names the pages of each sequence in order: position s of
+ * sequence b is row s % page_size of page page_table[b][s / page_size].  Entries past a sequence's last page are
+ * never followed; an id outside 0 .. num_pages-1 that a kernel does meet reads as zeros (attention) or leaves the
+ * row unwritten and is counted in overflow (append, fill), so a wrong table cannot fault.  Sequences share the
+ * pools, so memory is held for the positions in use, rounded up to pages, instead of batch * Smax.
+ *   en_kv_fill_paged    prefill: rows cu_seqlens[b] .. of a packed [T, src_head_rows, D] source (heads
+ *                       src_head_first .. +head_num-1, as en_transpose_pad_heads) to positions 0 .. len-1
+ *   en_kv_append_paged  one new row per (batch, head) at position kv_lens[b], as en_kv_append
+ *   en_decode_attn_paged  en_decode_attn over the pages (same kernel, the page a wave-uniform choice of buffer);
+ *                       workspace as there, sized by en_decode_attn_workspace_bytes(batch, head_num,
+ *                       max_pages_per_seq * page_size, size_per_head) */
+int en_kv_fill_paged(const void *src, void *pool, const int32_t *cu_seqlens, const int32_t *page_table, int batch,
+                     int max_seq_len, int head_num, int size_per_head, int src_head_rows, int src_head_first,
+                     int max_pages_per_seq, int page_size, int num_pages, const int64_t *pool_strides, int elem_size,
+                     int32_t *overflow, en_stream_t stream);
+int en_kv_append_paged(const void *k_new, const void *v_new, void *k_pool, void *v_pool, const int32_t *kv_lens,
+                       const int32_t *page_table, int batch, int head_num, int max_pages_per_seq, int page_size,
+                       int num_pages, int size_per_head, int64_t new_stride_b, int64_t new_stride_h,
+                       const int64_t *pool_strides, int elem_size, int32_t *overflow, en_stream_t stream);
+int en_decode_attn_paged(const void *q, const void *k_pool, const void *v_pool, void *ctx, const int32_t *kv_lens,
+                         const int32_t *page_table, int batch, int head_num, int max_pages_per_seq, int page_size,
+                         int num_pages, int size_per_head, const int64_t *k_strides, const int64_t *v_strides, float scale,
+                         int dtype, void *workspace, int64_t workspace_bytes, en_stream_t stream);
+
 /* Fused attention (an addition: the reference callers run matmul, softmax, matmul,
  * examples/bert/bert.py:108-119): ctx[b,h,i,:] = sum_j softmax_j(scale * <q_i, k_j>) v[b,h,j,:]
  * over the keys row i may see (same rule as en_scale_mask_softmax), without ever

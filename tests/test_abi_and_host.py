@@ -102,6 +102,18 @@ def test_entry_points_validate_before_launch():
     assert lib.en_decode_attn(16, 32, 48, 64, 80, 1, 1, 8, 64, i64x3, i64x3, 0.0, 1, None, 0, None) == -5      # scale must be positive
     assert lib.en_decode_attn(16, 32, 48, 64, 80, 1, 1, 8, 60, i64x3, i64x3, 1.0, 1, None, 0, None) == -5      # D not a multiple of 8
     assert lib.en_decode_attn(16, 32, 48, 64, 80, 1, 1, 2 ** 24, 64, i64x3, i64x3, 1.0, 1, None, 0, None) == -5   # 32-bit offsets inside a unit
+    # paged caches: q, k_pool, v_pool, ctx, lens, table, batch, heads, max_pages, page, num_pages, D, ...
+    assert lib.en_decode_attn_paged(16, 32, 48, 64, 80, None, 1, 1, 4, 64, 8, 64, i64x3, i64x3, 1.0, 1, None, 0, None) == -1   # no table
+    assert lib.en_decode_attn_paged(16, 32, 48, 64, 80, 96, 1, 1, 4, 48, 8, 64, i64x3, i64x3, 1.0, 1, None, 0, None) == -5    # page not a power of two
+    assert lib.en_decode_attn_paged(16, 32, 48, 64, 80, 96, 1, 1, 4, 8, 8, 64, i64x3, i64x3, 1.0, 1, None, 0, None) == -5     # page below 16
+    assert lib.en_decode_attn_paged(16, 32, 48, 64, 80, 96, 1, 1, 0, 64, 8, 64, i64x3, i64x3, 1.0, 1, None, 0, None) == -2    # no pages per sequence
+    assert lib.en_decode_attn_paged(16, 32, 48, 64, 80, 96, 1, 1, 4, 64, 8, 64, i64x3, i64x3, -1.0, 1, None, 0, None) == -5   # scale must be positive
+    assert lib.en_kv_append_paged(16, 32, 48, 64, 80, None, 1, 1, 4, 64, 8, 64, 64, 64, i64x3, 2, None, None) == -1            # no table
+    assert lib.en_kv_append_paged(16, 32, 48, 64, 80, 96, 1, 1, 4, 24, 8, 64, 64, 64, i64x3, 2, None, None) == -5              # page not a power of two
+    assert lib.en_kv_append_paged(16, 32, 48, 64, 80, 96, 1, 1, 4, 64, 8, 60, 64, 64, i64x3, 2, None, None) == -4              # rows of 120 bytes
+    assert lib.en_kv_fill_paged(16, 32, 48, None, 1, 8, 1, 64, 3, 0, 4, 64, 8, i64x3, 2, None, None) == -1                     # no table
+    assert lib.en_kv_fill_paged(16, 32, 48, 64, 1, 8, 4, 64, 6, 4, 4, 64, 8, i64x3, 2, None, None) == -2                       # heads 4..7 of a 6-row source
+    assert lib.en_kv_fill_paged(16, 32, 48, 64, 1, 8, 1, 64, 3, 0, 4, 64, 8, i64x3, 3, None, None) == -3                       # element size 3
     assert lib.en_decode_attn_workspace_bytes(64, 72, 2048, 128) == 0          # 4608 units fill the chip
     assert lib.en_decode_attn_workspace_bytes(1, 72, 2048, 128) == 72 * 4 * 130 * 4   # 72 units: four shares of 512 keys each
     assert lib.en_decode_attn_workspace_bytes(4, 72, 300, 128) == 0            # short caches are not shared
@@ -274,3 +286,30 @@ def test_workload_definitions():
     assert alg["layernorm_residual"] == 3 * 698 * 768 * 4
     vis = sum(n * n for n in inp["lens_list"])
     assert wl.algorithmic_flops(w, inp["lens_list"]) == 2.0 * 12 * 64 * vis
+
+
+def test_paged_cache_bookkeeping_on_the_host():
+    """Which pages a sequence holds is decided on the host: pages are taken at prefill and at page boundaries,
+    handed back on release, and an exhausted pool or a full table row raises before any kernel runs."""
+    import torch
+    from energonai_amd.model.kv_cache import PagedKVCache
+    c = PagedKVCache(3, 2, 64, 16, torch.float16, "cpu", page_size=16, pool_pages=7)
+    assert c.max_pages == 4 and c.max_seq_len == 64 and c.pages_in_use() == 0
+    c._assign([(0, 2), (1, 1), (2, 3)])
+    assert c.pages_in_use() == 6
+    t = c.table.tolist()
+    held = [p for row in t for p in row if p >= 0]
+    assert len(held) == 6 and len(set(held)) == 6 and all(0 <= p < 7 for p in held)
+    assert [sum(p >= 0 for p in row) for row in t] == [2, 1, 3]
+    assert t[0][2] == -1 and t[1][1] == -1
+    c._assign([(1, 2)])
+    assert c.pages_in_use() == 7
+    with pytest.raises(RuntimeError, match="used up"):
+        c._assign([(0, 3)])
+    c.release(2)
+    assert c.pages_in_use() == 4 and c.table[2].tolist() == [-1] * 4
+    c._assign([(0, 4)])
+    with pytest.raises(RuntimeError, match="max_seq_len"):
+        c._assign([(0, 5)])
+    with pytest.raises(ValueError):
+        PagedKVCache(1, 1, 64, 16, torch.float16, "cpu", page_size=24)
