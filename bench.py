@@ -642,9 +642,7 @@ def kernel_table(torch, K, layer, workloads, w, d, info, steps, step_only=False,
     def measure(fns, bytes_of, layout="padded"):
         table = {}
         for name, fn in fns.items():
-            for _ in range(3):
-                fn()
-            torch.cuda.synchronize()
+            _preheat(torch, fn)       # each row at the settled clock, like the timed steps themselves
             ms = _event_time_ms(fn, steps, torch)
             row = {"us": ms * 1e3, "alg_MB": bytes_of[name] / 1e6, "GBps": bytes_of[name] / (ms * 1e-3) / 1e9}
             row["hbm_frac"] = row["GBps"] / HBM_PEAK_GBS
