@@ -226,3 +226,39 @@ def test_block_decodes_the_same_from_pages(dtype):
     assert cache.pages_in_use() == 11                    # sequence 1 passed 16, sequence 2 passed 48
     cache.release(1)                                     # a finished sequence hands its two pages back
     assert cache.pages_in_use() == 9
+
+
+@pytest.mark.parametrize("seed", list(range(12)))
+def test_decode_attn_paged_random_shapes(seed):
+    """Random batch, heads, head size, page size, capacity and lengths: pages against the float64 oracle and against
+    the contiguous-cache kernel bit for bit."""
+    K, _ = _mods()
+    g = torch.Generator().manual_seed(1000 + seed)
+    pick = lambda xs: xs[int(torch.randint(0, len(xs), (1,), generator=g))]
+    dtype = pick([torch.float16, torch.bfloat16, torch.float32])
+    D = pick([32, 64, 80, 96, 128] if dtype != torch.float32 else [32, 64, 96, 128])
+    P = pick([16, 32, 64, 128])
+    B = int(torch.randint(1, 20, (1,), generator=g))
+    H = int(torch.randint(1, 9, (1,), generator=g))
+    S = P * int(torch.randint(1, max(2, 3000 // P), (1,), generator=g))
+    kv = torch.randint(0, S + 1, (B,), generator=g).tolist()
+    announce("decode attn paged random", seed, dtype, B, H, S, D, P, kv[:8])
+    q = torch.randn(B, H, 1, D, generator=g).to(dtype)
+    kc = torch.randn(B, H, S, D, generator=g).to(dtype)
+    vc = torch.randn(B, H, S, D, generator=g).to(dtype)
+    for b, n in enumerate(kv):
+        kc[b, :, n:] = float("nan")
+        vc[b, :, n:] = float("nan")
+    pool_pages = B * (S // P) + 3
+    k_pool, table = _scatter(kc, kv, P, pool_pages, torch.Generator().manual_seed(seed))
+    v_pool, _ = _scatter(vc, kv, P, pool_pages, torch.Generator().manual_seed(seed))
+    kv_t = torch.tensor(kv, dtype=torch.int32).cuda()
+    scale = D ** -0.5
+    _, _, want = eager.decode_attention(q, torch.nan_to_num(kc, nan=0.0), torch.nan_to_num(vc, nan=0.0), kv, scale,
+                                        acc_dtype=torch.float64)
+    for b, n in enumerate(kv):
+        if n == 0:
+            want[b] = 0
+    got = K.decode_attn_paged(q.cuda(), k_pool.cuda(), v_pool.cuda(), kv_t, table.cuda(), scale=scale)
+    assert_ctx_close(got.cpu(), want, dtype, "decode_attn_paged")
+    assert torch.equal(got, K.decode_attn(q.cuda(), kc.cuda(), vc.cuda(), kv_t, scale=scale))
