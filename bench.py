@@ -762,6 +762,48 @@ def copy_yardstick(torch, iters):
     return out
 
 
+def decode_sizes(torch, iters):
+    """The single-pass decode attention at batch sizes from one sequence up (72 heads of 128 channels, fp16, every
+    cache full): one workgroup per (batch, head) unit, the keys of a unit shared between workgroups (what the call
+    does for fewer than 512 units), and the same cache contents in pages of 64 positions shuffled over a pool."""
+    from energonai_amd import kernel as K
+    from energonai_amd.seqinfo import seq_info
+    H, D, P = 72, 128, 64
+    rows = []
+    for B in (1, 2, 4, 8, 16, 64):
+        for S in (2048, 8192):
+            if 2 * B * H * S * D * 2 > 6e9:
+                continue
+            dev = torch.device("cuda")
+            q = torch.randn(B, H, 1, D, device=dev, dtype=torch.float16)
+            kc = torch.randn(B, H, S, D, device=dev, dtype=torch.float16)
+            vc = torch.randn_like(kc)
+            info = seq_info(torch.full((B,), S, dtype=torch.int32, device=dev), B, dev)
+            out = torch.empty(B, H, 1, D, device=dev, dtype=torch.float16)
+            pages = B * (S // P)
+            perm = torch.randperm(pages, device=dev)
+            table = perm.view(B, S // P).to(torch.int32).contiguous()
+            k_pool = torch.empty((pages, H, P, D), dtype=kc.dtype, device=dev)
+            v_pool = torch.empty_like(k_pool)
+            k_pool[perm] = kc.view(B, H, S // P, P, D).permute(0, 2, 1, 3, 4).reshape(pages, H, P, D)
+            v_pool[perm] = vc.view(B, H, S // P, P, D).permute(0, 2, 1, 3, 4).reshape(pages, H, P, D)
+            need = K.decode_attn_workspace_bytes(B, H, S, D)
+            ws = torch.empty(max(need, 16), dtype=torch.uint8, device=dev)
+            fns = {"one_workgroup_per_unit": lambda: K.decode_attn(q, kc, vc, info, out=out, split=False),
+                   "as_called": lambda: K.decode_attn(q, kc, vc, info, out=out, workspace=ws),
+                   "paged": lambda: K.decode_attn_paged(q, k_pool, v_pool, info, table, out=out, workspace=ws)}
+            nbytes = 2 * B * H * S * D * 2
+            row = {"batch": B, "cached_positions": S, "units": B * H, "cache_MB": nbytes / 1e6,
+                   "shares_per_unit": (need // (B * H * (D + 2) * 4)) if need else 1}
+            for name, fn in fns.items():
+                _preheat(torch, fn)
+                us = _event_time_ms(fn, max(10, iters), torch) * 1e3
+                row[name] = {"us": us, "GBps": nbytes / us / 1e3}
+            rows.append(row)
+            del kc, vc, k_pool, v_pool
+    return {"heads": H, "size_per_head": D, "page": P, "dtype": "f16", "rows": rows}
+
+
 STREAM_MODES = {"copy": 0, "read": 1, "write": 2, "inplace": 0}
 PREFIX_MODES = {"inplace": 0, "write": 1, "read": 2, "out_of_place": 3}
 
@@ -918,6 +960,9 @@ def main(argv=None) -> int:
                          "copy / read only / write only with plain and non-temporal accesses, and in-place, write-only, "
                          "read-only and out-of-place passes over the causal prefixes of the c3 and c4 score tensors in "
                          "the [B,H,S,S] and the packed layout")
+    ap.add_argument("--decode-sizes", action="store_true",
+                    help="instead of the benchmark, time the single-pass decode attention from one sequence to 64 "
+                         "(keys of a unit shared between workgroups or not; contiguous caches and pages)")
     ns = ap.parse_args(argv)
     if ns.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this build measures one GPU's share of the path; --gpus must be 1 "
@@ -938,6 +983,12 @@ def main(argv=None) -> int:
         out = copy_yardstick(torch, ns.steps)
         if not ns.step_only:      # --step-only: the plain copy alone (the counter calibration run of bench_profiles.py)
             out["yardsticks"] = stream_yardsticks(torch, max(5, ns.steps))
+        out["library_source_hash"] = library_source_hash()
+        print(json.dumps(out))
+        return 0
+
+    if ns.decode_sizes:
+        out = decode_sizes(torch, ns.steps)
         out["library_source_hash"] = library_source_hash()
         print(json.dumps(out))
         return 0

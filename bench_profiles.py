@@ -387,9 +387,41 @@ def cmd_yardstick(ns) -> int:
     return 0
 
 
+def cmd_decode(ns) -> int:
+    """bench.py --decode-sizes (no profiler: event timings) as a table."""
+    cmd = ["python3", os.path.join(ROOT, "bench.py"), "--decode-sizes", "--steps", str(ns.steps)]
+    proc = subprocess.run(cmd, cwd=ROOT, stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True, timeout=ns.timeout)
+    if proc.returncode != 0:
+        sys.stderr.write(proc.stderr[-3000:])
+        raise SystemExit(f"bench.py exited with {proc.returncode}")
+    line = [json.loads(ln) for ln in proc.stdout.splitlines() if ln.startswith("{")][-1]
+    print("# Single-pass decode attention from one sequence to 64: one workgroup per unit, shared keys, pages\n")
+    print("Command (MI355X box, repo root; the summary below is this command's stdout; HIP-event timings, no profiler):\n")
+    print(f"```\npython3 bench_profiles.py decode\n  -> python3 bench.py --decode-sizes --steps {ns.steps}\n```\n")
+    print_sources(line)
+    print(f"{line['heads']} heads of {line['size_per_head']} channels, {line['dtype']}, every cache full; a (batch, head) "
+          "unit is one workgroup of 1024 lanes unless its keys are shared.  `as called`: what `en_decode_attn` does when "
+          "the caller brings the workspace (fewer than 512 units and at least 1024 cached positions: the keys of a unit "
+          "go to several workgroups and a second small kernel combines them; its time is included).  `pages`: "
+          f"`en_decode_attn_paged` on the same contents in pages of {line['page']} positions with shuffled ids.  "
+          "TB/s = K and V bytes of the cached positions over the time.\n")
+    print("| sequences | cached positions | units | K + V, MB | workgroups per unit | one workgroup per unit, us (TB/s) | "
+          "as called, us (TB/s) | pages, us (TB/s) |\n|---|---|---|---|---|---|---|---|")
+    cell = lambda r: f"{r['us']:.1f} ({r['GBps'] / 1e3:.2f})"
+    for r in line["rows"]:
+        print(f"| {r['batch']} | {r['cached_positions']} | {r['units']} | {r['cache_MB']:.0f} | {r['shares_per_unit']} | "
+              f"{cell(r['one_workgroup_per_unit'])} | {cell(r['as_called'])} | {cell(r['paged'])} |")
+    return 0
+
+
 def main(argv=None) -> int:
     ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
     sub = ap.add_subparsers(dest="cmd", required=True)
+    p = sub.add_parser("decode")
+    p.add_argument("--steps", type=int, default=20)
+    p.add_argument("--timeout", type=int, default=300)
+    p.add_argument("--raw-dir", default=None)
+    p.set_defaults(fn=cmd_decode)
     p = sub.add_parser("yardstick")
     p.add_argument("--steps", type=int, default=10)
     p.add_argument("--timeout", type=int, default=300)
