@@ -658,6 +658,11 @@ def kernel_table(torch, K, layer, workloads, w, d, info, steps, step_only=False,
                 row["yardstick_GBps"] = yard[key]
                 row["yardstick_pattern"] = key
                 row["frac_of_yardstick"] = row["GBps"] / yard[key]
+            # PV: also against the same bytes read tile by tile along the keys, its own walk, three workgroups per CU
+            walk = f"prefix_read_tile_walk_3_per_cu_{layout}"
+            if name == "attn_pv" and walk in yard:
+                row["tile_walk_yardstick_GBps"] = yard[walk]
+                row["frac_of_tile_walk_yardstick"] = row["GBps"] / yard[walk]
             table[name] = row
         return table
     step_layout = "packed" if ("prefix_read_packed" in yard) else "padded"
@@ -805,7 +810,11 @@ def decode_sizes(torch, iters):
 
 
 STREAM_MODES = {"copy": 0, "read": 1, "write": 2, "inplace": 0}
-PREFIX_MODES = {"inplace": 0, "write": 1, "read": 2, "out_of_place": 3}
+PREFIX_MODES = {"inplace": 0, "write": 1, "read": 2, "out_of_place": 3,
+                # read only, a 128-row tile at a time along the keys in 128- or 256-byte pieces per row (how PV walks its
+                # probabilities); "_3_per_cu": with the three workgroups per CU the attention kernels have
+                "read_tile_walk": 4, "read_tile_walk_3_per_cu": 5, "read_tile_walk_256B": 6,
+                "read_tile_walk_256B_3_per_cu": 7}
 
 
 def _preheat(torch, fn):
@@ -899,7 +908,7 @@ def workload_yardsticks(torch, w, d, info, packed_scores):
         for layout, packed in (("padded", 0), ("packed", 1)):
             if packed and not packed_scores:
                 continue
-            for mode in ("inplace", "write", "read"):
+            for mode in ("inplace", "write", "read", "read_tile_walk_3_per_cu"):
                 y[f"prefix_{mode}_{layout}"] = max(
                     prefix_yardstick_GBps(torch, info.lens, d["lens_list"], w.batch, w.heads, w.seq, w.dtype, packed, mode, nt)
                     for nt in (0, 1))

@@ -384,6 +384,18 @@ def cmd_yardstick(ns) -> int:
     print("| lengths, layout | " + " | ".join(cols) + " |\n|---|" + "---|" * len(cols))
     for name, row in y["prefix"].items():
         print(f"| {name.replace('_', ', ')} | " + " | ".join(f"{row[c]:.0f}" for c in cols) + " |")
+    print("\n## The same prefixes read the way PV walks them (`prefix_tile_walk_kernel`)\n")
+    print("One workgroup per tile of 128 rows, moving along the keys in steps of 128 bytes per row (64 fp16 keys, the key "
+          "tile of the attention kernels) or 256 bytes, every row as far as its prefix goes, the next step's loads in "
+          "flight while this step's are consumed; no LDS traffic, no arithmetic.  `3 per CU`: 48 KB of idle LDS per "
+          "workgroup, the occupancy of the attention kernels.  The bytes are those of the `read` column above.\n")
+    cols = [f"{m}{t}" for m in ("read_tile_walk", "read_tile_walk_3_per_cu", "read_tile_walk_256B",
+                                "read_tile_walk_256B_3_per_cu") for t in ("", "_nt")]
+    head = [("256 B" if "256B" in c else "128 B") + (", 3 per CU" if "3_per_cu" in c else "") +
+            (", non-temporal" if c.endswith("_nt") else "") for c in cols]
+    print("| lengths, layout | " + " | ".join(head) + " |\n|---|" + "---|" * len(cols))
+    for name, row in y["prefix"].items():
+        print(f"| {name.replace('_', ', ')} | " + " | ".join(f"{row[c]:.0f}" for c in cols) + " |")
     return 0
 
 

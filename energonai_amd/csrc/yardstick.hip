@@ -8,6 +8,7 @@
 //                   only rows q < seq_lens[b] exist; in the padded [B,H,S,S] layout or in the packed one.
 //                   Read and written back in place (scale_mask_softmax), written only (QK^T), read only (PV),
 //                   or read from one tensor and written to another.
+//   prefix_tile_walk_kernel  the same prefixes read a 128-row tile at a time along the keys, as PV reads them.
 //
 // Neither is called by any op of the library; bench.py times them (--copy-yardstick and the yardstick_GBps
 // column of its kernel tables).
@@ -113,6 +114,54 @@ __global__ __launch_bounds__(kBlock) void prefix_kernel(PrefixArgs p) {
   if (MODE == 2 && acc == 0x9e3779b9u && p.key == 1u) p.sink[0] = acc;
 }
 
+// The causal prefixes read the way the attention kernels walk them: a workgroup takes a tile of 128 rows and moves
+// along the keys in steps of 128 bytes per row (64 fp16 keys), every row as far as its own prefix goes, so that one
+// step touches 128 pieces of 128 bytes, a row pitch apart (PV reads its probabilities so; QK^T writes its scores
+// so).  Eight lanes per row piece, four rows per lane and step, the next step's loads in flight while this one's
+// are consumed.  `lds_bytes` of dynamic LDS that nothing uses limit the workgroups per CU to what a kernel holding
+// that much would have (48 KB: three per CU).  es = 2 only.
+template <bool NT, int PIECE = 128>
+__global__ __launch_bounds__(kBlock) void prefix_tile_walk_kernel(PrefixArgs p) {
+  extern __shared__ unsigned char unused_lds[];
+  constexpr int ROWS = 128;                     // rows per tile; PIECE: bytes per row and step
+  constexpr int LPP = PIECE / 16, GROUPS = kBlock / LPP, RPL = ROWS / GROUPS;
+  const int unit = blockIdx.y, b = unit / p.H;
+  const int ql = min(p.lens[b], p.S);
+  const int q0 = (int)blockIdx.x * ROWS;
+  if (q0 >= ql) return;
+  const int lane8 = threadIdx.x % LPP, rsub = threadIdx.x / LPP;
+  const int64_t unit_elems = p.packed ? packed_row_start<8 * kPackedRowVectors>(p.S) : (int64_t)p.S * p.S;
+  const unsigned char *base = p.a + unit * unit_elems * 2;
+  int64_t off[RPL];
+  int row_bytes[RPL];
+#pragma unroll
+  for (int i = 0; i < RPL; ++i) {
+    const int q = q0 + rsub + GROUPS * i;
+    off[i] = (p.packed ? packed_row_start<8 * kPackedRowVectors>(q) : (int64_t)q * p.S) * 2 + lane8 * 16;
+    row_bytes[i] = q < ql ? (q + 1) * 2 - lane8 * 16 : 0;           // bytes of the prefix from this lane's chunk on
+  }
+  const int steps = (min(q0 + ROWS, ql) * 2 + PIECE - 1) / PIECE;
+  uint32_t acc = 0;
+  uint4 cur[RPL], nxt[RPL];
+  auto fetch = [&](uint4 (&v)[RPL], int st) {
+#pragma unroll
+    for (int i = 0; i < RPL; ++i) {
+      v[i] = make_uint4(0u, 0u, 0u, 0u);
+      if (st * PIECE < row_bytes[i]) v[i] = load16<NT>(base + off[i] + (int64_t)st * PIECE);
+    }
+  };
+  fetch(cur, 0);
+  for (int st = 0; st < steps; ++st) {
+    fetch(nxt, st + 1);
+#pragma unroll
+    for (int i = 0; i < RPL; ++i) {
+      acc ^= cur[i].x ^ cur[i].y ^ cur[i].z ^ cur[i].w;
+      cur[i] = nxt[i];
+    }
+  }
+  if (acc == 0x9e3779b9u && p.key == 1u) p.sink[0] = acc;
+}
+
 template <int MODE>
 static void launch_stream(const void *src, void *dst, int64_t nvec, int nt, uint32_t *sink, hipStream_t s) {
   const int64_t want = ceil_div(nvec, (int64_t)kBlock * 4);
@@ -155,12 +204,24 @@ int en_prefix_yardstick(void *scores, void *scores_out, const int32_t *seq_lens,
   if (!scores || !seq_lens || (mode == 3 && !scores_out)) return EN_ERR_NULL;
   if (batch < 1 || head_num < 1 || seq_len < 1 || (int64_t)batch * head_num > 65535) return EN_ERR_SHAPE;
   if (elem_size != 2 && elem_size != 4) return EN_ERR_DTYPE;
-  if (mode < 0 || mode > 3) return EN_ERR_UNSUPPORTED;
+  if (mode < 0 || mode > 7) return EN_ERR_UNSUPPORTED;
+  if (mode >= 4 && elem_size != 2) return EN_ERR_DTYPE;
   if (!packed && ((int64_t)seq_len * elem_size) % 16 != 0) return EN_ERR_ALIGN;     // rows start on 16-byte boundaries
   if (!aligned_to(scores, 16) || (scores_out && !aligned_to(scores_out, 16))) return EN_ERR_ALIGN;
   PrefixArgs p{(unsigned char *)scores, (unsigned char *)scores_out, seq_lens, head_num, seq_len, elem_size, packed ? 1 : 0,
                0u, (uint32_t *)scores};
   hipStream_t s = (hipStream_t)stream;
+  if (mode >= 4) {      // 4: the tile walk with as many workgroups per CU as fit; 5: with three per CU
+    const dim3 grid((unsigned)ceil_div(seq_len, 128), (unsigned)(batch * head_num), 1);
+    const size_t lds = (mode == 5 || mode == 7) ? 48 * 1024 : 0;
+    if (mode >= 6) {
+      if (nontemporal) prefix_tile_walk_kernel<true, 256><<<grid, kBlock, lds, s>>>(p);
+      else prefix_tile_walk_kernel<false, 256><<<grid, kBlock, lds, s>>>(p);
+    } else if (nontemporal) prefix_tile_walk_kernel<true><<<grid, kBlock, lds, s>>>(p);
+    else prefix_tile_walk_kernel<false><<<grid, kBlock, lds, s>>>(p);
+    EN_RETURN_IF_LAUNCH_FAILED();
+    return EN_OK;
+  }
   switch (mode) {
     case 0: launch_prefix<0>(p, batch, nontemporal, s); break;
     case 1: launch_prefix<1>(p, batch, nontemporal, s); break;

@@ -407,7 +407,11 @@ int en_copy_bytes(const void *src, void *dst, int64_t nbytes, en_stream_t stream
  * tensor -- row q of (batch, head) unit u holds q + 1 elements, rows q < seq_lens[b] only -- in the [B,H,S,S]
  * layout or (packed != 0) the packed layout of en_packed_scores_elems: mode 0 reads every prefix and writes it
  * back in place (the pattern of en_scale_mask_softmax with tail_rows 1), 1 only writes (en_attn_qk), 2 only
- * reads (en_attn_pv), 3 reads scores and writes scores_out.  Whole 16-byte vectors are moved. */
+ * reads (en_attn_pv), 3 reads scores and writes scores_out.  Whole 16-byte vectors are moved.  Modes 0-3 take each
+ * row (packed: each unit) as one contiguous range.  Modes 4-7 (2-byte elements) only read, the way the attention
+ * kernels walk a score tensor: one workgroup per tile of 128 rows, moving along the keys in steps of 128 bytes per
+ * row (4, 5) or 256 bytes (6, 7), the next step's loads in flight while this step's are consumed; 5 and 7 hold
+ * 48 KB of LDS per workgroup, i.e. three workgroups per CU as the attention kernels have. */
 int en_stream_yardstick(const void *src, void *dst, int64_t nbytes, int mode, int nontemporal, en_stream_t stream);
 int en_prefix_yardstick(void *scores, void *scores_out, const int32_t *seq_lens, int batch, int head_num, int seq_len,
                         int packed, int mode, int nontemporal, int elem_size, en_stream_t stream);

@@ -244,7 +244,7 @@ def test_yardstick_kernels_touch_exactly_their_pattern():
     for packed in (0, 1):
         numel = packed_scores_elems(B, H, S, torch.float16) if packed else B * H * S * S
         src = torch.randn(numel, device="cuda").half()
-        for mode in (0, 1, 2, 3):
+        for mode in (0, 1, 2, 3, 4, 5, 6, 7):
             buf = src.clone()
             out = torch.full_like(src, 5.0)
             _lib.check(lib.en_prefix_yardstick(buf.data_ptr(), out.data_ptr(), lens_t.data_ptr(), B, H, S, packed, mode, 0, 2,
@@ -261,8 +261,8 @@ def test_yardstick_kernels_touch_exactly_their_pattern():
                     for q in range(lens[b]):
                         start = (unit * S + q) * S
                         touched[start:start + -(-(q + 1) // 8) * 8] = True
-            if mode in (0, 2):
-                assert torch.equal(buf, src)
+            if mode in (0, 2, 4, 5, 6, 7):     # 4..7: read only, a 128-row tile at a time along the keys
+                assert torch.equal(buf, src) and bool((out == 5.0).all())
             if mode == 1:
                 assert bool((buf.cpu()[touched] == 0).all()) and torch.equal(buf.cpu()[~touched], src.cpu()[~touched])
             if mode == 3:
