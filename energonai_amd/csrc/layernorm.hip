@@ -211,6 +211,10 @@ static int dispatch(const LnArgs &a, hipStream_t s) {
     if (nvec <= 2 * 64) done = launch_vpl<DTI, DTO, 64>(a, (nvec + 63) / 64, s);
     // at most four vectors per lane while the row fits 512 lanes: rows of 1025..2048 vectors measured 288 us
     // with 256 lanes x 6 vectors against 267 us with 512 lanes x 3 (20142 rows of 12288 fp16, residual added)
+    // rows that would put four vectors on each of 256 lanes go to 512 lanes x 2 when there are many of them:
+    // 7168-wide fp16 rows (896 vectors) x 9244: 60.6 -> 58.8 us, 8192-wide x 32768: 264 -> 256 us; with fewer
+    // vectors (5120-wide: 48 -> 52 us) or few rows (2048 rows: 15.4 -> 16.3 us) 256 lanes stay ahead
+    else if (nvec > 3 * 256 && nvec <= 4 * 256 && a.n1 >= 4096) done = launch_vpl<DTI, DTO, 512>(a, 2, s);
     else if (nvec <= 4 * 256) done = launch_vpl<DTI, DTO, 256>(a, (nvec + 255) / 256, s);
     else if (nvec <= 4 * 512) done = launch_vpl<DTI, DTO, 512>(a, (nvec + 511) / 512, s);
     else if (nvec <= 8 * 1024) done = launch_vpl<DTI, DTO, 1024>(a, (nvec + 1023) / 1024, s);
