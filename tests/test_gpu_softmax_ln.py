@@ -127,6 +127,8 @@ LN_CASES = [
     # n1, n2
     (698, 768), (64, 9216), (33, 7168), (20, 12288), (5, 1024), (7, 8), (3, 16384),
     (4, 40000),      # wide row: 1024-lane kernel
+    (4100, 7168),    # 896 fp16 vectors and many rows: 512 lanes x 2 vectors (fp32: 1792 vectors, 512 x 4)
+    (4097, 4000),    # fp32: 1000 vectors and many rows: 512 lanes x 2; fp16: 500 vectors on 256 lanes
     (3, 100),        # fp16: 100 % 8 != 0 -> generic kernel
     (2, 70001),      # too wide / odd: generic kernel
 ]
