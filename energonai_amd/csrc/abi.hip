@@ -71,7 +71,7 @@ __global__ __launch_bounds__(kBlock) void copy_kernel(const uint4 *__restrict__ 
 
 extern "C" {
 
-int en_version(void) { return 200; }
+int en_version(void) { return 300; }
 
 #ifndef EN_SOURCE_HASH
 #define EN_SOURCE_HASH "unknown"
