@@ -7,10 +7,10 @@ linear layers, so ``torch.nn.Linear`` (a library GEMM) stands in for them with t
 attribute names; ``LayerNorm1D`` becomes the fused LayerNorm of ``energonai_amd.kernel``.
 """
 from .gemm import gemm_tuning, set_gemm_tuning
-from .kv_cache import KVCache
+from .kv_cache import KVCache, PagedKVCache
 from .attention import MultiHeadAttention1D
 from .mlp import MLP1D
 from .endecoder import Block1D
 from .stack import PackedStack
 
-__all__ = ["KVCache", "MultiHeadAttention1D", "MLP1D", "Block1D", "PackedStack", "set_gemm_tuning", "gemm_tuning"]
+__all__ = ["KVCache", "PagedKVCache", "MultiHeadAttention1D", "MLP1D", "Block1D", "PackedStack", "set_gemm_tuning", "gemm_tuning"]

@@ -125,9 +125,10 @@ class PagedKVCache:
     def fill(self, k_src: torch.Tensor, v_src: torch.Tensor, info: SeqInfo, k_head_first: int = 0,
              v_head_first: int = 0, longest: Optional[int] = None, lens_host=None) -> None:
         """Prefill from packed projections seen as ``[T,Hs,D]``.  The pages are assigned on the host, which needs
-        the lengths there: ``lens_host`` if the caller has them, else they are read from the device once."""
+        the lengths there: ``lens_host`` if the caller has them, else ``info.lens_host()`` (one copy from the device per
+        batch, shared by every layer that fills its cache from the same ``info``)."""
         if lens_host is None:
-            lens_host = info.lens.tolist()
+            lens_host = info.lens_host()
         lens_host = [int(n) for n in lens_host]
         P = self.page_size
         for b in range(self.batch_size):

@@ -24,7 +24,7 @@ class SeqInfo:
     """Device-resident int32 lengths and exclusive prefix for one batch."""
 
     __slots__ = ("lens", "cu_seqlens", "batch_size", "_total", "_source", "_row_offsets", "_tile_tables", "_ready",
-                 "_ordered", "ephemeral")
+                 "_ordered", "ephemeral", "_lens_host")
 
     def __init__(self, lens: torch.Tensor, cu_seqlens: torch.Tensor, batch_size: int, total: Optional[int], source):
         self.lens = lens                # int32 [B] on the device
@@ -37,6 +37,7 @@ class SeqInfo:
         self._ready = []                # events recorded behind the kernels that produced the arrays above
         self._ordered = set()           # raw streams already ordered behind every event of _ready
         self.ephemeral = False          # built for one call only (lengths that cannot be cached): see tile_table_ptr
+        self._lens_host = None          # (version of lens, the lengths as a Python list)
 
     def produced_on_current_stream(self) -> None:
         """Call right after launching a kernel that writes one of this object's arrays: remembers the point
@@ -75,6 +76,15 @@ class SeqInfo:
             self._total = int(self.cu_seqlens[self.batch_size].item())
         return self._total
 
+
+    def lens_host(self):
+        """The lengths as a list of Python ints.  The first use copies them from the device (a sync, like
+        ``total``); later uses of the same lengths are free, so every layer of a stack can ask."""
+        version = self._lens_version()
+        if self._lens_host is None or version is None or self._lens_host[0] != version:
+            self.order_current_stream()
+            self._lens_host = (version, [int(n) for n in self.lens.tolist()])
+        return list(self._lens_host[1])
 
     def _lens_version(self):
         """Version counter of the lengths, part of every key under which something derived from them is kept:

@@ -262,3 +262,44 @@ def test_decode_attn_paged_random_shapes(seed):
     got = K.decode_attn_paged(q.cuda(), k_pool.cuda(), v_pool.cuda(), kv_t, table.cuda(), scale=scale)
     assert_ctx_close(got.cpu(), want, dtype, "decode_attn_paged")
     assert torch.equal(got, K.decode_attn(q.cuda(), kc.cuda(), vc.cuda(), kv_t, scale=scale))
+
+
+def test_stack_of_blocks_on_pages():
+    """Two blocks behind one depad, both with paged caches: the lengths are copied to the host once for both
+    (SeqInfo.lens_host), and prefill plus four decode steps give the bits of the same stack on contiguous caches."""
+    _, M = _mods()
+    from energonai_amd.seqinfo import seq_info
+    B, S, hid, heads = 4, 40, 128, 4
+    lens = [40, 7, 16, 33]
+    announce("stack on pages")
+    dtype = torch.float16
+
+    def stack(**kw):
+        return M.PackedStack([M.Block1D(hid, heads, 4.0, dtype=dtype, max_seq_len=64, **kw) for _ in range(2)]).cuda()
+    flat, paged = stack(), stack(kv_page_size=16)
+    g = torch.Generator().manual_seed(77)
+    with torch.no_grad():
+        for name, prm in flat.named_parameters():
+            if prm.dim() > 1:
+                prm.copy_(torch.randn(prm.shape, generator=g) / prm.shape[1] ** 0.5)
+            else:
+                prm.copy_((1.0 if name.endswith("weight") else 0.0) + 0.05 * torch.randn(prm.shape, generator=g))
+    paged.load_state_dict(flat.state_dict())
+    x = torch.randn(B, S, hid, generator=g).to(dtype)
+    valid = torch.zeros(B, S)
+    for b, n in enumerate(lens):
+        valid[b, S - n:] = 1
+    x = x * valid.unsqueeze(-1).to(dtype)
+    lens_t = torch.tensor(lens, dtype=torch.int32).cuda()
+    a = flat(x.cuda(), first_cache=True, seq_lens=lens_t)
+    b_ = paged(x.cuda(), first_cache=True, seq_lens=lens_t)
+    assert torch.equal(a, b_)
+    info = seq_info(lens_t, B, lens_t.device)
+    assert info.lens_host() == lens and info._lens_host is not None
+    for blk in paged.blocks:
+        assert blk.attn.kv_cache.pages_in_use() == sum((n + 15) // 16 for n in lens)
+    for step in range(4):
+        x = torch.cat((x, torch.randn(B, 1, hid, generator=g).to(dtype)), 1)
+        a = flat(x.cuda(), first_cache=False)
+        b_ = paged(x.cuda(), first_cache=False)
+        assert torch.equal(a[:, -1], b_[:, -1]), step
